@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X int8 hot path.
+
+One "step" = one pass of the hot path over one batch of synthetic input.  The headline workload is the 4096^3
+int8 GEMM of benchmark configuration 5 (int8 x int8 -> int32 on the matrix cores with the fused per-channel
+requantising epilogue); the decode GEMV (configuration 4, batch 1), DynamicQuant and the BERT dynamic MatMuls
+(configuration 3) are timed in the same run and reported under "extra".  Inputs are resident in HBM before the
+timed region.  Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm4096|gemm8192] [--no-cpu] [--no-extra]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA peak, TOP/s (5.0 POP/s)
+PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E peak, GB/s
+
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
+# script (summaries under profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {"gemm4096": None, "gemm8192": None}
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) / steps, wall * 1e3 / steps  # ms per step by HIP events, by host clock
+
+
+def make_matmul(c):
+    from mindspore_amd import kernels as K
+    qp = [K.QuantParam(float(s), int(z)) for s, z in zip(c["sw"], c["zw"])]
+    return K.MatmulInt8Kernel(c["w"], c["bias"], K.QuantParam(c["sx"], c["zx"]), qp, K.QuantParam(c["so"], c["zo"]),
+                              True, c["act"])
+
+
+def bench_gemm(size, steps, warmup):
+    import torch
+    from mindspore_amd import workloads as wl
+    c = wl.gemm_c5(size)
+    kern = make_matmul(c)
+    a = torch.from_numpy(c["a"]).cuda()
+    ev_ms, host_ms = time_steps(lambda: kern.run(a), steps, warmup)
+    ops = 2.0 * size * size * size
+    return dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c)
+
+
+def bench_gemv(steps, warmup, m=1):
+    """Decode step: the five 7B-class layer matrices, two layers' worth of distinct weights (404 MB) cycled so the
+    256 MB Infinity Cache cannot hold the working set."""
+    import torch
+    from mindspore_amd import workloads as wl
+    kerns, acts, total_bytes = [], [], 0
+    for layer in range(2):
+        for name, n, k in wl.DECODE_SHAPES:
+            c = wl.gemv_c4(name, n, k, m, seed=layer)
+            kerns.append(make_matmul(c))
+            acts.append(torch.from_numpy(c["a"]).cuda())
+            total_bytes += n * k + m * k + m * n + 16 * n
+    def step():
+        for kern, a in zip(kerns, acts):
+            kern.run(a)
+    ev_ms, _ = time_steps(step, steps, warmup)
+    per_shape = {}
+    for i, (name, n, k) in enumerate(wl.DECODE_SHAPES):
+        if name in per_shape:
+            continue
+        kern, a = kerns[i], acts[i]
+        ms, _ = time_steps(lambda: kern.run(a), max(steps, 20), 3)
+        per_shape[name] = dict(n=n, k=k, ms_warm=ms, gbps_warm=(n * k + m * k + m * n + 16 * n) / (ms * 1e-3) / 1e9)
+    gbps = total_bytes / (ev_ms * 1e-3) / 1e9
+    return dict(m=m, ms_per_decode_step_2_layers=ev_ms, bytes=total_bytes, gbps=gbps, frac_of_hbm_peak=gbps / PEAK_HBM_GBPS,
+                cache_warm_single_matrix=per_shape)
+
+
+def bench_bert(steps, warmup):
+    import torch
+    from mindspore_amd import kernels as K
+    from mindspore_amd import workloads as wl
+    out = {}
+    x = torch.from_numpy(wl.bert_c3_activation(768)).cuda()
+    dq = K.DynamicQuantKernel(False)
+    ms, _ = time_steps(lambda: dq.run(x, fetch_params=False), steps, warmup)
+    nbytes = x.numel() * 5
+    out["dynquant_4096x768"] = dict(ms=ms, gbps=nbytes / (ms * 1e-3) / 1e9, frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS)
+    q, _ = dq.run(x, fetch_params=False)
+    total_ops, total_ms = 0.0, 0.0
+    for name, n, k in wl.BERT_SHAPES:
+        wt = wl.bert_c3_weights(name, n, k)
+        mm = K.MatmulDynamicInt8Kernel(wt["w"], wt["bias"], [K.QuantParam(float(s), 0) for s in wt["sw"]])
+        qa = q if k == 768 else torch.randint(-128, 127, (4096, k), dtype=torch.int8, device="cuda")
+        ms, _ = time_steps(lambda: mm.run(qa, params_dev=dq.device_params()), steps, warmup)
+        ops = 2.0 * 4096 * n * k
+        out["dynmm_" + name] = dict(ms=ms, tops=ops / (ms * 1e-3) / 1e12)
+        total_ops += ops
+        total_ms += ms
+    out["dynmm_total_tops"] = total_ops / (total_ms * 1e-3) / 1e12
+    return out
+
+
+def cpu_baseline(case, size):
+    """nnacl's CPU path (compiled from the reference tree, oracle/_ref) -- or the restatement if that library did
+    not travel -- on a bounded sample: the first `rows` activation rows of the same GEMM, all host cores."""
+    from oracle import pyoracle
+    cores = min(16, os.cpu_count() or 1)
+    rows = 512 if size <= 4096 else 128
+    sub = dict(case)
+    sub["a"] = case["a"][:rows].copy()
+    if pyoracle.Reference.available():
+        eng, kind = pyoracle.reference(), "reference"
+        eng.threads = cores
+        eng.matmul_int8(**sub)
+        secs = eng.last_seconds
+    else:
+        eng, kind = pyoracle.oracle(), "port"
+        eng.set_threads(cores)
+        t0 = time.perf_counter()
+        eng.matmul_int8(**sub)
+        secs = time.perf_counter() - t0
+    ops = 2.0 * rows * size * size
+    return dict(value=ops / secs / 1e12, unit="TOP/s", cores=cores, kind=kind, seconds=secs,
+                sample="first %d of %d activation rows of the same %d^3 GEMM (A-pack + row sums + MatmulInt8Opt "
+                       "column stripes on %d threads)" % (rows, size, size, cores))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="gemm4096", choices=["gemm4096", "gemm8192"])
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extra", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this hot path is a single-GPU path; only --gpus 1 is supported (got %d)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from mindspore_amd import lib
+    lib.init(0)  # raises if the HIP library is missing or the GPU is not gfx950
+
+    size = 4096 if args.workload == "gemm4096" else 8192
+    g = bench_gemm(size, args.steps, args.warmup)
+    extra = {}
+    if not args.no_extra:
+        other = 8192 if size == 4096 else 4096
+        o = bench_gemm(other, max(3, args.steps // 5), 2)
+        extra["gemm%d" % other] = dict(ms=o["ms"], tops=o["tops"], frac_of_int8_peak=o["tops"] / PEAK_INT8_TOPS)
+        extra["gemv_decode_m1"] = bench_gemv(max(5, args.steps // 2), 3, 1)
+        extra["gemv_decode_m8"] = bench_gemv(max(5, args.steps // 2), 3, 8)
+        extra.update(bench_bert(max(5, args.steps // 2), 3))
+    result = {
+        "metric": "int8 GEMM TOPS + % i8 MFMA peak; decode GEMV HBM GB/s; vs nnacl CPU",
+        "value": g["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": g["ms"], "ms_per_step_host_clock": g["host_ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "i8", "data": "synthetic",
+        "config": {"workload": "config 5: int8 GEMM M=N=K=%d, per-channel requant to int8 (fused epilogue), zx=7, "
+                               "int32 bias" % size},
+        "roofline": {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
+                     "kernel": "gemm_i8_kernel<256,256,2,2,requant>", "ops_per_launch": g["ops"]},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(g["case"], size)
+    if extra:
+        result["extra"] = extra
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

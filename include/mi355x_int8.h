@@ -1,0 +1,199 @@
+/*
+ * mi355x_int8 -- C ABI of the MI355X (gfx950) implementation of MindSpore Lite's full-quant int8 inference hot path.
+ *
+ * The library is the drop-in for the arithmetic that Lite's CPU kernels delegate to nnacl.  A Lite provider kernel
+ * (mindspore::kernel::Kernel subclass registered with registry::RegisterKernel) maps onto it as
+ *     Prepare()/ReSize()  ->  mi_*_create      (quant-parameter derivation, weight packing, bias fold, upload)
+ *     Execute()           ->  mi_*_run_host    (host tensors, as a "CPU"-arch provider kernel receives them)
+ *                             mi_*_run         (device pointers + HIP stream, for chained device-resident tensors)
+ *     ~Kernel()           ->  mi_*_destroy
+ *
+ * Conventions
+ *   - every entry point returns an int status with the numeric values of Lite's RET_* codes
+ *     (mindspore/lite/include/errorcode.h:28-39); nothing throws across the boundary;
+ *   - plain pointers and sizes only; "host" pointers are ordinary process memory, "dev" pointers are HIP device
+ *     memory on the device chosen by mi_init; `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - handles are thread-compatible: distinct handles may be used from different threads, one handle from one
+ *     thread at a time;
+ *   - all tensors are dense row-major; images are NHWC; activation types use schema ActivationType values
+ *     (mindspore/lite/schema/ops_types.fbs:62-66): 0 none, 1 ReLU, 3 ReLU6.
+ *
+ * Reference paths below are relative to the reference tree:
+ *   NN/ = mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/      LK/ = mindspore/lite/src/litert/kernel/cpu/
+ */
+#ifndef MI355X_INT8_H_
+#define MI355X_INT8_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI_OK 0
+#define MI_ERROR (-1)         /* RET_ERROR: HIP failure or internal error */
+#define MI_NULL_PTR (-2)      /* RET_NULL_PTR */
+#define MI_PARAM_INVALID (-3) /* RET_PARAM_INVALID: shape/quant-parameter mismatch, nothing was launched */
+#define MI_MEMORY_FAILED (-6) /* RET_MEMORY_FAILED */
+#define MI_NOT_SUPPORT (-7)   /* RET_NOT_SUPPORT: the creator should decline and let the builtin CPU kernel run */
+
+#define MI_ACT_NONE 0
+#define MI_ACT_RELU 1
+#define MI_ACT_RELU6 3
+
+/* ---- library ---------------------------------------------------------------------------------------------- */
+
+/* Selects the HIP device and verifies it is gfx950.  Must be called once before any create/run call.
+ * Returns MI_NOT_SUPPORT when no such GPU is present (the provider then registers nothing). */
+int mi_init(int device);
+/* Message of the last failure on the calling thread ("" if none). */
+const char *mi_last_error(void);
+const char *mi_version(void);
+
+/* ---- quant-parameter derivation (host arithmetic, no GPU needed) -------------------------------------------- */
+
+/* real multiplier -> (31-bit mantissa, left shift >= 0, right shift <= 0).
+ * Replaces QuantizeRoundParameterWithDoublePrecision, NN/int8/quantize.c:39-51 (QuantizeMultiplier :113-161). */
+int mi_quantize_multiplier(double real_multiplier, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift);
+/* Clamp bounds of the fused activation in the quantised domain.
+ * Replaces CalculateActivationRangeQuantized, NN/int8/quantize.c:78-94. */
+int mi_activation_range(int32_t act_type, int32_t out_zp, double out_scale, int32_t *act_min, int32_t *act_max);
+/* (mult, ls, rs)[i] for real multiplier (float)in_scale*(float)filter_scale[i] / (float)out_scale, the derivation of
+ * MatmulBaseInt8CPUKernel::InitQuantParam (LK/int8/matmul_base_int8.cc:258-266) and
+ * ConvolutionBaseCPUKernel::SetQuantMultiplier (LK/base/convolution_base.cc:416-427). */
+int mi_requant_params(double in_scale, const double *filter_scales, int32_t n, double out_scale, int32_t *multiplier,
+                      int32_t *left_shift, int32_t *right_shift);
+/* One requantisation step on the host: MultiplyByQuantizedMultiplier, NN/int8/fixed_point.c:66-68. */
+int32_t mi_multiply_by_quantized_multiplier(int32_t value, int32_t multiplier, int32_t left_shift,
+                                            int32_t right_shift);
+
+/* ---- full-quant MatMul / FullConnection ------------------------------------------------------------------- */
+/* Replaces MatmulBaseInt8CPUKernel (LK/int8/matmul_base_int8.cc: InitQuantParam :235-273, TransferB :360-384,
+ * Run :530-571, RunImpl :129-150), FullconnectionInt8CPUKernel (LK/int8/fullconnection_int8.cc:26-67) and the nnacl
+ * functions they call: RowMajor2Row16x4MajorInt8 / RowMajor2Col16x4MajorInt8 (NN/int8/matmul_int8.c:158-236,722-736),
+ * CalcInputSums (:786-799), CalcWeightBiasSums (:802-819), MatmulInt8Opt (:296-331). */
+typedef struct mi_matmul mi_matmul;
+
+typedef struct mi_matmul_desc {
+  int32_t deep;        /* K */
+  int32_t col;         /* N: output channels */
+  int32_t b_transpose; /* 1: weight is [N,K] (FullConnection, MatMul transpose_b); 0: weight is [K,N] */
+  int32_t act_type;
+  double in_scale;
+  int32_t in_zp;
+  double out_scale;
+  int32_t out_zp;
+  int32_t filter_quant_num;    /* 1 (per tensor) or col (per output channel) */
+  const double *filter_scales; /* [filter_quant_num] */
+  const int32_t *filter_zps;   /* [filter_quant_num] */
+} mi_matmul_desc;
+
+/* weight_host: int8 const weight; bias_host: int32 [col] or NULL.  Both are consumed during the call. */
+int mi_matmul_create(const mi_matmul_desc *desc, const int8_t *weight_host, const int32_t *bias_host,
+                     mi_matmul **out);
+/* a_dev: int8 [rows, deep]; c_dev: int8 [rows, col].  Asynchronous on `stream`. */
+int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
+/* Same with host tensors: copies in, runs, copies out, synchronises. */
+int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host);
+/* Derived per-channel parameters (arrays of `col` entries, any may be NULL): multiplier / shifts, the folded bias
+ * K*zx*zw - zx*sum(w) + bias, and the clamp bounds. */
+int mi_matmul_get_params(const mi_matmul *h, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift,
+                         int32_t *folded_bias, int32_t *act_min, int32_t *act_max);
+void mi_matmul_destroy(mi_matmul *h);
+
+/* ---- Conv2DFusion int8 (group 1: 1x1 and im2col; group == channels: depthwise) ----------------------------- */
+/* Replaces Convolution1x1Int8CPUKernel (LK/int8/convolution_1x1_int8.cc: InitBiasByzp :158-217, InitParam :359-413,
+ * Pre1x1Trans :435-444, Run :572-621), ConvolutionInt8CPUKernel (LK/int8/convolution_int8.cc: InitWeightBias :53-157,
+ * Run :248-263), ConvolutionDepthwiseInt8CPUKernel (LK/int8/convolution_depthwise_int8.cc:33-197), the quant setup
+ * of ConvolutionBaseCPUKernel (LK/base/convolution_base.cc:246-499) and the nnacl functions they call: Conv1x1Int8
+ * (NN/int8/conv1x1_int8.c:31-40), Conv1x1InputPack (NN/base/conv1x1_base.c:19-40), ConvInt8 /
+ * Im2ColPackUnitInt8Opt (NN/int8/conv_int8.c:758-913), MatMulInt8_8x8_r (NN/int8/matmul_int8.c:333-364),
+ * ConvDwInt8 / ConvDwInt8Post (NN/int8/conv_depthwise_int8.c:24-140).
+ * mi_conv_create returns MI_NOT_SUPPORT for what the provider must leave to the builtin kernels: 3x3 stride-1
+ * dilation-1 dense convolutions (the reference runs an integer Winograd there on x86, which is not an exact
+ * convolution) and grouped convolutions other than depthwise. */
+typedef struct mi_conv mi_conv;
+
+typedef struct mi_conv_desc {
+  int32_t in_channel, out_channel;
+  int32_t kernel_h, kernel_w, stride_h, stride_w, dilation_h, dilation_w;
+  int32_t pad_u, pad_d, pad_l, pad_r;
+  int32_t group; /* 1, or in_channel == out_channel == group for depthwise */
+  int32_t act_type;
+  double in_scale;
+  int32_t in_zp;
+  double out_scale;
+  int32_t out_zp;
+  int32_t filter_quant_num;    /* 1 or out_channel */
+  const double *filter_scales;
+  const int32_t *filter_zps;
+} mi_conv_desc;
+
+/* weight_host: [OC][KH][KW][IC] for group 1, [C][KH][KW] for depthwise; bias_host int32 [OC] or NULL. */
+int mi_conv_create(const mi_conv_desc *desc, const int8_t *weight_host, const int32_t *bias_host, mi_conv **out);
+/* Output spatial size for an input of in_h x in_w with the descriptor's explicit padding. */
+int mi_conv_out_shape(const mi_conv *h, int32_t in_h, int32_t in_w, int32_t *out_h, int32_t *out_w);
+/* SAME-mode padding as Lite's shape inference computes it (NN/infer/conv2d_infer.c:34-50). */
+int mi_conv_same_pad(int32_t in, int32_t kernel, int32_t stride, int32_t dilation, int32_t *pad_before,
+                     int32_t *pad_after, int32_t *out);
+/* in_dev: int8 NHWC [batch,in_h,in_w,IC]; out_dev: int8 NHWC [batch,out_h,out_w,OC]. */
+int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_dev,
+                void *stream);
+int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_host);
+void mi_conv_destroy(mi_conv *h);
+
+/* ---- DynamicQuant (fp32 -> int8, per tensor) --------------------------------------------------------------- */
+/* Replaces DynamicQuantCPUKernel for axis_num_ == 0 (LK/int8/dynamic_quant.cc: CalculateMinMax :118-143,
+ * CalculatePerlayerScaleZp :156-186, QuantData :220-234, Run :288-366) and CalculateMinMaxFp32
+ * (NN/int8/dynamic_quant_int8.c:19-27), DoQuantizeFp32ToInt8 (NN/int8/quant_dtype_cast_int8.c:180-203). */
+typedef struct mi_dynquant mi_dynquant;
+
+/* The {scale, zero point} a run produced, as it lives in device memory for chaining into mi_dynmm_run_chained. */
+typedef struct mi_dq_params {
+  double scale;  /* what DynamicQuant publishes on the output tensor (LiteQuantParam.scale) */
+  float scale_f; /* the same narrowed to float, as both consumers use it */
+  int32_t zero_point;
+  float real_min, real_max;
+} mi_dq_params;
+
+int mi_dynquant_create(int32_t symmetric, mi_dynquant **out);
+/* x_dev: fp32 [n]; q_dev: int8 [n].  Asynchronous; the parameters stay on the device. */
+int mi_dynquant_run(mi_dynquant *h, const float *x_dev, int64_t n, int8_t *q_dev, void *stream);
+/* Waits for the last run on `stream` and returns its parameters (what the provider writes with SetQuantParams). */
+int mi_dynquant_get_params(mi_dynquant *h, void *stream, mi_dq_params *params_host);
+/* Device address of the mi_dq_params block of the last run. */
+const mi_dq_params *mi_dynquant_device_params(const mi_dynquant *h);
+int mi_dynquant_run_host(mi_dynquant *h, const float *x_host, int64_t n, int8_t *q_host, mi_dq_params *params_host);
+void mi_dynquant_destroy(mi_dynquant *h);
+
+/* ---- dynamic-quant MatMul (int8 x int8 -> fp32) -------------------------------------------------------------- */
+/* Replaces MatmulDynamicInt8CPUKernel (LK/int8/matmul_dynamic_int8.cc: RunImpl :40-65, Run :86-147), its base
+ * (LK/int8/matmul_dynamic_base_int8.cc: InitFilterQuantParam :66-110, InitInputQuantParam :146-176, TransferB
+ * :178-202) and DynamicMatmul4x16x4AIWI / CalcWeightSums (NN/int8/dynamic_matmul_int8.c:99-143,380-399). */
+typedef struct mi_dynmm mi_dynmm;
+
+typedef struct mi_dynmm_desc {
+  int32_t deep, col;
+  int32_t b_transpose;
+  int32_t act_type;
+  int32_t filter_quant_num; /* 1 or col; the zero point used is always filter_zps[0] (matmul_dynamic_int8.cc:52) */
+  const double *filter_scales;
+  const int32_t *filter_zps;
+} mi_dynmm_desc;
+
+/* bias_host: fp32 [col] or NULL */
+int mi_dynmm_create(const mi_dynmm_desc *desc, const int8_t *weight_host, const float *bias_host, mi_dynmm **out);
+/* Input scale / zero point given by value (read from the input tensor's quant params at every Run). */
+int mi_dynmm_run(mi_dynmm *h, const int8_t *a_dev, int32_t rows, double in_scale, int32_t in_zp, float *c_dev,
+                 void *stream);
+/* Input scale / zero point read on the device from the block a preceding mi_dynquant_run wrote. */
+int mi_dynmm_run_chained(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_dq_params *params_dev,
+                         float *c_dev, void *stream);
+int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in_scale, int32_t in_zp,
+                      float *c_host);
+void mi_dynmm_destroy(mi_dynmm *h);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_INT8_H_ */

@@ -1,0 +1,36 @@
+"""Builds libmi355x_int8.so (HIP kernels + C ABI) for gfx950 with hipcc.  Cross-compiles without a GPU."""
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libmi355x_int8.so")
+SOURCES = ["capi.hip", "gemm_i8.hip", "gemv_i8.hip", "conv_i8.hip", "dynquant.hip"]
+# -ffp-contract=off: the float steps of DynamicQuant / dynamic MatMul and the host-side multiplier derivation are
+# separately rounded operations in the reference and must not be fused.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+
+
+def build_library(verbose=False):
+    objs = []
+    procs = []
+    for src in SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = ["hipcc"] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        if verbose or p.returncode != 0:
+            print(" ".join(cmd))
+            print(out)
+        if p.returncode != 0:
+            raise RuntimeError("hipcc failed for %s" % cmd[-3])
+    link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
+    subprocess.check_call(link)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

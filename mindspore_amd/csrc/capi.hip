@@ -1,0 +1,809 @@
+// C ABI of libmi355x_int8.so: handle objects that own packed weights, derived quant parameters and workspaces on
+// the device, and route each Run to the right kernel.  Everything the Lite CPU wrappers do at Prepare()/ReSize()
+// time happens in mi_*_create on the host with strict IEEE arithmetic (this file is compiled with
+// -ffp-contract=off); the device only ever sees integers and already-rounded floats.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <vector>
+
+#include "common.h"
+#include "quant_math.h"
+
+namespace mi {
+
+static thread_local char g_err[512] = "";
+static int g_device = -1;
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+static int ensure_device() {
+  if (g_device < 0) {
+    set_error("mi_init has not been called (or found no gfx950 device)");
+    return MI_ERROR;
+  }
+  MI_HIP_CHECK(hipSetDevice(g_device));
+  return MI_OK;
+}
+
+// ---- host-side quant parameter derivation -----------------------------------------------------------------------
+// QuantizeMultiplier (reference nnacl/int8/quantize.c:113-161): |m| = q * 2^shift, q in [0.5, 1);
+// mult = round_half_up(q * 2^31) with the carry renormalised; the sign moves onto mult.
+static void quantize_multiplier(double m, int32_t *mult, int32_t *shift) {
+  if (m == 0.0 || m != m) {
+    *mult = 0;
+    *shift = 0;
+    return;
+  }
+  if (isinf(m)) {
+    *mult = m < 0 ? INT32_MIN : INT32_MAX;
+    *shift = 0;
+    return;
+  }
+  int e = 0;
+  const double q = frexp(fabs(m), &e);
+  uint64_t sig = (uint64_t)ldexp(q, 53);
+  uint64_t r = ((sig >> 21) + 1u) >> 1;
+  if (r == ((uint64_t)1 << 31)) {
+    r >>= 1;
+    ++e;
+  }
+  *shift = e;
+  *mult = m < 0 ? -(int32_t)r : (int32_t)r;
+}
+
+static void round_param(double m, int32_t *mult, int32_t *ls, int32_t *rs) {
+  int32_t shift = 0;
+  quantize_multiplier(m, mult, &shift);
+  *ls = shift < 0 ? 0 : shift;
+  *rs = shift < 0 ? shift : 0;
+}
+
+static void requant_params(double sx, const double *sw, int n, double so, int32_t *mult, int32_t *ls, int32_t *rs) {
+  const float fx = (float)sx, fo = (float)so;
+  for (int i = 0; i < n; ++i) {
+    volatile float prod = fx * (float)sw[i];  // float product first, as QuantArg.scale_ is float
+    round_param((double)prod / (double)fo, &mult[i], &ls[i], &rs[i]);
+  }
+}
+
+static int32_t quantize_to_int8_unclamped(float real, float scale, int32_t zp) {
+  volatile float t = real / scale;
+  volatile float u = t + (float)zp;
+  const double r = round((double)u);
+  return (r >= -2147483648.0 && r <= 2147483647.0) ? (int32_t)r : INT32_MIN;
+}
+
+static void activation_range(int act, int32_t zp, float scale, int32_t *mn, int32_t *mx) {
+  int32_t lo = INT8_MIN, hi = INT8_MAX;
+  const int32_t q0 = quantize_to_int8_unclamped(0.0f, scale, zp), q6 = quantize_to_int8_unclamped(6.0f, scale, zp);
+  if (act == MI_ACT_RELU) {
+    lo = std::max(lo, q0);
+  } else if (act == MI_ACT_RELU6) {
+    lo = std::max(lo, q0);
+    hi = std::min(hi, q6);
+  }
+  *mn = lo;
+  *mx = hi;
+}
+
+// ---- device memory helpers ------------------------------------------------------------------------------------------
+struct DevBuf {
+  void *p = nullptr;
+  size_t bytes = 0;
+  int ensure(size_t want) {
+    if (want <= bytes) return MI_OK;
+    if (p != nullptr) {
+      MI_HIP_CHECK(hipFree(p));
+      p = nullptr;
+      bytes = 0;
+    }
+    const size_t sz = (want + 4095) & ~(size_t)4095;
+    if (hipMalloc(&p, sz) != hipSuccess) {
+      p = nullptr;
+      set_error("hipMalloc(%zu) failed", sz);
+      return MI_MEMORY_FAILED;
+    }
+    bytes = sz;
+    return MI_OK;
+  }
+  void release() {
+    if (p != nullptr) (void)hipFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+};
+
+template <typename T>
+static int upload(DevBuf *b, const std::vector<T> &v) {
+  int rc = b->ensure(v.size() * sizeof(T) + 16);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(b->p, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice));
+  return MI_OK;
+}
+
+// ---- shared "requantising GEMM operand" state: packed weights + per-channel epilogue arrays ------------------------
+struct RequantState {
+  int n = 0, k = 0, n_pad = 0, k_pad = 0;
+  DevBuf w, mult, bias2, rshift, lshift, zw;
+  std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
+  int32_t amin = -128, amax = 127, zo = 0;
+  bool has_zw = false, fast = false;
+
+  RequantParams params() const {
+    RequantParams rq;
+    rq.mult = static_cast<const int32_t *>(mult.p);
+    rq.bias2 = static_cast<const int32_t *>(bias2.p);
+    rq.rshift = static_cast<const int32_t *>(rshift.p);
+    rq.lshift = static_cast<const int32_t *>(lshift.p);
+    rq.zw = static_cast<const int32_t *>(zw.p);
+    rq.zo = zo;
+    rq.amin = amin;
+    rq.amax = amax;
+    rq.has_zw = has_zw ? 1 : 0;
+    rq.fast = fast ? 1 : 0;
+    return rq;
+  }
+
+  // w_nk: [n][k] row-major (already transposed if needed)
+  int build(const int8_t *w_nk, int n_, int k_, const int32_t *bias, double sx, int32_t zx, double so, int32_t zo_,
+            int nfilt, const double *sw, const int32_t *zws, int act, bool pack_weights) {
+    n = n_;
+    k = k_;
+    n_pad = round_up(n, kNPad);
+    k_pad = round_up(k, kKPad);
+    zo = zo_;
+    const bool peroc = nfilt > 1;
+    h_mult.assign(n_pad, 0);
+    h_ls.assign(n_pad, 0);
+    h_rs.assign(n_pad, 0);
+    h_bias2.assign(n_pad, 0);
+    std::vector<int32_t> m1(nfilt), l1(nfilt), r1(nfilt);
+    requant_params(sx, sw, nfilt, so, m1.data(), l1.data(), r1.data());
+    activation_range(act, zo, (float)so, &amin, &amax);
+    std::vector<int32_t> e(n_pad, 0), zwv(n_pad, 0);
+    has_zw = false;
+    fast = true;
+    for (int c = 0; c < n; ++c) {
+      const int qi = peroc ? c : 0;
+      h_mult[c] = m1[qi];
+      h_ls[c] = l1[qi];
+      h_rs[c] = r1[qi];
+      e[c] = std::min(31, -r1[qi]);
+      zwv[c] = zws[qi];
+      if (zwv[c] != 0) has_zw = true;
+      int32_t wsum = 0;
+      const int8_t *row = w_nk + (size_t)c * k;
+      for (int i = 0; i < k; ++i) wsum += row[i];
+      uint32_t v = (uint32_t)k * (uint32_t)zx * (uint32_t)zwv[c] - (uint32_t)zx * (uint32_t)wsum;
+      if (bias != nullptr) v += (uint32_t)bias[c];
+      h_bias2[c] = (int32_t)v;
+      // can the cheap rounding form be used?  needs ls == 0, 1 <= e <= 30, no saturation case, and
+      // |srdhm| + 2^(e-1) representable
+      const int64_t vmax = std::min<int64_t>((int64_t)1 << 31, (int64_t)k * 16384 + llabs((long long)h_bias2[c]) +
+                                                                   (int64_t)k * 128 * llabs((long long)zwv[c]));
+      const int64_t xmax = ((vmax * llabs((long long)h_mult[c])) >> 31) + 1;
+      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN ||
+          xmax + ((int64_t)1 << (e[c] - 1)) > INT32_MAX)
+        fast = false;
+    }
+    for (int c = n; c < n_pad; ++c) e[c] = 1;
+    int rc;
+    if ((rc = upload(&mult, h_mult)) != MI_OK) return rc;
+    if ((rc = upload(&bias2, h_bias2)) != MI_OK) return rc;
+    if ((rc = upload(&rshift, e)) != MI_OK) return rc;
+    if ((rc = upload(&lshift, h_ls)) != MI_OK) return rc;
+    if ((rc = upload(&zw, zwv)) != MI_OK) return rc;
+    if (pack_weights) {
+      std::vector<int8_t> packed((size_t)n_pad * k_pad, 0);
+      for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * k_pad, w_nk + (size_t)c * k, (size_t)k);
+      if ((rc = upload(&w, packed)) != MI_OK) return rc;
+    }
+    return MI_OK;
+  }
+
+  void release() {
+    w.release();
+    mult.release();
+    bias2.release();
+    rshift.release();
+    lshift.release();
+    zw.release();
+  }
+};
+
+static int check_filter_quant(int nfilt, int channels, const double *scales, const int32_t *zps) {
+  if (scales == nullptr || zps == nullptr) {
+    set_error("filter quant params are null");
+    return MI_NULL_PTR;
+  }
+  if (nfilt != 1 && nfilt != channels) {
+    set_error("filter_quant_num must be 1 or the channel count (%d), got %d", channels, nfilt);
+    return MI_PARAM_INVALID;
+  }
+  return MI_OK;
+}
+
+static std::vector<int8_t> to_nk(const int8_t *w, int n, int k, int b_transpose) {
+  std::vector<int8_t> out((size_t)n * k);
+  if (b_transpose) {
+    memcpy(out.data(), w, out.size());
+  } else {
+    for (int kk = 0; kk < k; ++kk)
+      for (int c = 0; c < n; ++c) out[(size_t)c * k + kk] = w[(size_t)kk * n + c];
+  }
+  return out;
+}
+
+// Activations must reach the GEMM/GEMV kernels as 16-byte aligned rows of k16 bytes; returns the pointer/stride to
+// use, copying through `ws` when the caller's layout does not qualify.
+static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_t stream, const int8_t **a_out,
+                        int64_t *lda_out, int *k16_out) {
+  const int k16 = round_up(k, 16);
+  if (k16 == k && (reinterpret_cast<uintptr_t>(a) & 15) == 0) {
+    *a_out = a;
+    *lda_out = k;
+    *k16_out = k;
+    return MI_OK;
+  }
+  int rc = ws->ensure((size_t)rows * k16);
+  if (rc != MI_OK) return rc;
+  rc = launch_pad_rows(a, k, rows, k, static_cast<int8_t *>(ws->p), k16, stream);
+  if (rc != MI_OK) return rc;
+  *a_out = static_cast<const int8_t *>(ws->p);
+  *lda_out = k16;
+  *k16_out = k16;
+  return MI_OK;
+}
+
+static int run_requant_gemm(const RequantState &st, const int8_t *a, int64_t lda, int rows, int k16, int8_t *c,
+                            hipStream_t stream) {
+  const RequantParams rq = st.params();
+  if (rows <= kGemvMaxRows && (int64_t)rows * k16 <= 150 * 1024)
+    return launch_gemv_requant(a, lda, rows, k16, static_cast<const int8_t *>(st.w.p), st.k_pad, st.n, rq, c, st.n,
+                               stream);
+  return launch_gemm_requant(a, lda, rows, k16, static_cast<const int8_t *>(st.w.p), st.k_pad, st.n, rq, c, st.n,
+                             stream);
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+// =====================================================================================================================
+struct mi_matmul {
+  RequantState st;
+  DevBuf a_ws, h_in, h_out;
+};
+
+struct mi_conv {
+  mi_conv_desc d;
+  bool depthwise = false, direct_1x1 = false;
+  int fill = 0;
+  RequantState st;
+  DevBuf w16, dw_bias, col_ws, h_in, h_out;
+};
+
+struct mi_dynquant {
+  int symmetric = 0;
+  DevBuf partials, params, h_in, h_out;
+};
+
+struct mi_dynmm {
+  int n = 0, k = 0, n_pad = 0, k_pad = 0, act = 0;
+  int32_t zw0 = 0;
+  bool has_bias = false;
+  DevBuf w, wscale, wsum, bias, a_ws, h_in, h_out;
+};
+
+extern "C" {
+
+int mi_init(int device) {
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+    set_error("no HIP device visible");
+    return MI_NOT_SUPPORT;
+  }
+  if (device < 0 || device >= count) {
+    set_error("device %d out of range (%d visible)", device, count);
+    return MI_PARAM_INVALID;
+  }
+  hipDeviceProp_t prop;
+  MI_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    set_error("device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+    return MI_NOT_SUPPORT;
+  }
+  MI_HIP_CHECK(hipSetDevice(device));
+  g_device = device;
+  return MI_OK;
+}
+
+const char *mi_last_error(void) { return g_err; }
+const char *mi_version(void) { return "mi355x_int8 0.1 (gfx950)"; }
+
+int mi_quantize_multiplier(double real_multiplier, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift) {
+  if (multiplier == nullptr || left_shift == nullptr || right_shift == nullptr) return MI_NULL_PTR;
+  round_param(real_multiplier, multiplier, left_shift, right_shift);
+  return MI_OK;
+}
+
+int mi_activation_range(int32_t act_type, int32_t out_zp, double out_scale, int32_t *act_min, int32_t *act_max) {
+  if (act_min == nullptr || act_max == nullptr) return MI_NULL_PTR;
+  activation_range(act_type, out_zp, (float)out_scale, act_min, act_max);
+  return MI_OK;
+}
+
+int mi_requant_params(double in_scale, const double *filter_scales, int32_t n, double out_scale, int32_t *multiplier,
+                      int32_t *left_shift, int32_t *right_shift) {
+  if (filter_scales == nullptr || multiplier == nullptr || left_shift == nullptr || right_shift == nullptr)
+    return MI_NULL_PTR;
+  if (n < 0) return MI_PARAM_INVALID;
+  requant_params(in_scale, filter_scales, n, out_scale, multiplier, left_shift, right_shift);
+  return MI_OK;
+}
+
+int32_t mi_multiply_by_quantized_multiplier(int32_t value, int32_t multiplier, int32_t left_shift,
+                                            int32_t right_shift) {
+  return mul_by_quant_mult(value, multiplier, left_shift, right_shift);
+}
+
+// ---------------------------------------------------------------------------------------------------------- matmul
+int mi_matmul_create(const mi_matmul_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_matmul **out) {
+  if (d == nullptr || weight_host == nullptr || out == nullptr) {
+    set_error("mi_matmul_create: null argument");
+    return MI_NULL_PTR;
+  }
+  *out = nullptr;
+  if (d->deep <= 0 || d->col <= 0 || (d->act_type != MI_ACT_NONE && d->act_type != MI_ACT_RELU &&
+                                      d->act_type != MI_ACT_RELU6)) {
+    set_error("mi_matmul_create: bad shape/activation deep=%d col=%d act=%d", d->deep, d->col, d->act_type);
+    return MI_PARAM_INVALID;
+  }
+  int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
+  if (rc != MI_OK) return rc;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  mi_matmul *h = new (std::nothrow) mi_matmul();
+  if (h == nullptr) return MI_MEMORY_FAILED;
+  const std::vector<int8_t> w_nk = to_nk(weight_host, d->col, d->deep, d->b_transpose);
+  rc = h->st.build(w_nk.data(), d->col, d->deep, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
+                   d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
+  if (rc != MI_OK) {
+    mi_matmul_destroy(h);
+    return rc;
+  }
+  *out = h;
+  return MI_OK;
+}
+
+int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream) {
+  if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
+    set_error("mi_matmul_run: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) {
+    set_error("mi_matmul_run: rows=%d", rows);
+    return MI_PARAM_INVALID;
+  }
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  if ((rc = prepare_rows(a_dev, rows, h->st.k, &h->a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, s);
+}
+
+int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host) {
+  if (h == nullptr || a_host == nullptr || c_host == nullptr) {
+    set_error("mi_matmul_run_host: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) return MI_PARAM_INVALID;
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  const size_t in_bytes = (size_t)rows * h->st.k, out_bytes = (size_t)rows * h->st.n;
+  if ((rc = h->h_in.ensure(in_bytes)) != MI_OK || (rc = h->h_out.ensure(out_bytes)) != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(h->h_in.p, a_host, in_bytes, hipMemcpyHostToDevice));
+  rc = mi_matmul_run(h, static_cast<const int8_t *>(h->h_in.p), rows, static_cast<int8_t *>(h->h_out.p), nullptr);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(c_host, h->h_out.p, out_bytes, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+
+int mi_matmul_get_params(const mi_matmul *h, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift,
+                         int32_t *folded_bias, int32_t *act_min, int32_t *act_max) {
+  if (h == nullptr) return MI_NULL_PTR;
+  const size_t bytes = (size_t)h->st.n * sizeof(int32_t);
+  if (multiplier) memcpy(multiplier, h->st.h_mult.data(), bytes);
+  if (left_shift) memcpy(left_shift, h->st.h_ls.data(), bytes);
+  if (right_shift) memcpy(right_shift, h->st.h_rs.data(), bytes);
+  if (folded_bias) memcpy(folded_bias, h->st.h_bias2.data(), bytes);
+  if (act_min) *act_min = h->st.amin;
+  if (act_max) *act_max = h->st.amax;
+  return MI_OK;
+}
+
+void mi_matmul_destroy(mi_matmul *h) {
+  if (h == nullptr) return;
+  h->st.release();
+  h->a_ws.release();
+  h->h_in.release();
+  h->h_out.release();
+  delete h;
+}
+
+// ------------------------------------------------------------------------------------------------------------ conv
+int mi_conv_same_pad(int32_t in, int32_t kernel, int32_t stride, int32_t dilation, int32_t *pad_before,
+                     int32_t *pad_after, int32_t *out) {
+  if (pad_before == nullptr || pad_after == nullptr || out == nullptr) return MI_NULL_PTR;
+  if (stride <= 0 || kernel <= 0 || dilation <= 0 || in <= 0) return MI_PARAM_INVALID;
+  const int o = (in + stride - 1) / stride;
+  const int all = (o - 1) * stride + (kernel - 1) * dilation + 1 - in;
+  *out = o;
+  if (all < 0) {
+    *pad_before = *pad_after = 0;
+  } else {
+    *pad_before = all / 2;
+    *pad_after = all - all / 2;
+  }
+  return MI_OK;
+}
+
+int mi_conv_create(const mi_conv_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_conv **out) {
+  if (d == nullptr || weight_host == nullptr || out == nullptr) {
+    set_error("mi_conv_create: null argument");
+    return MI_NULL_PTR;
+  }
+  *out = nullptr;
+  if (d->in_channel <= 0 || d->out_channel <= 0 || d->kernel_h <= 0 || d->kernel_w <= 0 || d->stride_h <= 0 ||
+      d->stride_w <= 0 || d->dilation_h <= 0 || d->dilation_w <= 0 || d->pad_u < 0 || d->pad_d < 0 || d->pad_l < 0 ||
+      d->pad_r < 0 || d->group <= 0 ||
+      (d->act_type != MI_ACT_NONE && d->act_type != MI_ACT_RELU && d->act_type != MI_ACT_RELU6)) {
+    set_error("mi_conv_create: bad descriptor");
+    return MI_PARAM_INVALID;
+  }
+  const bool depthwise = d->group > 1 && d->group == d->in_channel && d->group == d->out_channel;
+  if (d->group != 1 && !depthwise) {
+    set_error("grouped convolution (group=%d) is left to the builtin kernel", d->group);
+    return MI_NOT_SUPPORT;
+  }
+  if (!depthwise && d->kernel_h == 3 && d->kernel_w == 3 && d->stride_h == 1 && d->stride_w == 1 &&
+      d->dilation_h == 1 && d->dilation_w == 1) {
+    set_error("3x3 stride-1 dilation-1 convolution is left to the builtin (Winograd) kernel");
+    return MI_NOT_SUPPORT;
+  }
+  int rc = check_filter_quant(d->filter_quant_num, d->out_channel, d->filter_scales, d->filter_zps);
+  if (rc != MI_OK) return rc;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  mi_conv *h = new (std::nothrow) mi_conv();
+  if (h == nullptr) return MI_MEMORY_FAILED;
+  h->d = *d;
+  h->d.filter_scales = nullptr;
+  h->d.filter_zps = nullptr;
+  h->depthwise = depthwise;
+  const int oc = d->out_channel;
+  if (depthwise) {
+    const int plane = d->kernel_h * d->kernel_w;
+    // requant arrays only; the folded bias is not used (zero points are applied to the operands)
+    std::vector<int8_t> dummy((size_t)oc, 0);
+    rc = h->st.build(dummy.data(), oc, 1, nullptr, d->in_scale, 0, d->out_scale, d->out_zp, d->filter_quant_num,
+                     d->filter_scales, d->filter_zps, d->act_type, false);
+    std::vector<int16_t> w16((size_t)plane * oc);
+    for (int c = 0; c < oc; ++c) {
+      const int32_t z = d->filter_quant_num > 1 ? d->filter_zps[c] : d->filter_zps[0];
+      for (int t = 0; t < plane; ++t) w16[(size_t)t * oc + c] = (int16_t)((int32_t)weight_host[(size_t)c * plane + t] - z);
+    }
+    std::vector<int32_t> b(oc, 0);
+    if (bias_host != nullptr) memcpy(b.data(), bias_host, (size_t)oc * sizeof(int32_t));
+    if (rc == MI_OK) rc = upload(&h->w16, w16);
+    if (rc == MI_OK) rc = upload(&h->dw_bias, b);
+  } else {
+    const int kdim = d->kernel_h * d->kernel_w * d->in_channel;
+    const bool is_1x1 = d->kernel_h == 1 && d->kernel_w == 1;
+    const bool trivial_geom = d->stride_h == 1 && d->stride_w == 1 && d->pad_u == 0 && d->pad_d == 0 &&
+                              d->pad_l == 0 && d->pad_r == 0;
+    h->direct_1x1 = is_1x1 && trivial_geom;
+    h->fill = is_1x1 ? 0 : d->in_zp;
+    rc = h->st.build(weight_host, oc, kdim, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
+                     d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
+  }
+  if (rc != MI_OK) {
+    mi_conv_destroy(h);
+    return rc;
+  }
+  *out = h;
+  return MI_OK;
+}
+
+int mi_conv_out_shape(const mi_conv *h, int32_t in_h, int32_t in_w, int32_t *out_h, int32_t *out_w) {
+  if (h == nullptr || out_h == nullptr || out_w == nullptr) return MI_NULL_PTR;
+  const mi_conv_desc &d = h->d;
+  const int eh = (d.kernel_h - 1) * d.dilation_h + 1, ew = (d.kernel_w - 1) * d.dilation_w + 1;
+  if (in_h <= 0 || in_w <= 0 || in_h + d.pad_u + d.pad_d < eh || in_w + d.pad_l + d.pad_r < ew) {
+    set_error("mi_conv_out_shape: input %dx%d too small", in_h, in_w);
+    return MI_PARAM_INVALID;
+  }
+  *out_h = (in_h + d.pad_u + d.pad_d - eh) / d.stride_h + 1;
+  *out_w = (in_w + d.pad_l + d.pad_r - ew) / d.stride_w + 1;
+  return MI_OK;
+}
+
+int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_dev,
+                void *stream) {
+  if (h == nullptr || in_dev == nullptr || out_dev == nullptr) {
+    set_error("mi_conv_run: null argument");
+    return MI_NULL_PTR;
+  }
+  if (batch < 0) return MI_PARAM_INVALID;
+  int oh = 0, ow = 0;
+  int rc = mi_conv_out_shape(h, in_h, in_w, &oh, &ow);
+  if (rc != MI_OK) return rc;
+  if (batch == 0) return MI_OK;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const mi_conv_desc &d = h->d;
+  ConvGeom g{batch,       in_h,       in_w,       d.in_channel, oh,           ow,           d.out_channel, d.kernel_h,
+             d.kernel_w,  d.stride_h, d.stride_w, d.dilation_h, d.dilation_w, d.pad_u,      d.pad_l};
+  const int64_t pixels = (int64_t)batch * oh * ow;
+  if (pixels > 0x7fffffff) {
+    set_error("mi_conv_run: too many output pixels");
+    return MI_PARAM_INVALID;
+  }
+  if (h->depthwise) {
+    return launch_conv_dw(in_dev, g, static_cast<const int16_t *>(h->w16.p), static_cast<const int32_t *>(h->dw_bias.p),
+                          (int)(int8_t)d.in_zp, h->st.params(), out_dev, s);
+  }
+  const int k = h->st.k;
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  if (h->direct_1x1) {
+    if ((rc = prepare_rows(in_dev, (int)pixels, k, &h->col_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  } else {
+    k16 = round_up(k, 16);
+    if ((rc = h->col_ws.ensure((size_t)pixels * k16)) != MI_OK) return rc;
+    if ((rc = launch_im2col(in_dev, g, h->fill, static_cast<int8_t *>(h->col_ws.p), k16, s)) != MI_OK) return rc;
+    a = static_cast<const int8_t *>(h->col_ws.p);
+    lda = k16;
+  }
+  return run_requant_gemm(h->st, a, lda, (int)pixels, k16, out_dev, s);
+}
+
+int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_host) {
+  if (h == nullptr || in_host == nullptr || out_host == nullptr) {
+    set_error("mi_conv_run_host: null argument");
+    return MI_NULL_PTR;
+  }
+  int oh = 0, ow = 0;
+  int rc = mi_conv_out_shape(h, in_h, in_w, &oh, &ow);
+  if (rc != MI_OK) return rc;
+  if (batch < 0) return MI_PARAM_INVALID;
+  if (batch == 0) return MI_OK;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  const size_t in_bytes = (size_t)batch * in_h * in_w * h->d.in_channel;
+  const size_t out_bytes = (size_t)batch * oh * ow * h->d.out_channel;
+  if ((rc = h->h_in.ensure(in_bytes)) != MI_OK || (rc = h->h_out.ensure(out_bytes)) != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(h->h_in.p, in_host, in_bytes, hipMemcpyHostToDevice));
+  rc = mi_conv_run(h, static_cast<const int8_t *>(h->h_in.p), batch, in_h, in_w, static_cast<int8_t *>(h->h_out.p),
+                   nullptr);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(out_host, h->h_out.p, out_bytes, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+
+void mi_conv_destroy(mi_conv *h) {
+  if (h == nullptr) return;
+  h->st.release();
+  h->w16.release();
+  h->dw_bias.release();
+  h->col_ws.release();
+  h->h_in.release();
+  h->h_out.release();
+  delete h;
+}
+
+// ------------------------------------------------------------------------------------------------------- dynquant
+int mi_dynquant_create(int32_t symmetric, mi_dynquant **out) {
+  if (out == nullptr) return MI_NULL_PTR;
+  *out = nullptr;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  mi_dynquant *h = new (std::nothrow) mi_dynquant();
+  if (h == nullptr) return MI_MEMORY_FAILED;
+  h->symmetric = symmetric ? 1 : 0;
+  if ((rc = h->partials.ensure(sizeof(float2) * kDqMaxBlocks)) != MI_OK ||
+      (rc = h->params.ensure(sizeof(mi_dq_params))) != MI_OK) {
+    mi_dynquant_destroy(h);
+    return rc;
+  }
+  *out = h;
+  return MI_OK;
+}
+
+int mi_dynquant_run(mi_dynquant *h, const float *x_dev, int64_t n, int8_t *q_dev, void *stream) {
+  if (h == nullptr || (n > 0 && (x_dev == nullptr || q_dev == nullptr))) {
+    set_error("mi_dynquant_run: null argument");
+    return MI_NULL_PTR;
+  }
+  if (n < 0) return MI_PARAM_INVALID;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  return launch_dynquant(x_dev, n, h->symmetric, static_cast<float2 *>(h->partials.p),
+                         static_cast<mi_dq_params *>(h->params.p), q_dev, static_cast<hipStream_t>(stream));
+}
+
+int mi_dynquant_get_params(mi_dynquant *h, void *stream, mi_dq_params *params_host) {
+  if (h == nullptr || params_host == nullptr) return MI_NULL_PTR;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI_HIP_CHECK(hipMemcpyAsync(params_host, h->params.p, sizeof(mi_dq_params), hipMemcpyDeviceToHost, s));
+  MI_HIP_CHECK(hipStreamSynchronize(s));
+  return MI_OK;
+}
+
+const mi_dq_params *mi_dynquant_device_params(const mi_dynquant *h) {
+  return h == nullptr ? nullptr : static_cast<const mi_dq_params *>(h->params.p);
+}
+
+int mi_dynquant_run_host(mi_dynquant *h, const float *x_host, int64_t n, int8_t *q_host, mi_dq_params *params_host) {
+  if (h == nullptr || params_host == nullptr || (n > 0 && (x_host == nullptr || q_host == nullptr))) {
+    set_error("mi_dynquant_run_host: null argument");
+    return MI_NULL_PTR;
+  }
+  if (n < 0) return MI_PARAM_INVALID;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  if ((rc = h->h_in.ensure((size_t)n * 4 + 16)) != MI_OK || (rc = h->h_out.ensure((size_t)n + 16)) != MI_OK) return rc;
+  if (n > 0) MI_HIP_CHECK(hipMemcpy(h->h_in.p, x_host, (size_t)n * 4, hipMemcpyHostToDevice));
+  rc = mi_dynquant_run(h, static_cast<const float *>(h->h_in.p), n, static_cast<int8_t *>(h->h_out.p), nullptr);
+  if (rc != MI_OK) return rc;
+  if ((rc = mi_dynquant_get_params(h, nullptr, params_host)) != MI_OK) return rc;
+  if (n > 0) MI_HIP_CHECK(hipMemcpy(q_host, h->h_out.p, (size_t)n, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+
+void mi_dynquant_destroy(mi_dynquant *h) {
+  if (h == nullptr) return;
+  h->partials.release();
+  h->params.release();
+  h->h_in.release();
+  h->h_out.release();
+  delete h;
+}
+
+// ---------------------------------------------------------------------------------------------------------- dynmm
+int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {
+  if (d == nullptr || weight_host == nullptr || out == nullptr) {
+    set_error("mi_dynmm_create: null argument");
+    return MI_NULL_PTR;
+  }
+  *out = nullptr;
+  if (d->deep <= 0 || d->col <= 0 || (d->act_type != MI_ACT_NONE && d->act_type != MI_ACT_RELU &&
+                                      d->act_type != MI_ACT_RELU6)) {
+    set_error("mi_dynmm_create: bad shape/activation");
+    return MI_PARAM_INVALID;
+  }
+  int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
+  if (rc != MI_OK) return rc;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  mi_dynmm *h = new (std::nothrow) mi_dynmm();
+  if (h == nullptr) return MI_MEMORY_FAILED;
+  h->n = d->col;
+  h->k = d->deep;
+  h->n_pad = round_up(h->n, kNPad);
+  h->k_pad = round_up(h->k, kKPad);
+  h->act = d->act_type;
+  h->zw0 = d->filter_zps[0];
+  h->has_bias = bias_host != nullptr;
+  const std::vector<int8_t> w_nk = to_nk(weight_host, h->n, h->k, d->b_transpose);
+  std::vector<int8_t> packed((size_t)h->n_pad * h->k_pad, 0);
+  std::vector<float> ws(h->n_pad, 0.0f), bs(h->n_pad, 0.0f);
+  std::vector<int32_t> wsum(h->n_pad, 0);
+  for (int c = 0; c < h->n; ++c) {
+    memcpy(packed.data() + (size_t)c * h->k_pad, w_nk.data() + (size_t)c * h->k, (size_t)h->k);
+    int32_t s = 0;
+    for (int i = 0; i < h->k; ++i) s += w_nk[(size_t)c * h->k + i];
+    wsum[c] = s;
+    ws[c] = (float)d->filter_scales[d->filter_quant_num > 1 ? c : 0];
+    if (bias_host != nullptr) bs[c] = bias_host[c];
+  }
+  rc = upload(&h->w, packed);
+  if (rc == MI_OK) rc = upload(&h->wscale, ws);
+  if (rc == MI_OK) rc = upload(&h->wsum, wsum);
+  if (rc == MI_OK && h->has_bias) rc = upload(&h->bias, bs);
+  if (rc != MI_OK) {
+    mi_dynmm_destroy(h);
+    return rc;
+  }
+  *out = h;
+  return MI_OK;
+}
+
+static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float sx, int32_t zx,
+                          const mi_dq_params *qp_dev, float *c_dev, hipStream_t s) {
+  if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
+    set_error("mi_dynmm_run: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) return MI_PARAM_INVALID;
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  if ((rc = prepare_rows(a_dev, rows, h->k, &h->a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  DequantParams dq;
+  dq.wscale = static_cast<const float *>(h->wscale.p);
+  dq.bias = h->has_bias ? static_cast<const float *>(h->bias.p) : nullptr;
+  dq.wsum = static_cast<const int32_t *>(h->wsum.p);
+  dq.qp_dev = qp_dev;
+  dq.sx = sx;
+  dq.zx = zx;
+  dq.zw0 = h->zw0;
+  dq.deep = h->k;
+  dq.act = h->act;
+  return launch_gemm_dequant(a, lda, rows, k16, static_cast<const int8_t *>(h->w.p), h->k_pad, h->n, dq, c_dev, h->n,
+                             s);
+}
+
+int mi_dynmm_run(mi_dynmm *h, const int8_t *a_dev, int32_t rows, double in_scale, int32_t in_zp, float *c_dev,
+                 void *stream) {
+  return dynmm_run_impl(h, a_dev, rows, (float)in_scale, in_zp, nullptr, c_dev, static_cast<hipStream_t>(stream));
+}
+
+int mi_dynmm_run_chained(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_dq_params *params_dev, float *c_dev,
+                         void *stream) {
+  if (params_dev == nullptr) {
+    set_error("mi_dynmm_run_chained: params_dev is null");
+    return MI_NULL_PTR;
+  }
+  return dynmm_run_impl(h, a_dev, rows, 0.0f, 0, params_dev, c_dev, static_cast<hipStream_t>(stream));
+}
+
+int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in_scale, int32_t in_zp, float *c_host) {
+  if (h == nullptr || a_host == nullptr || c_host == nullptr) {
+    set_error("mi_dynmm_run_host: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) return MI_PARAM_INVALID;
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  const size_t in_bytes = (size_t)rows * h->k, out_bytes = (size_t)rows * h->n * sizeof(float);
+  if ((rc = h->h_in.ensure(in_bytes)) != MI_OK || (rc = h->h_out.ensure(out_bytes)) != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(h->h_in.p, a_host, in_bytes, hipMemcpyHostToDevice));
+  rc = mi_dynmm_run(h, static_cast<const int8_t *>(h->h_in.p), rows, in_scale, in_zp, static_cast<float *>(h->h_out.p),
+                    nullptr);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(c_host, h->h_out.p, out_bytes, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+
+void mi_dynmm_destroy(mi_dynmm *h) {
+  if (h == nullptr) return;
+  h->w.release();
+  h->wscale.release();
+  h->wsum.release();
+  h->bias.release();
+  h->a_ws.release();
+  h->h_in.release();
+  h->h_out.release();
+  delete h;
+}
+
+}  // extern "C"

@@ -1,0 +1,85 @@
+// Internal declarations shared by the HIP translation units of libmi355x_int8.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355x_int8.h"
+
+namespace mi {
+
+void set_error(const char *fmt, ...);
+
+#define MI_HIP_CHECK(expr)                                                                   \
+  do {                                                                                       \
+    hipError_t _e = (expr);                                                                  \
+    if (_e != hipSuccess) {                                                                  \
+      mi::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+      return MI_ERROR;                                                                       \
+    }                                                                                        \
+  } while (0)
+
+inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
+inline int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Weight rows (output channels) and the contraction dimension are padded so that no kernel needs bounds checks on
+// the weight operand: rows to a multiple of kNPad, K to a multiple of kKPad (bytes), zero filled.
+constexpr int kNPad = 256;
+constexpr int kKPad = 128;
+
+// ---- int8 requantising epilogue parameters (device arrays are padded to kNPad entries) ----
+struct RequantParams {
+  const int32_t *mult;    // 31-bit mantissa per channel
+  const int32_t *bias2;   // K*zx*zw - zx*sum(w) + bias
+  const int32_t *rshift;  // e = -right_shift clamped to [0, 31]
+  const int32_t *lshift;  // left shift (generic path only)
+  const int32_t *zw;      // weight zero point per channel (HAS_ZW only)
+  int32_t zo, amin, amax;
+  int has_zw;  // any weight zero point is non-zero -> input row sums are needed
+  int fast;    // host proved: all lshift == 0, 1 <= e <= 30, no mult == INT32_MIN, rounding add cannot overflow
+};
+
+// ---- fp32 dequantising epilogue (dynamic-quant MatMul) ----
+struct DequantParams {
+  const float *wscale;           // (float)filter_scale per channel (padded; per-tensor is broadcast at Prepare)
+  const float *bias;             // fp32 bias or nullptr
+  const int32_t *wsum;           // sum_k w[n][k]
+  const mi_dq_params *qp_dev;    // input scale / zero point on the device, or nullptr -> use sx / zx below
+  float sx;
+  int32_t zx;
+  int32_t zw0;
+  int32_t deep;  // true K
+  int32_t act;
+};
+
+// A: int8 activations [M][lda] (lda in bytes, multiple of 16, base 16-byte aligned, K % 16 == 0);
+// W: packed weights [n_pad][k_pad]; C: [M][ldc] elements.
+int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+                        const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
+int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+                        const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
+
+// Skinny-M path (m <= kGemvMaxRows): streams the weights once with 16-byte coalesced loads.
+constexpr int kGemvMaxRows = 8;
+int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+                        const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
+
+// Copies [rows][k] (row stride src_ld bytes) into a zero-padded [rows][k16] buffer, k16 = round_up(k, 16).
+int launch_pad_rows(const int8_t *src, int64_t src_ld, int rows, int k, int8_t *dst, int k16, hipStream_t stream);
+
+struct ConvGeom {
+  int batch, in_h, in_w, in_c, out_h, out_w, out_c;
+  int kernel_h, kernel_w, stride_h, stride_w, dilation_h, dilation_w, pad_u, pad_l;
+};
+// im2col into [batch*out_h*out_w][k16] with K order (kh, kw, ic); out-of-image taps are `fill`, the K tail is zero.
+int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, int k16, hipStream_t stream);
+// Depthwise conv + requantisation, weights pre-offset to int16 [KH*KW][C].
+int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
+                   const RequantParams &rq, int8_t *out, hipStream_t stream);
+
+// DynamicQuant: per-block min/max partials, then quantise (every block re-reduces the partials).
+constexpr int kDqMaxBlocks = 1024;
+int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, mi_dq_params *params, int8_t *q,
+                    hipStream_t stream);
+
+}  // namespace mi

@@ -1,0 +1,144 @@
+// Data-movement kernels in front of the GEMM for Conv2D int8, and the depthwise convolution.
+//   pad_rows : [rows][k] -> zero-padded [rows][k16]           (activations whose K is not a multiple of 16)
+//   im2col   : NHWC image -> [pixels][k16], K order (kh, kw, ic) as Im2ColPackUnitInt8Opt lays rows out
+//              (reference mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/conv_int8.c:758-807); taps outside
+//              the image take `fill`: the input zero point for the im2col convolution (conv_int8.c:877) and 0 for
+//              the strided/padded 1x1 convolution (Conv1x1InputPack into a zeroed buffer,
+//              .../nnacl/base/conv1x1_base.c:19-40, mindspore/lite/src/litert/kernel/cpu/int8/
+//              convolution_1x1_int8.cc:396)
+//   conv_dw  : depthwise conv + requantisation (ConvDwInt8 / ConvDwInt8Post,
+//              .../nnacl/int8/conv_depthwise_int8.c:24-140)
+// All three are HBM/latency bound byte movers: one thread produces 16 contiguous output bytes (or one output
+// element for the depthwise kernel, consecutive threads on consecutive channels) so stores coalesce.
+#include "common.h"
+#include "quant_math.h"
+
+namespace mi {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void pad_rows_kernel(const int8_t *__restrict__ src, int64_t src_ld, int rows,
+                                                       int k, int8_t *__restrict__ dst, int k16) {
+  const int chunks_per_row = k16 >> 4;
+  const int64_t total = (int64_t)rows * chunks_per_row;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int row = (int)(idx / chunks_per_row), ch = (int)(idx - (int64_t)row * chunks_per_row);
+    const int8_t *s = src + (int64_t)row * src_ld + ch * 16;
+    union {
+      v4i v;
+      int8_t b[16];
+    } u;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) u.b[j] = (ch * 16 + j < k) ? s[j] : (int8_t)0;
+    *reinterpret_cast<v4i *>(dst + (int64_t)row * k16 + ch * 16) = u.v;
+  }
+}
+
+int launch_pad_rows(const int8_t *src, int64_t src_ld, int rows, int k, int8_t *dst, int k16, hipStream_t stream) {
+  const int64_t total = (int64_t)rows * (k16 >> 4);
+  const int blocks = (int)((total + 255) / 256 < 65535 * 16 ? (total + 255) / 256 : 65535 * 16);
+  hipLaunchKernelGGL(pad_rows_kernel, dim3(blocks > 0 ? blocks : 1), dim3(256), 0, stream, src, src_ld, rows, k, dst,
+                     k16);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+__global__ __launch_bounds__(256) void im2col_kernel(const int8_t *__restrict__ in, ConvGeom g, int fill,
+                                                     int8_t *__restrict__ dst, int k16) {
+  const int kdim = g.kernel_h * g.kernel_w * g.in_c;
+  const int chunks_per_row = k16 >> 4;
+  const int64_t pixels = (int64_t)g.batch * g.out_h * g.out_w;
+  const int64_t total = pixels * chunks_per_row;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t p = idx / chunks_per_row;
+    const int ch = (int)(idx - p * chunks_per_row);
+    const int b = (int)(p / ((int64_t)g.out_h * g.out_w));
+    const int rem = (int)(p - (int64_t)b * g.out_h * g.out_w);
+    const int oh = rem / g.out_w, ow = rem - oh * g.out_w;
+    const int ih0 = oh * g.stride_h - g.pad_u, iw0 = ow * g.stride_w - g.pad_l;
+    const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * g.in_c;
+    union {
+      v4i v;
+      int8_t b[16];
+    } u;
+    int kk = ch * 16;
+    int tap = kk / g.in_c, ic = kk - tap * g.in_c;
+    int kh = tap / g.kernel_w, kw = tap - kh * g.kernel_w;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      int8_t val = 0;
+      if (kk + j < kdim) {
+        const int ih = ih0 + kh * g.dilation_h, iw = iw0 + kw * g.dilation_w;
+        const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+        val = inside ? img[((int64_t)ih * g.in_w + iw) * g.in_c + ic] : (int8_t)fill;
+      }
+      u.b[j] = val;
+      if (++ic == g.in_c) {
+        ic = 0;
+        if (++kw == g.kernel_w) {
+          kw = 0;
+          ++kh;
+        }
+      }
+    }
+    *reinterpret_cast<v4i *>(dst + p * k16 + ch * 16) = u.v;
+  }
+}
+
+int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, int k16, hipStream_t stream) {
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * (k16 >> 4);
+  const int64_t want = (total + 255) / 256;
+  const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
+  hipLaunchKernelGGL(im2col_kernel, dim3(blocks), dim3(256), 0, stream, in, g, fill, dst, k16);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+__global__ __launch_bounds__(256) void conv_dw_kernel(const int8_t *__restrict__ in, ConvGeom g,
+                                                      const int16_t *__restrict__ w16,
+                                                      const int32_t *__restrict__ bias, int zx8, RequantParams rq,
+                                                      int8_t *__restrict__ out) {
+  const int ch = g.out_c;
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * ch;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t p = idx / ch;
+    const int c = (int)(idx - p * ch);
+    const int b = (int)(p / ((int64_t)g.out_h * g.out_w));
+    const int rem = (int)(p - (int64_t)b * g.out_h * g.out_w);
+    const int oh = rem / g.out_w, ow = rem - oh * g.out_w;
+    const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * ch;
+    uint32_t acc = (uint32_t)bias[c];
+    for (int kh = 0; kh < g.kernel_h; ++kh) {
+      const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
+      if (ih < 0 || ih >= g.in_h) continue;
+      for (int kw = 0; kw < g.kernel_w; ++kw) {
+        const int iw = ow * g.stride_w - g.pad_l + kw * g.dilation_w;
+        if (iw < 0 || iw >= g.in_w) continue;
+        const int16_t xv = (int16_t)((int)img[((int64_t)ih * g.in_w + iw) * ch + c] - zx8);
+        const int16_t wv = w16[(kh * g.kernel_w + kw) * ch + c];
+        acc += (uint32_t)((int32_t)xv * (int32_t)wv);
+      }
+    }
+    const int32_t mult = rq.mult[c], e = rq.rshift[c], ls = rq.lshift[c];
+    int32_t y = rdiv_pot(srdhm((int32_t)(acc << ls), mult), e);
+    y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+    y = y > rq.amin ? y : rq.amin;  // MSMAX first, then MSMIN (conv_depthwise_int8.c:49-50)
+    y = y < rq.amax ? y : rq.amax;
+    out[idx] = (int8_t)y;
+  }
+}
+
+int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
+                   const RequantParams &rq, int8_t *out, hipStream_t stream) {
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * g.out_c;
+  const int64_t want = (total + 255) / 256;
+  const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
+  hipLaunchKernelGGL(conv_dw_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+}  // namespace mi

@@ -1,0 +1,263 @@
+"""Host-side mirror of the Lite int8 kernel wrappers over the C ABI.
+
+Each class plays the role of one reference CPU kernel class (same inputs, same quant-parameter meaning, same error
+behaviour: construction = Prepare(), ``run`` = Run()):
+
+  MatmulInt8Kernel / FullconnectionInt8Kernel  <-  MatmulInt8CPUKernel / FullconnectionInt8CPUKernel
+  ConvolutionInt8Kernel                        <-  Convolution1x1Int8 / ConvolutionInt8 / ConvolutionDepthwiseInt8
+  DynamicQuantKernel                           <-  DynamicQuantCPUKernel
+  MatmulDynamicInt8Kernel                      <-  MatmulDynamicInt8CPUKernel
+
+``run`` accepts either NumPy arrays (host tensors: copied to the GPU, computed, copied back) or torch CUDA tensors
+(device tensors: computed in place on torch's current stream, no copies).  torch is only used as a device-memory
+and stream provider.
+"""
+import ctypes as C
+from collections import namedtuple
+
+import numpy as np
+
+from . import lib as _lib
+
+QuantParam = namedtuple("QuantParam", ["scale", "zero_point"])
+ACT_NONE, ACT_RELU, ACT_RELU6 = _lib.ACT_NONE, _lib.ACT_RELU, _lib.ACT_RELU6
+
+
+def _is_torch(x):
+    return type(x).__module__.startswith("torch")
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _quant_arrays(params):
+    params = list(params)
+    if not params:
+        raise ValueError("at least one weight quant param is required")
+    scales = (C.c_double * len(params))(*[float(p.scale) for p in params])
+    zps = (C.c_int32 * len(params))(*[int(p.zero_point) for p in params])
+    return len(params), scales, zps
+
+
+def _host_i8(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype != np.int8:
+        raise TypeError("expected an int8 tensor, got %s" % a.dtype)
+    return a
+
+
+class _Handle:
+    _destroy = None
+
+    def __init__(self):
+        self._h = C.c_void_p(None)
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            getattr(_lib.load(), self._destroy)(self._h)
+            self._h = C.c_void_p(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class MatmulInt8Kernel(_Handle):
+    """Full-quant int8 MatMul: C = requant(A x W^T).  weight is [N, K] when transpose_b else [K, N]; bias int32 [N]."""
+    _destroy = "mi_matmul_destroy"
+
+    def __init__(self, weight, bias, in_quant, weight_quant, out_quant, transpose_b=True, act=ACT_NONE, device=0):
+        super().__init__()
+        L = _lib.init(device)
+        weight = _host_i8(weight)
+        if weight.ndim != 2:
+            raise ValueError("weight must be 2-D")
+        self.n, self.k = (weight.shape if transpose_b else weight.shape[::-1])
+        if bias is not None:
+            bias = np.ascontiguousarray(bias)
+            if bias.dtype != np.int32:
+                raise TypeError("full-quant MatMul needs an int32 bias")  # matmul_base_int8.cc:420-424
+            if bias.size != self.n:
+                raise ValueError("bias has %d entries, expected %d" % (bias.size, self.n))
+        nq, scales, zps = _quant_arrays(weight_quant)
+        d = _lib.MatmulDesc(self.k, self.n, 1 if transpose_b else 0, act, float(in_quant.scale),
+                            int(in_quant.zero_point), float(out_quant.scale), int(out_quant.zero_point), nq, scales,
+                            zps)
+        _lib.check(L.mi_matmul_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
+                                      C.byref(self._h)), "mi_matmul_create")
+
+    def run(self, a):
+        L = _lib.load()
+        if _is_torch(a):
+            import torch
+            if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.shape[-1] != self.k:
+                raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % self.k)
+            rows = a.numel() // self.k
+            out = torch.empty(a.shape[:-1] + (self.n,), dtype=torch.int8, device=a.device)
+            _lib.check(L.mi_matmul_run(self._h, a.data_ptr(), rows, out.data_ptr(), _stream()), "mi_matmul_run")
+            return out
+        a = _host_i8(a)
+        if a.shape[-1] != self.k:
+            raise ValueError("expected [..., %d], got %s" % (self.k, a.shape))
+        rows = a.size // self.k
+        out = np.empty(a.shape[:-1] + (self.n,), np.int8)
+        _lib.check(L.mi_matmul_run_host(self._h, a.ctypes.data, rows, out.ctypes.data), "mi_matmul_run_host")
+        return out
+
+    def params(self):
+        L = _lib.load()
+        arrs = [np.empty(self.n, np.int32) for _ in range(4)]
+        lo, hi = C.c_int32(0), C.c_int32(0)
+        _lib.check(L.mi_matmul_get_params(self._h, *[x.ctypes.data for x in arrs], C.byref(lo), C.byref(hi)),
+                   "mi_matmul_get_params")
+        return dict(multiplier=arrs[0], left_shift=arrs[1], right_shift=arrs[2], folded_bias=arrs[3],
+                    act_min=lo.value, act_max=hi.value)
+
+
+class FullconnectionInt8Kernel(MatmulInt8Kernel):
+    """FullConnection always uses a [N, K] weight (fullconnection_int8.cc:33-34)."""
+
+    def __init__(self, weight, bias, in_quant, weight_quant, out_quant, act=ACT_NONE, device=0):
+        super().__init__(weight, bias, in_quant, weight_quant, out_quant, True, act, device)
+
+
+class ConvolutionInt8Kernel(_Handle):
+    """Conv2DFusion int8, NHWC.  weight [OC, KH, KW, IC] (group 1) or [C, KH, KW] (depthwise, group == C).
+    pad = (up, down, left, right).  Raises MiError with code MI_NOT_SUPPORT for the cases a provider must decline."""
+    _destroy = "mi_conv_destroy"
+
+    def __init__(self, weight, bias, in_quant, weight_quant, out_quant, stride=(1, 1), dilation=(1, 1),
+                 pad=(0, 0, 0, 0), group=1, act=ACT_NONE, device=0):
+        super().__init__()
+        L = _lib.init(device)
+        weight = _host_i8(weight)
+        if group == 1:
+            if weight.ndim != 4:
+                raise ValueError("weight must be [OC, KH, KW, IC]")
+            oc, kh, kw, ic = weight.shape
+        else:
+            if weight.ndim == 4 and weight.shape[3] == 1:
+                weight = weight.reshape(weight.shape[:3])
+            if weight.ndim != 3:
+                raise ValueError("depthwise weight must be [C, KH, KW]")
+            oc, kh, kw = weight.shape
+            ic = oc
+        if bias is not None:
+            bias = np.ascontiguousarray(bias)
+            if bias.dtype != np.int32 or bias.size != oc:
+                raise ValueError("bias must be int32 [%d]" % oc)
+        self.ic, self.oc = ic, oc
+        nq, scales, zps = _quant_arrays(weight_quant)
+        d = _lib.ConvDesc(ic, oc, kh, kw, stride[0], stride[1], dilation[0], dilation[1], pad[0], pad[1], pad[2],
+                          pad[3], group, act, float(in_quant.scale), int(in_quant.zero_point),
+                          float(out_quant.scale), int(out_quant.zero_point), nq, scales, zps)
+        _lib.check(L.mi_conv_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
+                                    C.byref(self._h)), "mi_conv_create")
+
+    def out_shape(self, in_h, in_w):
+        oh, ow = C.c_int32(0), C.c_int32(0)
+        _lib.check(_lib.load().mi_conv_out_shape(self._h, in_h, in_w, C.byref(oh), C.byref(ow)), "mi_conv_out_shape")
+        return oh.value, ow.value
+
+    def run(self, x):
+        L = _lib.load()
+        if x.ndim != 4 or x.shape[3] != self.ic:
+            raise ValueError("expected NHWC with %d channels, got %s" % (self.ic, tuple(x.shape)))
+        b, ih, iw, _ = x.shape
+        oh, ow = self.out_shape(ih, iw)
+        if _is_torch(x):
+            import torch
+            if x.dtype != torch.int8 or not x.is_cuda or not x.is_contiguous():
+                raise ValueError("expected a contiguous CUDA int8 tensor")
+            out = torch.empty((b, oh, ow, self.oc), dtype=torch.int8, device=x.device)
+            _lib.check(L.mi_conv_run(self._h, x.data_ptr(), b, ih, iw, out.data_ptr(), _stream()), "mi_conv_run")
+            return out
+        x = _host_i8(x)
+        out = np.empty((b, oh, ow, self.oc), np.int8)
+        _lib.check(L.mi_conv_run_host(self._h, x.ctypes.data, b, ih, iw, out.ctypes.data), "mi_conv_run_host")
+        return out
+
+
+class DynamicQuantKernel(_Handle):
+    """Per-tensor DynamicQuant fp32 -> int8.  ``run`` returns (q, QuantParam) -- the QuantParam is what the
+    reference kernel writes onto its output tensor."""
+    _destroy = "mi_dynquant_destroy"
+
+    def __init__(self, symmetric=False, device=0):
+        super().__init__()
+        L = _lib.init(device)
+        _lib.check(L.mi_dynquant_create(1 if symmetric else 0, C.byref(self._h)), "mi_dynquant_create")
+        self.last = None
+
+    def run(self, x, fetch_params=True):
+        L = _lib.load()
+        p = _lib.DqParams()
+        if _is_torch(x):
+            import torch
+            if x.dtype != torch.float32 or not x.is_cuda or not x.is_contiguous():
+                raise ValueError("expected a contiguous CUDA float32 tensor")
+            q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+            s = _stream()
+            _lib.check(L.mi_dynquant_run(self._h, x.data_ptr(), x.numel(), q.data_ptr(), s), "mi_dynquant_run")
+            if not fetch_params:
+                return q, None
+            _lib.check(L.mi_dynquant_get_params(self._h, s, C.byref(p)), "mi_dynquant_get_params")
+        else:
+            x = np.ascontiguousarray(x)
+            if x.dtype != np.float32:
+                raise TypeError("DynamicQuant needs a float32 input")  # dynamic_quant.cc:389-395
+            q = np.empty(x.shape, np.int8)
+            _lib.check(L.mi_dynquant_run_host(self._h, x.ctypes.data, x.size, q.ctypes.data, C.byref(p)),
+                       "mi_dynquant_run_host")
+        self.last = p
+        return q, QuantParam(p.scale, p.zero_point)
+
+    def device_params(self):
+        return _lib.load().mi_dynquant_device_params(self._h)
+
+
+class MatmulDynamicInt8Kernel(_Handle):
+    """Dynamic-quant MatMul: int8 activations (scale / zero point supplied at every run) x int8 weights -> fp32."""
+    _destroy = "mi_dynmm_destroy"
+
+    def __init__(self, weight, bias, weight_quant, transpose_b=True, act=ACT_NONE, device=0):
+        super().__init__()
+        L = _lib.init(device)
+        weight = _host_i8(weight)
+        self.n, self.k = (weight.shape if transpose_b else weight.shape[::-1])
+        if bias is not None:
+            bias = np.ascontiguousarray(bias)
+            if bias.dtype != np.float32:
+                raise TypeError("dynamic MatMul needs a float32 bias")  # matmul_dynamic_int8.cc:48-51
+            if bias.size != self.n:
+                raise ValueError("bias has %d entries, expected %d" % (bias.size, self.n))
+        nq, scales, zps = _quant_arrays(weight_quant)
+        d = _lib.DynmmDesc(self.k, self.n, 1 if transpose_b else 0, act, nq, scales, zps)
+        _lib.check(L.mi_dynmm_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
+                                     C.byref(self._h)), "mi_dynmm_create")
+
+    def run(self, a, in_quant=None, params_dev=None):
+        L = _lib.load()
+        if _is_torch(a):
+            import torch
+            if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.shape[-1] != self.k:
+                raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % self.k)
+            rows = a.numel() // self.k
+            out = torch.empty(a.shape[:-1] + (self.n,), dtype=torch.float32, device=a.device)
+            if params_dev is not None:
+                _lib.check(L.mi_dynmm_run_chained(self._h, a.data_ptr(), rows, params_dev, out.data_ptr(), _stream()),
+                           "mi_dynmm_run_chained")
+            else:
+                _lib.check(L.mi_dynmm_run(self._h, a.data_ptr(), rows, float(in_quant.scale),
+                                          int(in_quant.zero_point), out.data_ptr(), _stream()), "mi_dynmm_run")
+            return out
+        a = _host_i8(a)
+        rows = a.size // self.k
+        out = np.empty(a.shape[:-1] + (self.n,), np.float32)
+        _lib.check(L.mi_dynmm_run_host(self._h, a.ctypes.data, rows, float(in_quant.scale), int(in_quant.zero_point),
+                                       out.ctypes.data), "mi_dynmm_run_host")
+        return out

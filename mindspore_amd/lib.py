@@ -1,0 +1,130 @@
+"""ctypes binding of libmi355x_int8.so (the C ABI declared in include/mi355x_int8.h).
+
+There is no CPU fallback: if the library is missing, or no gfx950 GPU is present when a kernel is created, the
+call raises."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libmi355x_int8.so")
+
+MI_OK, MI_ERROR, MI_NULL_PTR, MI_PARAM_INVALID, MI_MEMORY_FAILED, MI_NOT_SUPPORT = 0, -1, -2, -3, -6, -7
+ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
+
+EXPORTS = [
+    "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_activation_range", "mi_requant_params",
+    "mi_multiply_by_quantized_multiplier",
+    "mi_matmul_create", "mi_matmul_run", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
+    "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_destroy",
+    "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
+    "mi_dynquant_run_host", "mi_dynquant_destroy",
+    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_destroy",
+]
+
+
+class MatmulDesc(C.Structure):
+    _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
+                ("in_scale", C.c_double), ("in_zp", C.c_int32), ("out_scale", C.c_double), ("out_zp", C.c_int32),
+                ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
+                ("filter_zps", C.POINTER(C.c_int32))]
+
+
+class ConvDesc(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "in_channel", "out_channel", "kernel_h", "kernel_w", "stride_h", "stride_w", "dilation_h", "dilation_w",
+        "pad_u", "pad_d", "pad_l", "pad_r", "group", "act_type")] + [
+        ("in_scale", C.c_double), ("in_zp", C.c_int32), ("out_scale", C.c_double), ("out_zp", C.c_int32),
+        ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
+        ("filter_zps", C.POINTER(C.c_int32))]
+
+
+class DynmmDesc(C.Structure):
+    _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
+                ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
+                ("filter_zps", C.POINTER(C.c_int32))]
+
+
+class DqParams(C.Structure):
+    _fields_ = [("scale", C.c_double), ("scale_f", C.c_float), ("zero_point", C.c_int32), ("real_min", C.c_float),
+                ("real_max", C.c_float)]
+
+
+class MiError(RuntimeError):
+    def __init__(self, what, code, message):
+        super().__init__("%s failed with status %d: %s" % (what, code, message))
+        self.code = code
+
+
+_lib = None
+_initialised = False
+
+
+def load():
+    """Loads the shared library (no GPU needed for this step)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("%s is not built: run `python -m mindspore_amd.build` (hipcc, gfx950)" % LIB_PATH)
+    # A process must hold ONE HIP runtime.  PyTorch ships its own libamdhip64 (same SONAME as /opt/rocm's); when this
+    # process is going to use torch for device memory and streams, torch's copy has to be the one that is loaded, so
+    # import it before the dynamic loader resolves this library's dependency.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, dbl = C.c_void_p, C.c_int32, C.c_int64, C.c_double
+    pi32 = C.POINTER(C.c_int32)
+    L.mi_init.argtypes = [C.c_int]
+    L.mi_last_error.restype = C.c_char_p
+    L.mi_version.restype = C.c_char_p
+    L.mi_quantize_multiplier.argtypes = [dbl, pi32, pi32, pi32]
+    L.mi_activation_range.argtypes = [i32, i32, dbl, pi32, pi32]
+    L.mi_requant_params.argtypes = [dbl, C.POINTER(dbl), i32, dbl, pi32, pi32, pi32]
+    L.mi_multiply_by_quantized_multiplier.argtypes = [i32, i32, i32, i32]
+    L.mi_multiply_by_quantized_multiplier.restype = i32
+    L.mi_matmul_create.argtypes = [C.POINTER(MatmulDesc), vp, vp, C.POINTER(vp)]
+    L.mi_matmul_run.argtypes = [vp, vp, i32, vp, vp]
+    L.mi_matmul_run_host.argtypes = [vp, vp, i32, vp]
+    L.mi_matmul_get_params.argtypes = [vp, vp, vp, vp, vp, pi32, pi32]
+    L.mi_matmul_destroy.argtypes = [vp]
+    L.mi_matmul_destroy.restype = None
+    L.mi_conv_create.argtypes = [C.POINTER(ConvDesc), vp, vp, C.POINTER(vp)]
+    L.mi_conv_out_shape.argtypes = [vp, i32, i32, pi32, pi32]
+    L.mi_conv_same_pad.argtypes = [i32, i32, i32, i32, pi32, pi32, pi32]
+    L.mi_conv_run.argtypes = [vp, vp, i32, i32, i32, vp, vp]
+    L.mi_conv_run_host.argtypes = [vp, vp, i32, i32, i32, vp]
+    L.mi_conv_destroy.argtypes = [vp]
+    L.mi_conv_destroy.restype = None
+    L.mi_dynquant_create.argtypes = [i32, C.POINTER(vp)]
+    L.mi_dynquant_run.argtypes = [vp, vp, i64, vp, vp]
+    L.mi_dynquant_get_params.argtypes = [vp, vp, C.POINTER(DqParams)]
+    L.mi_dynquant_device_params.argtypes = [vp]
+    L.mi_dynquant_device_params.restype = vp
+    L.mi_dynquant_run_host.argtypes = [vp, vp, i64, vp, C.POINTER(DqParams)]
+    L.mi_dynquant_destroy.argtypes = [vp]
+    L.mi_dynquant_destroy.restype = None
+    L.mi_dynmm_create.argtypes = [C.POINTER(DynmmDesc), vp, vp, C.POINTER(vp)]
+    L.mi_dynmm_run.argtypes = [vp, vp, i32, dbl, i32, vp, vp]
+    L.mi_dynmm_run_chained.argtypes = [vp, vp, i32, vp, vp, vp]
+    L.mi_dynmm_run_host.argtypes = [vp, vp, i32, dbl, i32, vp]
+    L.mi_dynmm_destroy.argtypes = [vp]
+    L.mi_dynmm_destroy.restype = None
+    _lib = L
+    return L
+
+
+def check(code, what):
+    if code != MI_OK:
+        raise MiError(what, code, load().mi_last_error().decode())
+
+
+def init(device=0):
+    """Selects the GPU; raises if there is no gfx950 device."""
+    global _initialised
+    L = load()
+    if not _initialised:
+        check(L.mi_init(device), "mi_init")
+        _initialised = True
+    return L

@@ -69,7 +69,7 @@ def gemm_c5(size, seed=0):
     m = n = k = size
     sw = s.uniform(1e-4, 1e-2, (n,)).astype(np.float32).astype(np.float64)
     sx = 0.02
-    so = float(np.float32(sx * float(np.mean(sw)) * np.sqrt(k) * 40.0))
+    so = float(np.float32(sx * float(np.mean(sw)) * np.sqrt(k) * 150.0))
     return dict(
         a=s.integers(-128, 127, (m, k)).astype(np.int8), w=s.integers(-128, 127, (n, k)).astype(np.int8),
         bias=s.integers(-5000, 5000, (n,)).astype(np.int32), sx=sx, zx=7, sw=sw, zw=np.zeros(n, np.int32), so=so,
@@ -86,7 +86,7 @@ def gemv_c4(name, n, k, m, seed=0):
     w = np.clip(np.round(s.normal((n, k)) * 32.0), -127, 127).astype(np.int8)
     sw = s.uniform(0.001, 0.01, (n,)).astype(np.float32).astype(np.float64)
     sx = 0.05
-    so = float(np.float32(sx * float(np.mean(sw)) * np.sqrt(k) * 32.0 * 40.0 / 2.0))
+    so = float(np.float32(sx * float(np.mean(sw)) * np.sqrt(k) * 32.0 * 2.0))
     return dict(
         a=s.integers(-128, 127, (m, k)).astype(np.int8), w=w, bias=s.integers(-5000, 5000, (n,)).astype(np.int32),
         sx=sx, zx=int(s.integers(-8, 8, (1,))[0]), sw=sw, zw=np.zeros(n, np.int32), so=so, zo=0, act=0)

@@ -1,0 +1,291 @@
+"""GPU parity: every entry point of the C ABI against the CPU oracle (bit-exact for int8 outputs, bit-exact for the
+fp32 outputs of the dynamic MatMul, exact scale/zero point for DynamicQuant) and against the committed golden
+vectors produced by the compiled nnacl."""
+import os
+
+import numpy as np
+import pytest
+
+from mindspore_amd import kernels as K
+from mindspore_amd.kernels import QuantParam as QP
+from oracle.pyoracle import conv_shape
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "small_cases.npz")
+
+
+def _qps(sw, zw):
+    return [QP(float(s), int(z)) for s, z in zip(np.atleast_1d(sw), np.atleast_1d(zw))]
+
+
+def _mm_case(rng, m, n, k, peroc, zwnz, hb, act, bt=True, so_mul=100.0):
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w_nk = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    nf = n if peroc else 1
+    sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+    zw = rng.integers(-10, 11, nf).astype(np.int32) if zwnz else np.zeros(nf, np.int32)
+    bias = rng.integers(-5000, 5001, n).astype(np.int32) if hb else None
+    sx, zx = float(rng.uniform(0.01, 0.05)), int(rng.integers(-20, 21))
+    so = float(sx * sw.mean() * np.sqrt(k) * so_mul)
+    zo = int(rng.integers(-20, 21))
+    w = w_nk if bt else np.ascontiguousarray(w_nk.T)
+    return dict(a=a, w=w, bias=bias, sx=sx, zx=zx, sw=sw, zw=zw, so=so, zo=zo, act=act, b_transpose=bt)
+
+
+def _gpu_matmul(case, device_tensors=False):
+    kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
+                              QP(case["so"], case["zo"]), case["b_transpose"], case["act"])
+    if device_tensors:
+        import torch
+        out = kern.run(torch.from_numpy(case["a"]).cuda())
+        torch.cuda.synchronize()
+        return out.cpu().numpy(), kern
+    return kern.run(case["a"]), kern
+
+
+MM_SHAPES = [(1, 1, 1), (1, 64, 16), (2, 5, 7), (3, 100, 15), (4, 256, 128), (5, 260, 129), (7, 33, 1000), (8, 512, 768),
+             (9, 64, 64), (31, 31, 31), (64, 64, 128), (65, 65, 130), (128, 768, 768), (129, 257, 513),
+             (300, 100, 17), (500, 1030, 96), (1000, 3, 256), (2049, 1100, 64)]
+
+
+@pytest.mark.parametrize("m,n,k", MM_SHAPES)
+def test_matmul_shapes(orc, m, n, k):
+    rng = np.random.default_rng(m * 7919 + n * 31 + k)
+    orc.set_threads(16)
+    for it in range(4):
+        case = _mm_case(rng, m, n, k, bool(it & 1), bool(it & 2), it != 2, [0, 1, 3, 0][it], it != 3)
+        got, _ = _gpu_matmul(case, device_tensors=bool(it & 1))
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
+
+
+def test_matmul_generic_rounding_paths(orc):
+    """Cases the fast epilogue must not take: real multiplier >= 1 (left shift), shift 0, huge bias (wrap)."""
+    rng = np.random.default_rng(5)
+    for m in (3, 200):
+        for so_mul in (1e-4, 1e-3, 0.02):
+            case = _mm_case(rng, m, 70, 40, True, True, True, 0, True, so_mul)
+            case["bias"] = rng.integers(-2 ** 31, 2 ** 31 - 1, 70).astype(np.int32)
+            got, kern = _gpu_matmul(case)
+            assert np.array_equal(got, orc.matmul_int8(**case)), (m, so_mul)
+            p = kern.params()
+            mult, ls, rs = orc.requant_params(case["sx"], case["sw"], case["so"])
+            assert np.array_equal(p["multiplier"], mult) and np.array_equal(p["left_shift"], ls)
+            assert np.array_equal(p["right_shift"], rs)
+
+
+def test_matmul_reuse_and_row_counts(orc):
+    """One handle, many row counts (GEMV path, each GEMM tile choice, and back)."""
+    rng = np.random.default_rng(6)
+    case = _mm_case(rng, 1, 384, 256, True, False, True, 0)
+    kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
+                              QP(case["so"], case["zo"]), True, 0)
+    for m in (1, 8, 9, 700, 3, 5000, 2):
+        a = rng.integers(-128, 128, (m, 256), dtype=np.int8)
+        case["a"] = a
+        assert np.array_equal(kern.run(a), orc.matmul_int8(**case)), m
+
+
+def test_golden_small_cases(orc):
+    g = np.load(GOLDEN)
+    for i in range(int(g["mm_count"][0])):
+        p = "mm%d_" % i
+        sx, zx, so, zo, act, bt, hb = g[p + "meta"]
+        kern = K.MatmulInt8Kernel(g[p + "w"], g[p + "bias"] if hb else None, QP(sx, int(zx)),
+                                  _qps(g[p + "sw"], g[p + "zw"]), QP(so, int(zo)), bool(bt), int(act))
+        assert np.array_equal(kern.run(g[p + "a"]), g[p + "c"]), p
+    for i in range(int(g["cv_count"][0])):
+        p = "cv%d_" % i
+        sx, zx, so, zo, act, hb = g[p + "meta"]
+        kh, kw, sh, sw_, dh, dw_, pu, pd, pl, pr, depthwise = [int(v) for v in g[p + "geom"]]
+        w = g[p + "w"]
+        kern = K.ConvolutionInt8Kernel(w, g[p + "bias"] if hb else None, QP(sx, int(zx)),
+                                       _qps(g[p + "sw"], g[p + "zw"]), QP(so, int(zo)), (sh, sw_), (dh, dw_),
+                                       (pu, pd, pl, pr), w.shape[0] if depthwise else 1, int(act))
+        assert np.array_equal(kern.run(g[p + "x"]), g[p + "y"]), p
+    for i in range(int(g["dq_count"][0])):
+        p = "dq%d_" % i
+        s, z, sym = g[p + "meta"]
+        q, qp = K.DynamicQuantKernel(bool(sym)).run(g[p + "x"])
+        assert qp.scale == s and qp.zero_point == int(z), p
+        assert np.array_equal(q, g[p + "q"]), p
+    for i in range(int(g["dm_count"][0])):
+        p = "dm%d_" % i
+        sx, zx, act, bt, hb = g[p + "meta"]
+        kern = K.MatmulDynamicInt8Kernel(g[p + "w"], g[p + "bias"] if hb else None, _qps(g[p + "sw"], g[p + "zw"]),
+                                         bool(bt), int(act))
+        got = kern.run(g[p + "a"], QP(sx, int(zx)))
+        assert np.array_equal(got.view(np.uint32), g[p + "c"].view(np.uint32)), p
+
+
+CONV_CASES = [
+    (1, 5, 5, 3, 4, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1)),
+    (2, 6, 7, 5, 9, (3, 3), (2, 1), (1, 1), (1, 1, 1, 1)),
+    (1, 8, 8, 4, 8, (5, 3), (1, 1), (1, 1), (2, 2, 1, 1)),
+    (1, 9, 9, 2, 3, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2)),
+    (1, 4, 6, 16, 5, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (2, 5, 5, 7, 6, (1, 1), (2, 2), (1, 1), (0, 0, 0, 0)),
+    (1, 5, 5, 3, 10, (1, 1), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (1, 6, 6, 3, 4, (1, 1), (2, 2), (1, 1), (1, 0, 1, 0)),
+    (1, 7, 5, 3, 17, (2, 2), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (1, 40, 40, 32, 64, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1)),
+    (3, 28, 28, 64, 300, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
+    (1, 30, 30, 24, 16, (7, 7), (2, 2), (1, 1), (3, 3, 3, 3)),
+]
+
+
+def _conv_case(rng, b, ih, iw, ic, oc, kernel, stride, dil, pad, peroc, zwnz, hb, act, dw=False):
+    shape = conv_shape(b, ih, iw, ic, oc, kernel, stride, dil, pad)
+    x = rng.integers(-128, 128, (b, ih, iw, ic), dtype=np.int8)
+    w = rng.integers(-128, 128, (oc, kernel[0], kernel[1]) if dw else (oc, kernel[0], kernel[1], ic), dtype=np.int8)
+    nf = oc if peroc else 1
+    sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+    zw = rng.integers(-10, 11, nf).astype(np.int32) if zwnz else np.zeros(nf, np.int32)
+    bias = rng.integers(-3000, 3001, oc).astype(np.int32) if hb else None
+    sx, zx = float(rng.uniform(0.01, 0.05)), int(rng.integers(-20, 21))
+    kdim = kernel[0] * kernel[1] * (1 if dw else ic)
+    so = float(sx * sw.mean() * np.sqrt(kdim) * 100)
+    zo = int(rng.integers(-20, 21))
+    return dict(x=x, w=w, bias=bias, shape=shape, sx=sx, zx=zx, sw=sw, zw=zw, so=so, zo=zo, act=act)
+
+
+def _gpu_conv(case, stride, dil, pad, group=1, device_tensors=False):
+    kern = K.ConvolutionInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
+                                   QP(case["so"], case["zo"]), stride, dil, pad, group, case["act"])
+    if device_tensors:
+        import torch
+        out = kern.run(torch.from_numpy(case["x"]).cuda())
+        torch.cuda.synchronize()
+        return out.cpu().numpy()
+    return kern.run(case["x"])
+
+
+@pytest.mark.parametrize("idx", range(len(CONV_CASES)))
+def test_conv_cases(orc, idx):
+    rng = np.random.default_rng(900 + idx)
+    orc.set_threads(16)
+    b, ih, iw, ic, oc, kernel, stride, dil, pad = CONV_CASES[idx]
+    for it in range(4):
+        case = _conv_case(rng, b, ih, iw, ic, oc, kernel, stride, dil, pad, bool(it & 1), bool(it & 2), it != 3,
+                          [0, 1, 3, 0][it])
+        got = _gpu_conv(case, stride, dil, pad, 1, device_tensors=bool(it & 1))
+        want = orc.conv_int8(**case)
+        assert np.array_equal(got, want), (idx, it, int((got != want).sum()))
+
+
+DW_CASES = [
+    (1, 6, 6, 5, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (2, 7, 5, 8, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1)),
+    (1, 9, 9, 3, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2)),
+    (1, 56, 56, 96, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
+    (1, 15, 18, 16, (5, 5), (1, 2), (1, 1), (2, 2, 2, 2)),
+]
+
+
+@pytest.mark.parametrize("idx", range(len(DW_CASES)))
+def test_depthwise_cases(orc, idx):
+    rng = np.random.default_rng(950 + idx)
+    orc.set_threads(16)
+    b, ih, iw, ch, kernel, stride, dil, pad = DW_CASES[idx]
+    for it in range(4):
+        case = _conv_case(rng, b, ih, iw, ch, ch, kernel, stride, dil, pad, bool(it & 1), bool(it & 2), it != 3,
+                          [0, 1, 3, 0][it], dw=True)
+        got = _gpu_conv(case, stride, dil, pad, ch, device_tensors=bool(it & 1))
+        assert np.array_equal(got, orc.conv_dw_int8(**case)), (idx, it)
+
+
+def test_conv_declines_what_the_provider_must_not_claim():
+    w = np.zeros((8, 3, 3, 4), np.int8)
+    with pytest.raises(K._lib.MiError) as e:
+        K.ConvolutionInt8Kernel(w, None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0), (1, 1), (1, 1), (1, 1, 1, 1))
+    assert e.value.code == K._lib.MI_NOT_SUPPORT
+    with pytest.raises(K._lib.MiError) as e:  # grouped, not depthwise
+        K.ConvolutionInt8Kernel(np.zeros((8, 3, 3), np.int8), None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0), (2, 2),
+                                group=4)
+    assert e.value.code == K._lib.MI_NOT_SUPPORT
+
+
+def _dq_inputs():
+    rng = np.random.default_rng(300)
+    xs = [rng.standard_normal(5000).astype(np.float32), rng.standard_normal((37, 91)).astype(np.float32) * 5 + 3,
+          np.zeros(700, np.float32), np.full(1000, 2.5, np.float32), np.array([1.0], np.float32),
+          rng.uniform(-1e-3, 1e-3, 4096).astype(np.float32), np.linspace(-7.5, 9.25, 3001, dtype=np.float32),
+          (rng.standard_normal(2048) * 1e6).astype(np.float32), rng.standard_normal(1 << 20).astype(np.float32),
+          rng.standard_normal(4099 * 257).astype(np.float32) * 3]
+    sp = rng.standard_normal(3000).astype(np.float32)
+    sp[5], sp[77], sp[900] = np.nan, 12.5, -13.25
+    xs.append(sp)
+    xs.append(np.array([np.inf, -np.inf, 1.0, -2.0, 3e38, -3e38, np.nan, 0.0] * 9, np.float32))
+    return xs
+
+
+def test_dynamic_quant(orc):
+    import torch
+    for i, x in enumerate(_dq_inputs()):
+        for sym in (False, True):
+            kern = K.DynamicQuantKernel(sym)
+            q_ref, s_ref, z_ref = orc.dynamic_quant(x, sym)
+            q, qp = kern.run(x)
+            assert qp.scale == s_ref and qp.zero_point == z_ref, (i, sym, qp, s_ref, z_ref)
+            assert np.array_equal(q, q_ref), (i, sym)
+            xt = torch.from_numpy(x).cuda()
+            q2, qp2 = kern.run(xt)
+            assert qp2 == qp and np.array_equal(q2.cpu().numpy(), q_ref)
+            # unaligned device pointer
+            if x.size > 8:
+                q3, qp3 = kern.run(xt.reshape(-1)[1:])
+                q3r, s3, z3 = orc.dynamic_quant(x.reshape(-1)[1:], sym)
+                assert qp3.scale == s3 and qp3.zero_point == z3 and np.array_equal(q3.cpu().numpy(), q3r)
+
+
+def test_dynamic_matmul(orc):
+    import torch
+    rng = np.random.default_rng(401)
+    orc.set_threads(16)
+    for it, (m, n, k) in enumerate([(1, 1, 1), (5, 9, 17), (33, 70, 64), (130, 65, 300), (9, 256, 1000),
+                                    (700, 300, 129), (64, 2304, 768)]):
+        a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+        w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        nf = n if it & 1 else 1
+        sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+        zw = np.full(nf, 0 if it & 2 else int(rng.integers(-5, 6)), np.int32)
+        bias = rng.standard_normal(n).astype(np.float32) if it & 4 else None
+        sx, zx, act = float(rng.uniform(0.01, 0.1)), int(rng.integers(-128, 128)), [0, 1, 3][it % 3]
+        bt = it != 3
+        wmem = w if bt else np.ascontiguousarray(w.T)
+        kern = K.MatmulDynamicInt8Kernel(wmem, bias, _qps(sw, zw), bt, act)
+        want = orc.dynamic_matmul(a, wmem, bias, sx, zx, sw, zw, act, bt)
+        got = kern.run(a, QP(sx, zx))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (it, m, n, k)
+        got2 = kern.run(torch.from_numpy(a).cuda(), QP(sx, zx)).cpu().numpy()
+        assert np.array_equal(got2.view(np.uint32), want.view(np.uint32))
+
+
+def test_dynamic_quant_chained_into_matmul(orc):
+    """DynamicQuant -> dynamic MatMul with the scale / zero point handed over in device memory."""
+    import torch
+    rng = np.random.default_rng(402)
+    x = (rng.standard_normal((200, 96)) * 2).astype(np.float32)
+    w = rng.integers(-127, 128, (80, 96), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, 80).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(80).astype(np.float32)
+    dq = K.DynamicQuantKernel(False)
+    mm = K.MatmulDynamicInt8Kernel(w, bias, _qps(sw, np.zeros(80, np.int32)))
+    q, _ = dq.run(torch.from_numpy(x).cuda(), fetch_params=False)
+    y = mm.run(q, params_dev=dq.device_params())
+    torch.cuda.synchronize()
+    q_ref, s, z = orc.dynamic_quant(x)
+    want = orc.dynamic_matmul(q_ref, w, bias, s, z, sw, np.zeros(80, np.int32))
+    assert np.array_equal(q.cpu().numpy(), q_ref)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_error_paths():
+    L = K._lib.init()
+    assert L.mi_matmul_run(None, None, 1, None, None) == K._lib.MI_NULL_PTR
+    with pytest.raises(K._lib.MiError) as e:
+        K.MatmulInt8Kernel(np.zeros((4, 8), np.int8), None, QP(0.1, 0), [QP(0.1, 0)] * 3, QP(0.1, 0))
+    assert e.value.code == K._lib.MI_PARAM_INVALID
+    with pytest.raises(TypeError):
+        K.MatmulInt8Kernel(np.zeros((4, 8), np.int8), np.zeros(4, np.float32), QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0))
