@@ -192,11 +192,12 @@ struct RequantState {
       const int64_t vmax = std::min<int64_t>((int64_t)1 << 31, (int64_t)k * 16384 + llabs((long long)h_bias2[c]) +
                                                                    (int64_t)k * 128 * llabs((long long)zwv[c]));
       const int64_t xmax = ((vmax * llabs((long long)h_mult[c])) >> 31) + 1;
-      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN ||
-          xmax + ((int64_t)1 << (e[c] - 1)) > INT32_MAX)
+      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN || vmax >= ((int64_t)1 << 31) ||
+          xmax + ((int64_t)1 << (e[c] - 1)) + (llabs((long long)zo) << e[c]) > INT32_MAX)
         fast = false;
     }
     for (int c = n; c < n_pad; ++c) e[c] = 1;
+    if (amin > amax) fast = false;
     int rc;
     if ((rc = upload(&mult, h_mult)) != MI_OK) return rc;
     if ((rc = upload(&bias2, h_bias2)) != MI_OK) return rc;
@@ -265,14 +266,23 @@ static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_
   return MI_OK;
 }
 
+// The GEMM kernels write rows with vector stores; when the caller's row length or base address does not allow that,
+// they write to a padded scratch output which is then compacted into the caller's tensor.
 static int run_requant_gemm(const RequantState &st, const int8_t *a, int64_t lda, int rows, int k16, int8_t *c,
-                            hipStream_t stream) {
+                            DevBuf *c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
+  const int8_t *w = static_cast<const int8_t *>(st.w.p);
   if (rows <= kGemvMaxRows && (int64_t)rows * k16 <= 150 * 1024)
-    return launch_gemv_requant(a, lda, rows, k16, static_cast<const int8_t *>(st.w.p), st.k_pad, st.n, rq, c, st.n,
-                               stream);
-  return launch_gemm_requant(a, lda, rows, k16, static_cast<const int8_t *>(st.w.p), st.k_pad, st.n, rq, c, st.n,
-                             stream);
+    return launch_gemv_requant(a, lda, rows, k16, w, st.k_pad, st.n, rq, c, st.n, stream);
+  if ((st.n & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 3) == 0)
+    return launch_gemm_requant(a, lda, rows, k16, w, st.k_pad, st.n, rq, c, st.n, stream);
+  const int n4 = round_up(st.n, 4);
+  int rc = c_ws->ensure((size_t)rows * n4);
+  if (rc != MI_OK) return rc;
+  RequantParams rq_pad = rq;
+  rc = launch_gemm_requant(a, lda, rows, k16, w, st.k_pad, n4, rq_pad, static_cast<int8_t *>(c_ws->p), n4, stream);
+  if (rc != MI_OK) return rc;
+  return launch_copy_rows(c_ws->p, n4, rows, st.n, c, st.n, stream);
 }
 
 }  // namespace mi
@@ -282,7 +292,7 @@ using namespace mi;
 // =====================================================================================================================
 struct mi_matmul {
   RequantState st;
-  DevBuf a_ws, h_in, h_out;
+  DevBuf a_ws, c_ws, h_in, h_out;
 };
 
 struct mi_conv {
@@ -290,7 +300,7 @@ struct mi_conv {
   bool depthwise = false, direct_1x1 = false;
   int fill = 0;
   RequantState st;
-  DevBuf w16, dw_bias, col_ws, h_in, h_out;
+  DevBuf w16, dw_bias, col_ws, c_ws, h_in, h_out;
 };
 
 struct mi_dynquant {
@@ -302,7 +312,7 @@ struct mi_dynmm {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, act = 0;
   int32_t zw0 = 0;
   bool has_bias = false;
-  DevBuf w, wscale, wsum, bias, a_ws, h_in, h_out;
+  DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out;
 };
 
 extern "C" {
@@ -402,7 +412,7 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
   int64_t lda = 0;
   int k16 = 0;
   if ((rc = prepare_rows(a_dev, rows, h->st.k, &h->a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
-  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, s);
+  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, &h->c_ws, s);
 }
 
 int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host) {
@@ -440,6 +450,7 @@ void mi_matmul_destroy(mi_matmul *h) {
   if (h == nullptr) return;
   h->st.release();
   h->a_ws.release();
+  h->c_ws.release();
   h->h_in.release();
   h->h_out.release();
   delete h;
@@ -579,7 +590,7 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
     a = static_cast<const int8_t *>(h->col_ws.p);
     lda = k16;
   }
-  return run_requant_gemm(h->st, a, lda, (int)pixels, k16, out_dev, s);
+  return run_requant_gemm(h->st, a, lda, (int)pixels, k16, out_dev, &h->c_ws, s);
 }
 
 int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_host) {
@@ -610,6 +621,7 @@ void mi_conv_destroy(mi_conv *h) {
   h->w16.release();
   h->dw_bias.release();
   h->col_ws.release();
+  h->c_ws.release();
   h->h_in.release();
   h->h_out.release();
   delete h;
@@ -757,8 +769,14 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   dq.zw0 = h->zw0;
   dq.deep = h->k;
   dq.act = h->act;
-  return launch_gemm_dequant(a, lda, rows, k16, static_cast<const int8_t *>(h->w.p), h->k_pad, h->n, dq, c_dev, h->n,
-                             s);
+  const int8_t *w = static_cast<const int8_t *>(h->w.p);
+  if ((h->n & 3) == 0 && (reinterpret_cast<uintptr_t>(c_dev) & 15) == 0)
+    return launch_gemm_dequant(a, lda, rows, k16, w, h->k_pad, h->n, dq, c_dev, h->n, s);
+  const int n4 = round_up(h->n, 4);
+  if ((rc = h->c_ws.ensure((size_t)rows * n4 * sizeof(float))) != MI_OK) return rc;
+  if ((rc = launch_gemm_dequant(a, lda, rows, k16, w, h->k_pad, n4, dq, static_cast<float *>(h->c_ws.p), n4, s)) != MI_OK)
+    return rc;
+  return launch_copy_rows(h->c_ws.p, (int64_t)n4 * 4, rows, h->n * 4, c_dev, (int64_t)h->n * 4, s);
 }
 
 int mi_dynmm_run(mi_dynmm *h, const int8_t *a_dev, int32_t rows, double in_scale, int32_t in_zp, float *c_dev,
@@ -801,6 +819,7 @@ void mi_dynmm_destroy(mi_dynmm *h) {
   h->wsum.release();
   h->bias.release();
   h->a_ws.release();
+  h->c_ws.release();
   h->h_in.release();
   h->h_out.release();
   delete h;

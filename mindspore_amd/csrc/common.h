@@ -23,9 +23,9 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 inline int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // Weight rows (output channels) and the contraction dimension are padded so that no kernel needs bounds checks on
-// the weight operand: rows to a multiple of kNPad, K to a multiple of kKPad (bytes), zero filled.
+// the weight operand: rows to a multiple of kNPad, K to a multiple of kKPad (bytes, two 128-byte GEMM steps), zero filled.
 constexpr int kNPad = 256;
-constexpr int kKPad = 128;
+constexpr int kKPad = 256;
 
 // ---- int8 requantising epilogue parameters (device arrays are padded to kNPad entries) ----
 struct RequantParams {
@@ -36,7 +36,8 @@ struct RequantParams {
   const int32_t *zw;      // weight zero point per channel (HAS_ZW only)
   int32_t zo, amin, amax;
   int has_zw;  // any weight zero point is non-zero -> input row sums are needed
-  int fast;    // host proved: all lshift == 0, 1 <= e <= 30, no mult == INT32_MIN, rounding add cannot overflow
+  int fast;    // host proved: all lshift == 0, 1 <= e <= 30, no mult == INT32_MIN, amin <= amax, and none of
+               // acc + bias2, srdhm + 2^(e-1) + (zo << e) can overflow int32
 };
 
 // ---- fp32 dequantising epilogue (dynamic-quant MatMul) ----
@@ -53,7 +54,8 @@ struct DequantParams {
 };
 
 // A: int8 activations [M][lda] (lda in bytes, multiple of 16, base 16-byte aligned, K % 16 == 0);
-// W: packed weights [n_pad][k_pad]; C: [M][ldc] elements.
+// W: packed weights [n_pad][k_pad]; C: [M][ldc] elements with n % 4 == 0, ldc % 4 == 0 and a 4-byte (int8) /
+// 16-byte (fp32) aligned base -- other output shapes go through a padded scratch buffer and launch_copy_rows.
 int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
 int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
@@ -66,6 +68,10 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t
 
 // Copies [rows][k] (row stride src_ld bytes) into a zero-padded [rows][k16] buffer, k16 = round_up(k, 16).
 int launch_pad_rows(const int8_t *src, int64_t src_ld, int rows, int k, int8_t *dst, int k16, hipStream_t stream);
+
+// dst[row][0..row_bytes) = src[row][0..row_bytes); strides in bytes.
+int launch_copy_rows(const void *src, int64_t src_ld, int rows, int row_bytes, void *dst, int64_t dst_ld,
+                     hipStream_t stream);
 
 struct ConvGeom {
   int batch, in_h, in_w, in_c, out_h, out_w, out_c;

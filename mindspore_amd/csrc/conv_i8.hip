@@ -44,6 +44,30 @@ int launch_pad_rows(const int8_t *src, int64_t src_ld, int rows, int k, int8_t *
   return MI_OK;
 }
 
+// Compacts rows: dst[row][0..row_bytes) = src[row][0..row_bytes) with different row strides (used when a GEMM wrote
+// into a padded scratch output because the caller's row length does not allow vector stores).
+__global__ __launch_bounds__(256) void copy_rows_kernel(const char *__restrict__ src, int64_t src_ld, int rows,
+                                                        int row_bytes, char *__restrict__ dst, int64_t dst_ld) {
+  const int64_t total = (int64_t)rows * row_bytes;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t row = idx / row_bytes;
+    const int col = (int)(idx - row * row_bytes);
+    dst[row * dst_ld + col] = src[row * src_ld + col];
+  }
+}
+
+int launch_copy_rows(const void *src, int64_t src_ld, int rows, int row_bytes, void *dst, int64_t dst_ld,
+                     hipStream_t stream) {
+  const int64_t total = (int64_t)rows * row_bytes;
+  const int64_t want = (total + 255) / 256;
+  const int blocks = (int)(want < 1 ? 1 : (want > 262144 ? 262144 : want));
+  hipLaunchKernelGGL(copy_rows_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<const char *>(src), src_ld, rows,
+                     row_bytes, static_cast<char *>(dst), dst_ld);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 __global__ __launch_bounds__(256) void im2col_kernel(const int8_t *__restrict__ in, ConvGeom g, int fill,
                                                      int8_t *__restrict__ dst, int k16) {
   const int kdim = g.kernel_h * g.kernel_w * g.in_c;

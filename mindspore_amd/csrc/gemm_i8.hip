@@ -5,14 +5,20 @@
 //   EPI_DEQUANT : zero-point corrections, (sx*sw) * (float)acc, + bias, activation         -> fp32
 //                 (DynamicMatmul4x16x4AIWI, .../nnacl/int8/dynamic_matmul_int8.c:99-143)
 //
-// Data movement.  Both operands are K-contiguous: activations A[M][K] and packed weights W[n_pad][k_pad].  A
-// workgroup owns a TILE_M x TILE_N output tile and walks K in steps of 128 bytes.  Each step stages
-// (TILE_M + TILE_N) rows x 128 B in LDS (double buffered); a row is eight 16-byte chunks and chunk c of row r is
-// stored at slot c ^ ((r >> 1) & 7), which makes both the 16-byte stores of the loader and the 16-byte operand
-// reads of the MFMA loop bank-conflict free.  The weight tile is the MFMA "A" operand (its rows are output
+// Both operands are K-contiguous: activations A[M][K] and packed weights W[n_pad][k_pad].  A workgroup of four
+// waves (2 x 2) owns a TILE_M x TILE_N output tile; the weight tile is the MFMA "A" operand (its rows are output
 // channels) and the activation tile the "B" operand, so a lane ends up holding 4 consecutive output channels of
-// one output row: the epilogue packs them into one 32-bit store, and the input-row sum a lane needs is the one it
-// accumulated itself from its activation fragments (v_dot4 against 0x01010101).
+// one output row: the epilogue packs them into one 32-bit store, per-channel parameters are 16-byte loads, and
+// the input-row sum a lane needs is the one it accumulated itself (v_dot4 against 0x01010101).
+//
+// Two main loops share the epilogue:
+//   direct : K % 256 == 0.  Tiles travel global -> LDS with asynchronous 16-byte-per-lane loads
+//            (global_load_lds_dwordx4), four LDS stages of 64 bytes of K, three tiles in flight, one barrier per
+//            stage; operand fragments for K sub-step s+1 are read from LDS while the MFMAs of sub-step s run.
+//   staged : any K % 16 == 0.  Tiles travel global -> registers -> LDS (the tail of K is zero-filled in
+//            registers), two LDS stages of 128 bytes of K.
+// LDS rows are XOR-swizzled in units of 16 bytes so that 8 consecutive lanes of a 16-byte access always cover
+// all 32 banks.
 #include "common.h"
 #include "quant_math.h"
 
@@ -22,61 +28,480 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int BK = 128;  // bytes of K per LDS stage
 enum { EPI_REQUANT = 0, EPI_DEQUANT = 1 };
-
-__device__ __forceinline__ int lds_slot(int row, int chunk) { return chunk ^ ((row >> 1) & 7); }
 
 struct GemmArgs {
   const int8_t *a;
   int64_t lda;
   int m;
-  int kchunks;  // valid 16-byte chunks per activation row (K / 16)
+  int k;  // bytes of K that may be read from A (multiple of 16)
   const int8_t *w;
-  int ldw;     // k_pad
-  int ktiles;  // k_pad / 128
+  int ldw;  // k_pad
   int n;
   int tiles_m, tiles_n;
   void *c;
   int64_t ldc;
 };
 
-template <int TILE_N, int TILE_M, int WAVES_N, int WAVES_M, int EPI, bool HAS_ZW, bool FAST>
-__global__ __launch_bounds__(WAVES_N *WAVES_M * 64) void gemm_i8_kernel(GemmArgs g, RequantParams rq,
-                                                                         DequantParams dq) {
-  constexpr int THREADS = WAVES_N * WAVES_M * 64;
-  constexpr int WN = TILE_N / WAVES_N, WM = TILE_M / WAVES_M;
-  constexpr int TN = WN / 32, TM = WM / 32;
+// Asynchronous 16-byte-per-lane copy global -> LDS: lane L's 16 bytes land at lds_wave_base + 16 * L;
+// lds_wave_base must be wave-uniform.  Completion is tracked by vmcnt, in issue order.
+__device__ __forceinline__ void async_copy16(const void *global_src, void *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)global_src,
+                                   (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
+
+// Hardware deals consecutive workgroup ids round-robin over the 8 XCDs (each with its own L2), so ids that share an
+// XCD are mapped to a compact block of tiles, 4 tiles tall: the CUs of one XCD then share operand panels in L2.
+__device__ __forceinline__ void tile_coords(const GemmArgs &g, int *tile_m, int *tile_n) {
+  int id = blockIdx.x;
+  const int nb = gridDim.x, per = nb >> 3;
+  if (id < per * 8) id = (id & 7) * per + (id >> 3);
+  constexpr int G = 4;
+  const int width = G * g.tiles_n;
+  const int group = id / width, first = group * G;
+  const int gsize = min(g.tiles_m - first, G);
+  *tile_m = first + (id % width) % gsize;
+  *tile_n = (id % width) / gsize;
+}
+
+// clamp to [lo, hi] in one instruction (valid for lo <= hi)
+__device__ __forceinline__ int med3_i32(int x, int lo, int hi) {
+  int y;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(y) : "v"(x), "v"(lo), "v"(hi));
+  return y;
+}
+
+__device__ __forceinline__ uint32_t pack4(int y0, int y1, int y2, int y3) {
+  // low bytes of four ints -> one dword (v_perm_b32 x3)
+  const uint32_t p01 = __builtin_amdgcn_perm((uint32_t)y1, (uint32_t)y0, 0x0c0c0400u);
+  const uint32_t p23 = __builtin_amdgcn_perm((uint32_t)y3, (uint32_t)y2, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+}
+
+// ---- epilogue.  acc[i][j][4*q + e] is output channel n_w + 32*i + 8*q + 4*h + e of output row m_w + 32*j + r.
+//      C rows are written with 4-byte (int8) / 16-byte (fp32) stores; the host guarantees n % 4 == 0, ldc % 4 == 0
+//      and an aligned base (it routes other shapes through a padded scratch output). ----
+//      Per-channel parameters are read from LDS (array p of kEpiArrays x TILE_N ints, filled by EpiParams below):
+//      global loads here would share the vmcnt counter with the output stores and serialise on them. ----
+constexpr int kEpiArrays = 5;
+
+// The workgroup's per-channel epilogue parameters: thread t holds channel n0 + t of each array (fetched at kernel
+// start, so the latency is hidden by the main loop) and drops them into LDS once the main loop is done.
+template <int TILE_N, int EPI>
+struct EpiParams {
+  int v[kEpiArrays];
+  __device__ __forceinline__ void fetch(const RequantParams &rq, const DequantParams &dq, int n0, int tid) {
+#pragma unroll
+    for (int a = 0; a < kEpiArrays; ++a) v[a] = 0;
+    if (tid < TILE_N) {
+      const int n = n0 + tid;  // arrays are padded to a multiple of 256 channels
+      if (EPI == EPI_REQUANT) {
+        v[0] = rq.mult[n];
+        v[1] = rq.bias2[n];
+        v[2] = rq.rshift[n];
+        v[3] = rq.zw[n];
+        v[4] = rq.lshift[n];
+      } else {
+        v[0] = __float_as_int(dq.wscale[n]);
+        v[1] = dq.wsum[n];
+        v[2] = dq.bias != nullptr ? __float_as_int(dq.bias[n]) : 0;
+      }
+    }
+  }
+  // call after a barrier that follows the last LDS read of the main loop; ends with a barrier
+  __device__ __forceinline__ void to_lds(int *p, int tid) const {
+    if (tid < TILE_N) {
+#pragma unroll
+      for (int a = 0; a < kEpiArrays; ++a) p[a * TILE_N + tid] = v[a];
+    }
+    __syncthreads();
+  }
+};
+
+template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST>
+__device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)[TM], const GemmArgs &g,
+                                              const RequantParams &rq, const DequantParams &dq, const int *p,
+                                              char *cstage, int n_tile, int n_w, int m_w, int r, int h) {
+  if (HAS_ZW) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) rowsum[j] += __shfl_xor(rowsum[j], 32);
+  }
+  if (EPI == EPI_REQUANT) {
+    int8_t *c = static_cast<int8_t *>(g.c);
+    const int amin_v = rq.amin, amax_v = rq.amax;
+    // A 128-channel-wide wave tile goes through LDS so that global memory sees whole 128-byte rows: written
+    // straight from the accumulator layout, every store instruction would touch 32 rows with 8 bytes each, and the
+    // L2 write path then becomes the bottleneck of the whole kernel.  Wave-private staging tile, 128 rows x 128 B:
+    // 16-byte chunk c of row R sits at slot c ^ (R & 7), and inside a chunk dword d sits at (d + (R >> 3)) & 3, which
+    // makes both the dword writes (32 rows, one column) and the 16-byte row reads bank-conflict free.
+    constexpr bool kStageC = (TN == 4 && TM == 4);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nb = n_w + i * 32 + q * 8 + h * 4;
+        if (nb >= g.n) continue;
+        const int *pl = p + (nb - n_tile);
+        const v4i mult4 = *reinterpret_cast<const v4i *>(pl);
+        const v4i bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+        const v4i e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
+        v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
+        int64_t c64[4] = {0, 0, 0, 0};
+        if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
+        if (FAST) {
+          // y = ((srdhm(v, mult) + half - (x < 0)) >> e) + zo with v = acc + bias2 folds into
+          //   x = (acc * mult + (bias2 * mult + 2^30)) >> 31 ;  y = (x + (half + (zo << e)) + (x >> 31)) >> e
+          // (exact because the host proved that none of the intermediate sums can leave int32 / int64)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            pre4[e] = ((1 << e4[e]) >> 1) + (int32_t)((uint32_t)rq.zo << e4[e]);
+            c64[e] = (int64_t)bias4[e] * (int64_t)mult4[e] + ((int64_t)1 << 30);
+          }
+        } else {
+          ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          const int m = m_w + j * 32 + r;
+          int y[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (FAST) {
+              int32_t v = acc[i][j][q * 4 + e];
+              if (HAS_ZW) v -= rowsum[j] * zw4[e];
+              const int64_t p = (int64_t)v * (int64_t)mult4[e] + c64[e];
+              const int32_t x = (int32_t)(p >> 31);
+              const int32_t t = (x + pre4[e] + (x >> 31)) >> e4[e];
+              y[e] = med3_i32(t, amin_v, amax_v);
+            } else {
+              uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
+              if (HAS_ZW) v -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
+              v += (uint32_t)bias4[e];
+              int32_t t = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
+              t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
+              t = t < rq.amax ? t : rq.amax;
+              y[e] = t > rq.amin ? t : rq.amin;
+            }
+          }
+          const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
+          if (kStageC) {
+            const int row = j * 32 + r;
+            const int slot = (2 * i + (q >> 1)) ^ (r & 7), d = (2 * q + h + (r >> 3)) & 3;
+            *reinterpret_cast<uint32_t *>(cstage + row * 128 + slot * 16 + d * 4) = packed;
+          } else if (m < g.m) {
+            *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
+          }
+        }
+      }
+    }
+    if (kStageC) {
+      const int lane = h * 32 + r;
+      const int c16 = lane & 7, lrow = lane >> 3;
+      const int n = n_w + c16 * 16;
+      const bool vec16 = ((g.ldc & 15) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const int row = lrow + 8 * t;
+        const v4i x = *reinterpret_cast<const v4i *>(cstage + row * 128 + ((c16 ^ lrow) << 4));
+        v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == t & 3
+        o[0] = x[(0 + t) & 3];
+        o[1] = x[(1 + t) & 3];
+        o[2] = x[(2 + t) & 3];
+        o[3] = x[(3 + t) & 3];
+        const int m = m_w + row;
+        if (m < g.m && n < g.n) {
+          int8_t *dst = c + (int64_t)m * g.ldc + n;
+          if (vec16 && n + 16 <= g.n) {
+            *reinterpret_cast<v4i *>(dst) = o;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
+          }
+        }
+      }
+    }
+  } else {
+    float *c = static_cast<float *>(g.c);
+    float sx = dq.sx;
+    int32_t zx = dq.zx;
+    if (dq.qp_dev != nullptr) {
+      sx = dq.qp_dev->scale_f;
+      zx = dq.qp_dev->zero_point;
+    }
+    const uint32_t kzz = (uint32_t)dq.deep * (uint32_t)zx * (uint32_t)dq.zw0;
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nb = n_w + i * 32 + q * 8 + h * 4;
+        if (nb >= g.n) continue;
+        const int *pl = p + (nb - n_tile);
+        const v4f ws4 = *reinterpret_cast<const v4f *>(pl);
+        const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+        const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
+        float ms[4];
+        uint32_t corr[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          ms[e] = __fmul_rn(sx, ws4[e]);
+          corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e];
+        }
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          const int m = m_w + j * 32 + r;
+          v4f o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            uint32_t v = (uint32_t)acc[i][j][q * 4 + e] + corr[e];
+            if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
+            float d = __fmul_rn(ms[e], (float)(int32_t)v);
+            if (dq.bias != nullptr) d = __fadd_rn(d, b4[e]);
+            if (dq.act == MI_ACT_RELU) {
+              d = (0.0f > d) ? 0.0f : d;
+            } else if (dq.act == MI_ACT_RELU6) {
+              d = (0.0f > d) ? 0.0f : d;
+              d = (6.0f < d) ? 6.0f : d;
+            }
+            o[e] = d;
+          }
+          if (m < g.m) *reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + nb) = o;
+        }
+      }
+    }
+  }
+}
+
+#ifdef MI_EXP_TIMING
+__device__ unsigned long long mi_dbg[4096 * 8];
+extern "C" int mi_dbg_read(unsigned long long *dst, int n) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi_dbg), sizeof(unsigned long long) * n);
+}
+#define MI_T(...) __VA_ARGS__
+#else
+#define MI_T(...)
+#endif
+
+template <int TN, int TM>
+struct Frag {
+  v4i w[TN], a[TM];
+};
+
+template <int TN, int TM, bool HAS_ZW>
+__device__ __forceinline__ void mma_frag(v16i (&acc)[TN][TM], int (&rowsum)[TM], const Frag<TN, TM> &f) {
+  if (HAS_ZW) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      int t = rowsum[j];
+      t = __builtin_amdgcn_sdot4(f.a[j].x, 0x01010101, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].y, 0x01010101, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].z, 0x01010101, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].w, 0x01010101, t, false);
+      rowsum[j] = t;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.a[j], acc[i][j], 0, 0, 0);
+}
+
+// Instruction-order hints for one K sub-step: spread the LDS operand reads between the MFMAs instead of issuing them
+// in one burst, so that the matrix pipe always has the next MFMA queued.
+template <int TN, int TM>
+__device__ __forceinline__ void hint_interleave_reads() {
+  // one read after each of the first MFMAs: the reads are all issued early in the sub-step, so their data has the
+  // remaining MFMAs' time to arrive before the next sub-step needs it
+  constexpr int kReads = TN + TM, kMfma = TN * TM;
+  if constexpr (kMfma >= kReads) {
+#pragma unroll
+    for (int i = 0; i < kReads; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < kMfma; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, kReads / kMfma, 0);
+    }
+  }
+}
+
+// =====================================================================================================================
+// direct main loop: 4 LDS stages x 64 bytes of K, asynchronous global -> LDS loads three tiles ahead
+// =====================================================================================================================
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
+__global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+  constexpr int BKD = 64, NST = 4;
+  constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
+  constexpr int STAGE = (TILE_N + TILE_M) * BKD;
+  constexpr int WPW = TILE_N / 16 / 4, APW = TILE_M / 16 / 4, LPW = WPW + APW;  // 1 KiB blocks per wave and tile
+  static_assert(WPW >= 1 && APW >= 1, "tile too small");
+  __shared__ __attribute__((aligned(1024))) char lds[NST * STAGE];
+
+  int tile_m, tile_n;
+  tile_coords(g, &tile_m, &tile_n);
+  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wm = wave >> 1;
+  const int r = lane & 31, h = lane >> 5;
+  const int ktiles = g.ldw / BKD;  // multiple of 4
+  EpiParams<TILE_N, EPI> epi;
+  epi.fetch(rq, dq, n0, tid);
+
+  // loader: a 1 KiB block holds 16 rows x 64 B.  Lane L fills slot (L & 3) of row (L >> 2) of its block, i.e. it
+  // fetches logical chunk (L & 3) ^ swizzle(row), swizzle(row) = (row >> 1) & 3.
+  const int drow = lane >> 2;
+  const int dchunk = (lane & 3) ^ ((lane >> 3) & 3);
+  const int8_t *wsrc = g.w + (int64_t)(n0 + wave * WPW * 16 + drow) * g.ldw + dchunk * 16;
+  const int8_t *asrc[APW];
+#pragma unroll
+  for (int i = 0; i < APW; ++i) {
+    int m = m0 + (wave * APW + i) * 16 + drow;
+    m = m < g.m ? m : g.m - 1;
+    asrc[i] = g.a + (int64_t)m * g.lda + dchunk * 16;
+  }
+  auto dma_tile = [&](int stage, int kt) {
+    char *sw = lds + stage * STAGE + wave * WPW * 1024;
+    char *sa = lds + stage * STAGE + TILE_N * BKD + wave * APW * 1024;
+#pragma unroll
+    for (int i = 0; i < WPW; ++i) async_copy16(wsrc + (int64_t)i * 16 * g.ldw + kt * BKD, sw + i * 1024);
+#pragma unroll
+    for (int i = 0; i < APW; ++i) async_copy16(asrc[i] + kt * BKD, sa + i * 1024);
+  };
+
+  v16i acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+  int rowsum[TM];
+#pragma unroll
+  for (int j = 0; j < TM; ++j) rowsum[j] = 0;
+
+  // operand fragments: this lane's rows are r + multiples of 32, so its swizzle is a lane constant
+  const int frag_swz = (r >> 1) & 3;
+  const int w_off = (wn * WN + r) * BKD, a_off = TILE_N * BKD + (wm * WM + r) * BKD;
+  Frag<TN, TM> f0, f1;
+  auto read_frag = [&](Frag<TN, TM> &f, int stage, int s) {
+    const char *base = lds + stage * STAGE + (((2 * s + h) ^ frag_swz) << 4);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) f.w[i] = *reinterpret_cast<const v4i *>(base + w_off + i * 32 * BKD);
+#pragma unroll
+    for (int j = 0; j < TM; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * BKD);
+  };
+
+  MI_T(unsigned long long t_vm = 0, t_bar = 0;)
+  // One 64-byte K step on LDS stage `st` (tile kt).  On entry f0 holds sub-step 0 of this stage.
+  //   sub-step 0 : MFMAs on f0 while f1 <- sub-step 1 of this stage
+  //   barrier    : first wait until at most LPW of this wave's loads are outstanding (loads complete in order, so
+  //                that is "tile kt+1 has landed, tile kt+2 may still be in flight"), then meet the other waves:
+  //                now tile kt+1 is complete in LDS and nobody reads stage (st+3)&3 (tile kt-1) any more
+  //   sub-step 1 : refill that stage with tile kt+3, f0 <- sub-step 0 of tile kt+1, MFMAs on f1
+  // Past the end of K the loads re-fetch the last tile into a stage nobody reads again, which keeps the
+  // outstanding-load count the same in every step.
+  auto step = [&](int kt, int st) {
+    read_frag(f1, st, 1);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
+    hint_interleave_reads<TN, TM>();
+    __builtin_amdgcn_sched_barrier(0);
+    MI_T(unsigned long long tb0 = clock64();)
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPW) : "memory");
+    MI_T(unsigned long long tb1 = clock64();)
+    asm volatile("s_barrier" ::: "memory");
+    MI_T(unsigned long long tb2 = clock64(); t_vm += tb1 - tb0; t_bar += tb2 - tb1;)
+    __builtin_amdgcn_sched_barrier(0);
+    const int nxt = kt + 3 < ktiles ? kt + 3 : ktiles - 1;
+    dma_tile((st + 3) & 3, nxt);
+    read_frag(f0, (st + 1) & 3, 0);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
+    {
+      constexpr int kMfma = TN * TM;
+      if constexpr (kMfma >= LPW) {
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < kMfma; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, LPW / kMfma, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, (TN + TM) / kMfma, 0);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  MI_T(unsigned long long t_start = clock64(), w_start = wall_clock64();)
+  dma_tile(0, 0);
+  dma_tile(1, 1);
+  dma_tile(2, 2);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LPW) : "memory");
+  read_frag(f0, 0, 0);
+  MI_T(unsigned long long t_pro = clock64();)
+  for (int kt = 0; kt < ktiles; kt += 4) {
+    step(kt, 0);
+    step(kt + 1, 1);
+    step(kt + 2, 2);
+    step(kt + 3, 3);
+  }
+  // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  MI_T(unsigned long long t_loop = clock64();)
+  epi.to_lds(reinterpret_cast<int *>(lds), tid);
+  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+                                                   lds + kEpiArrays * TILE_N * 4 + wave * 16384, n0, n0 + wn * WN,
+                                                   m0 + wm * WM, r, h);
+#ifdef MI_EXP_TIMING
+  if (tid == 0 && blockIdx.x < 4096) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned long long t_end = clock64(), w_end = wall_clock64();
+    unsigned long long *d = mi_dbg + blockIdx.x * 8;
+    d[0] = t_pro - t_start;
+    d[1] = t_loop - t_pro;
+    d[2] = t_end - t_loop;
+    d[3] = w_start;
+    d[4] = w_end;
+    d[5] = t_vm;
+    d[6] = t_bar;
+  }
+#endif
+}
+
+// =====================================================================================================================
+// staged main loop: 2 LDS stages x 128 bytes of K, global -> registers -> LDS, zero fill past K
+// =====================================================================================================================
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
+__global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+  constexpr int BK = 128, THREADS = 256;
+  constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
+  constexpr int STAGE = (TILE_N + TILE_M) * BK;
   constexpr int W_CHUNKS = TILE_N * 8 / THREADS, A_CHUNKS = TILE_M * 8 / THREADS;
   constexpr int ROWS_PER_PASS = THREADS / 8;
-  constexpr int STAGE_BYTES = (TILE_N + TILE_M) * BK;
-  static_assert(W_CHUNKS >= 1 && A_CHUNKS >= 1, "tile too small for the thread count");
+  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
 
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-
-  // ---- tile assignment: hardware deals consecutive workgroup ids round-robin over the 8 XCDs (each with its own
-  //      L2), so ids that share an XCD are mapped to a compact block of tiles, 4 tiles tall ----
-  int id = blockIdx.x;
-  {
-    const int nb = gridDim.x, per = nb >> 3;
-    if (id < per * 8) id = (id & 7) * per + (id >> 3);
-  }
   int tile_m, tile_n;
-  {
-    constexpr int G = 4;
-    const int width = G * g.tiles_n;
-    const int group = id / width, first = group * G;
-    const int gsize = min(g.tiles_m - first, G);
-    tile_m = first + (id % width) % gsize;
-    tile_n = (id % width) / gsize;
-  }
+  tile_coords(g, &tile_m, &tile_n);
   const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wn = wave % WAVES_N, wm = wave / WAVES_N;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wm = wave >> 1;
   const int r = lane & 31, h = lane >> 5;
+  const int ktiles = g.ldw / BK, kchunks = g.k >> 4;
+  EpiParams<TILE_N, EPI> epi;
+  epi.fetch(rq, dq, n0, tid);
 
-  // ---- loader: thread t moves chunk (t & 7) of rows (t >> 3) + i * ROWS_PER_PASS ----
+  // loader: thread t moves chunk (t & 7) of rows (t >> 3) + i * ROWS_PER_PASS; chunk c of row R is stored at slot
+  // c ^ (R & 7)
   const int lc = tid & 7, lrow = tid >> 3;
   v4i wreg[W_CHUNKS], areg[A_CHUNKS];
   const int8_t *wsrc = g.w + (int64_t)(n0 + lrow) * g.ldw + lc * 16;
@@ -91,7 +516,7 @@ __global__ __launch_bounds__(WAVES_N *WAVES_M * 64) void gemm_i8_kernel(GemmArgs
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i)
       wreg[i] = *reinterpret_cast<const v4i *>(wsrc + (int64_t)i * ROWS_PER_PASS * g.ldw + kt * BK);
-    const bool valid = kt * 8 + lc < g.kchunks;
+    const bool valid = kt * 8 + lc < kchunks;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       v4i z = {0, 0, 0, 0};
@@ -99,17 +524,17 @@ __global__ __launch_bounds__(WAVES_N *WAVES_M * 64) void gemm_i8_kernel(GemmArgs
     }
   };
   auto store_tile = [&](int stage) {
-    char *sw = smem + stage * STAGE_BYTES;
+    char *sw = lds + stage * STAGE;
     char *sa = sw + TILE_N * BK;
 #pragma unroll
     for (int i = 0; i < W_CHUNKS; ++i) {
       const int row = lrow + i * ROWS_PER_PASS;
-      *reinterpret_cast<v4i *>(sw + row * BK + (lds_slot(row, lc) << 4)) = wreg[i];
+      *reinterpret_cast<v4i *>(sw + row * BK + ((lc ^ (row & 7)) << 4)) = wreg[i];
     }
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int row = lrow + i * ROWS_PER_PASS;
-      *reinterpret_cast<v4i *>(sa + row * BK + (lds_slot(row, lc) << 4)) = areg[i];
+      *reinterpret_cast<v4i *>(sa + row * BK + ((lc ^ (row & 7)) << 4)) = areg[i];
     }
   };
 
@@ -124,182 +549,58 @@ __global__ __launch_bounds__(WAVES_N *WAVES_M * 64) void gemm_i8_kernel(GemmArgs
 #pragma unroll
   for (int j = 0; j < TM; ++j) rowsum[j] = 0;
 
-  const int frag_swz = (r >> 1) & 7;  // rows handled by this lane are r + multiples of 32
-  const int w_row0 = wn * WN + r, a_row0 = wm * WM + r;
+  const int frag_swz = r & 7;
+  const int w_off = (wn * WN + r) * BK, a_off = TILE_N * BK + (wm * WM + r) * BK;
+  Frag<TN, TM> f0, f1;
+  auto read_frag = [&](Frag<TN, TM> &f, int stage, int s) {
+    const char *base = lds + stage * STAGE + (((2 * s + h) ^ frag_swz) << 4);
+#pragma unroll
+    for (int i = 0; i < TN; ++i) f.w[i] = *reinterpret_cast<const v4i *>(base + w_off + i * 32 * BK);
+#pragma unroll
+    for (int j = 0; j < TM; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * BK);
+  };
 
   load_tile(0);
   store_tile(0);
   __syncthreads();
-  for (int kt = 0; kt < g.ktiles; ++kt) {
-    const bool more = kt + 1 < g.ktiles;
+  read_frag(f0, 0, 0);
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const int st = kt & 1;
+    const bool more = kt + 1 < ktiles;
     if (more) load_tile(kt + 1);
-    const char *sw = smem + (kt & 1) * STAGE_BYTES;
-    const char *sa = sw + TILE_N * BK;
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int slot = ((2 * s + h) ^ frag_swz) << 4;
-      v4i wf[TN], af[TM];
-#pragma unroll
-      for (int i = 0; i < TN; ++i) wf[i] = *reinterpret_cast<const v4i *>(sw + (w_row0 + i * 32) * BK + slot);
-#pragma unroll
-      for (int j = 0; j < TM; ++j) af[j] = *reinterpret_cast<const v4i *>(sa + (a_row0 + j * 32) * BK + slot);
-      if (HAS_ZW) {
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          int t = rowsum[j];
-          t = __builtin_amdgcn_sdot4(af[j].x, 0x01010101, t, false);
-          t = __builtin_amdgcn_sdot4(af[j].y, 0x01010101, t, false);
-          t = __builtin_amdgcn_sdot4(af[j].z, 0x01010101, t, false);
-          t = __builtin_amdgcn_sdot4(af[j].w, 0x01010101, t, false);
-          rowsum[j] = t;
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[i], af[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) store_tile((kt + 1) & 1);
+    read_frag(f1, st, 1);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
+    read_frag(f0, st, 2);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
+    read_frag(f1, st, 3);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
+    if (more) store_tile(st ^ 1);
     __syncthreads();
+    if (more) read_frag(f0, st ^ 1, 0);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
   }
 
-  // ---- epilogue.  acc[i][j][4*q + e] is output channel n0 + wn*WN + 32*i + 8*q + 4*h + e of output row
-  //      m0 + wm*WM + 32*j + r ----
-  if (HAS_ZW) {
-#pragma unroll
-    for (int j = 0; j < TM; ++j) rowsum[j] += __shfl_xor(rowsum[j], 32);
-  }
-
-  if (EPI == EPI_REQUANT) {
-    int8_t *c = static_cast<int8_t *>(g.c);
-    const bool vec_ok = ((g.n & 3) == 0) && ((g.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(c) & 3) == 0);
-#pragma unroll
-    for (int i = 0; i < TN; ++i) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int nb = n0 + wn * WN + i * 32 + q * 8 + h * 4;
-        if (nb >= g.n) continue;
-        const v4i mult4 = *reinterpret_cast<const v4i *>(rq.mult + nb);
-        const v4i bias4 = *reinterpret_cast<const v4i *>(rq.bias2 + nb);
-        const v4i e4 = *reinterpret_cast<const v4i *>(rq.rshift + nb);
-        v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, half4 = {0, 0, 0, 0};
-        if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(rq.zw + nb);
-        if (!FAST) ls4 = *reinterpret_cast<const v4i *>(rq.lshift + nb);
-        if (FAST) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) half4[e] = (1 << e4[e]) >> 1;
-        }
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          const int m = m0 + wm * WM + j * 32 + r;
-          uint32_t packed = 0;
-          int8_t bytes[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
-            if (HAS_ZW) v -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
-            v += (uint32_t)bias4[e];
-            int32_t y;
-            if (FAST) {
-              y = rdiv_pot_fast(srdhm_nosat((int32_t)v, mult4[e]), e4[e], half4[e]);
-            } else {
-              y = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
-            }
-            y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
-            y = y < rq.amax ? y : rq.amax;
-            y = y > rq.amin ? y : rq.amin;
-            bytes[e] = (int8_t)y;
-            packed |= ((uint32_t)y & 0xffu) << (8 * e);
-          }
-          if (m < g.m) {
-            int8_t *dst = c + (int64_t)m * g.ldc + nb;
-            if (vec_ok) {
-              *reinterpret_cast<uint32_t *>(dst) = packed;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (nb + e < g.n) dst[e] = bytes[e];
-            }
-          }
-        }
-      }
-    }
-  } else {
-    float *c = static_cast<float *>(g.c);
-    const bool vec_ok = ((g.n & 3) == 0) && ((g.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
-    float sx = dq.sx;
-    int32_t zx = dq.zx;
-    if (dq.qp_dev != nullptr) {
-      sx = dq.qp_dev->scale_f;
-      zx = dq.qp_dev->zero_point;
-    }
-    const uint32_t kzz = (uint32_t)dq.deep * (uint32_t)zx * (uint32_t)dq.zw0;
-#pragma unroll
-    for (int i = 0; i < TN; ++i) {
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int nb = n0 + wn * WN + i * 32 + q * 8 + h * 4;
-        if (nb >= g.n) continue;
-        const v4f ws4 = *reinterpret_cast<const v4f *>(dq.wscale + nb);
-        const v4i wsum4 = *reinterpret_cast<const v4i *>(dq.wsum + nb);
-        v4f b4 = {0.f, 0.f, 0.f, 0.f};
-        if (dq.bias != nullptr) b4 = *reinterpret_cast<const v4f *>(dq.bias + nb);
-        float ms[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) ms[e] = __fmul_rn(sx, ws4[e]);
-#pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          const int m = m0 + wm * WM + j * 32 + r;
-          v4f o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
-            if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
-            v -= (uint32_t)zx * (uint32_t)wsum4[e];
-            v += kzz;
-            float d = __fmul_rn(ms[e], (float)(int32_t)v);
-            if (dq.bias != nullptr) d = __fadd_rn(d, b4[e]);
-            if (dq.act == MI_ACT_RELU) {
-              d = (0.0f > d) ? 0.0f : d;
-            } else if (dq.act == MI_ACT_RELU6) {
-              d = (0.0f > d) ? 0.0f : d;
-              d = (6.0f < d) ? 6.0f : d;
-            }
-            o[e] = d;
-          }
-          if (m < g.m) {
-            float *dst = c + (int64_t)m * g.ldc + nb;
-            if (vec_ok) {
-              *reinterpret_cast<v4f *>(dst) = o;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (nb + e < g.n) dst[e] = o[e];
-            }
-          }
-        }
-      }
-    }
-  }
+  __syncthreads();
+  epi.to_lds(reinterpret_cast<int *>(lds), tid);
+  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+                                                   lds + kEpiArrays * TILE_N * 4 + wave * 16384, n0, n0 + wn * WN,
+                                                   m0 + wm * WM, r, h);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
-  constexpr int WAVES_N = 2, WAVES_M = 2;
-  auto kern = gemm_i8_kernel<TILE_N, TILE_M, WAVES_N, WAVES_M, EPI, HAS_ZW, FAST>;
-  constexpr int lds_bytes = 2 * (TILE_N + TILE_M) * BK;
-  static bool attr_set = false;  // benign race: idempotent
-  if (!attr_set) {
-    MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     lds_bytes));
-    attr_set = true;
-  }
   g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
   g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
   const int blocks = g.tiles_m * g.tiles_n;
-  hipLaunchKernelGGL(kern, dim3(blocks), dim3(WAVES_N * WAVES_M * 64), lds_bytes, stream, g, rq, dq);
+  // the asynchronous global->LDS loader cannot zero-fill, so it needs every 64-byte K step of A to be in bounds
+  if (g.k == g.ldw) {
+    hipLaunchKernelGGL((gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
+                       rq, dq);
+  } else {
+    hipLaunchKernelGGL((gemm_staged_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
+                       rq, dq);
+  }
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -314,14 +615,17 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
 
-static int check_args(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n, const void *c) {
+static int check_args(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n, const void *c,
+                      int64_t ldc, int c_align) {
   if (a == nullptr || w == nullptr || c == nullptr) {
     set_error("gemm: null pointer");
     return MI_NULL_PTR;
   }
   if (m <= 0 || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k || k_pad % kKPad != 0 || k_pad < k ||
-      (reinterpret_cast<uintptr_t>(a) & 15) != 0) {
-    set_error("gemm: unsupported operand geometry m=%d n=%d k=%d lda=%lld k_pad=%d", m, n, k, (long long)lda, k_pad);
+      (reinterpret_cast<uintptr_t>(a) & 15) != 0 || (n & 3) != 0 || (ldc & 3) != 0 || ldc < n ||
+      (reinterpret_cast<uintptr_t>(c) & (c_align - 1)) != 0) {
+    set_error("gemm: unsupported operand geometry m=%d n=%d k=%d lda=%lld k_pad=%d ldc=%lld", m, n, k, (long long)lda,
+              k_pad, (long long)ldc);
     return MI_PARAM_INVALID;
   }
   return MI_OK;
@@ -329,9 +633,9 @@ static int check_args(const int8_t *a, int64_t lda, int m, int k, const int8_t *
 
 int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
-  int rc = check_args(a, lda, m, k, w, k_pad, n, c);
+  int rc = check_args(a, lda, m, k, w, k_pad, n, c, ldc, 4);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k / 16, w, k_pad, k_pad / BK, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w, k_pad, n, 0, 0, c, ldc};
   DequantParams dq{};
   if (rq.has_zw) {
     return rq.fast ? launch_pick_tile<EPI_REQUANT, true, true>(g, rq, dq, stream)
@@ -343,9 +647,9 @@ int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t
 
 int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream) {
-  int rc = check_args(a, lda, m, k, w, k_pad, n, c);
+  int rc = check_args(a, lda, m, k, w, k_pad, n, c, ldc, 16);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k / 16, w, k_pad, k_pad / BK, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w, k_pad, n, 0, 0, c, ldc};
   RequantParams rq{};
   return dq.zw0 != 0 ? launch_pick_tile<EPI_DEQUANT, true, false>(g, rq, dq, stream)
                      : launch_pick_tile<EPI_DEQUANT, false, false>(g, rq, dq, stream);

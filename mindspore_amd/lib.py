@@ -6,7 +6,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmi355x_int8.so")
+LIB_PATH = os.environ.get("MI355X_INT8_LIB", os.path.join(HERE, "libmi355x_int8.so"))
 
 MI_OK, MI_ERROR, MI_NULL_PTR, MI_PARAM_INVALID, MI_MEMORY_FAILED, MI_NOT_SUPPORT = 0, -1, -2, -3, -6, -7
 ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
