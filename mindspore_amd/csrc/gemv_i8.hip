@@ -2,21 +2,29 @@
 // against an [n_pad][k_pad] int8 weight matrix.  The kernel is HBM-bound on the weight stream, so the design goal
 // is "every weight byte crosses HBM once, in 1 KiB coalesced wave loads, with enough loads in flight":
 //   - a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes);
-//   - it keeps two groups of U segments x R rows of 16-byte loads in flight (software prefetch);
+//   - it keeps D 16-byte loads per lane (D KiB per wave) in flight at all times, refilling a register slot as soon
+//     as its chunk has been consumed;
 //   - the M activation rows are staged once per workgroup in LDS and re-read as 16-byte fragments;
 //   - products use v_dot4_i32_i8; the K reduction across lanes happens once at the end.
 // Arithmetic reference: MatmulInt8Opt, mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/matmul_int8.c:296-331.
 #include "common.h"
 #include "quant_math.h"
 
+#include <type_traits>
+
 namespace mi {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 
+// Sum over the 64 lanes of a wave, returned as a wave-uniform value: DPP adds inside each row of 16 lanes
+// (quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_ror:4, row_ror:8), then one lane per row is read back.
 __device__ __forceinline__ int wave_sum(int v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
-  return v;
+  v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xF, 0xF, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xF, 0xF, false);
+  return __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+         __builtin_amdgcn_readlane(v, 48);
 }
 
 __device__ __forceinline__ int dot16(v4i w, v4i a, int acc) {
@@ -38,35 +46,51 @@ struct GemvArgs {
   int64_t ldc;
 };
 
-template <int M, int R, int U>
+// One wave owns R consecutive output channels and walks its R x K weight bytes as a stream of 1 KiB chunks
+// (chunk c = K segment c / R of row c % R, so one activation fragment serves R consecutive chunks).  D chunks are
+// in flight: a register slot is refilled with the chunk D positions ahead as soon as it has been consumed.  When
+// R * ceil(K / 1 KiB) <= D the whole share of the wave is requested up front and nothing loops.
+// No weight load is predicated (a predicated load makes the compiler wait for earlier loads before issuing later
+// ones): lanes past the end of a row re-read its last 16 bytes and chunks past the end of the stream re-read the
+// last chunk; both meet a zero activation fragment or are not accumulated.
+template <int M, int R, int D>
 __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
+  static_assert(D % R == 0, "the slot -> row mapping must be static");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  v4i *sa = reinterpret_cast<v4i *>(smem);  // [M][kchunks]
+  v4i *sa = reinterpret_cast<v4i *>(smem);  // [M][nseg * 64], zero past K
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n_base = (blockIdx.x * 4 + wave) * R;
   const int nseg = (g.kchunks + 63) >> 6;
-  const int ngroups = (nseg + U - 1) / U;
+  const int kc_pad = nseg * 64;
+  const int total = nseg * R;
+  const int last_off = (g.kchunks - 1) * 16;
   const int8_t *wrow = g.w + (int64_t)n_base * g.ldw;
 
-  v4i wcur[U][R], wnext[U][R];
-  auto load_group = [&](v4i(&dst)[U][R], int grp) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int chunk = (grp * U + u) * 64 + lane;
-      const bool valid = chunk < g.kchunks;
-#pragma unroll
-      for (int rr = 0; rr < R; ++rr) {
-        v4i z = {0, 0, 0, 0};
-        dst[u][rr] = valid ? *reinterpret_cast<const v4i *>(wrow + (int64_t)rr * g.ldw + (int64_t)chunk * 16) : z;
-      }
-    }
+  auto load_chunk = [&](int c) -> v4i {
+    c = c < total ? c : total - 1;
+    const int seg = c / R, rr = c % R;
+    int off = seg * 1024 + lane * 16;
+    off = off < last_off ? off : last_off;
+    return *reinterpret_cast<const v4i *>(wrow + (int64_t)rr * g.ldw + off);
   };
-  load_group(wcur, 0);
+  v4i buf[D];
+#pragma unroll
+  for (int i = 0; i < D; ++i) buf[i] = load_chunk(i);
+  // lane rr*M + m finishes output (m, n_base + rr): fetch its channel's parameters now, so their latency hides
+  // behind the weight stream (the parameter arrays are padded to a multiple of 256 channels)
+  const int my_rr = lane / M, my_m = lane - my_rr * M;
+  const int my_n = n_base + (lane < R * M ? my_rr : 0);
+  const int32_t p_mult = rq.mult[my_n], p_e = rq.rshift[my_n], p_ls = rq.lshift[my_n], p_bias2 = rq.bias2[my_n];
+  const int32_t p_zw = rq.zw[my_n];
 
-  // stage the activations
-  for (int idx = tid; idx < M * g.kchunks; idx += 256) {
-    const int m = idx / g.kchunks, ch = idx - m * g.kchunks;
-    sa[idx] = *reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda + (int64_t)ch * 16);
+  // stage the activations (the weight loads above are already in flight)
+#pragma unroll
+  for (int m = 0; m < M; ++m) {
+    const v4i *arow = reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda);
+    for (int ch = tid; ch < kc_pad; ch += 256) {
+      v4i z = {0, 0, 0, 0};
+      sa[m * kc_pad + ch] = ch < g.kchunks ? arow[ch] : z;
+    }
   }
   __syncthreads();
 
@@ -79,31 +103,35 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
 #pragma unroll
   for (int m = 0; m < M; ++m) asum[m] = 0;
 
-  for (int grp = 0; grp < ngroups; ++grp) {
-    if (grp + 1 < ngroups) load_group(wnext, grp + 1);
+  v4i af[M];
+  auto pass = [&](int base, auto refill) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int chunk = (grp * U + u) * 64 + lane;
-      if (chunk < g.kchunks) {
+    for (int i = 0; i < D; ++i) {
+      const int c = base + i;
+      const v4i w = buf[i];
+      if (decltype(refill)::value) buf[i] = load_chunk(c + D);
+      if (i % R == 0) {  // first row of a K segment: fetch the activation fragments for it (zero past the stream)
+        if (M > 2) __builtin_amdgcn_sched_barrier(0);  // keeps the fragments of later segments out of registers
+        const int seg = c / R;
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-          const v4i af = sa[m * g.kchunks + chunk];
+          v4i z = {0, 0, 0, 0};
+          af[m] = seg < nseg ? sa[m * kc_pad + seg * 64 + lane] : z;
           if (rq.has_zw) {
             v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-            asum[m] = dot16(af, ones, asum[m]);
+            asum[m] = dot16(af[m], ones, asum[m]);
           }
-#pragma unroll
-          for (int rr = 0; rr < R; ++rr) acc[rr][m] = dot16(wcur[u][rr], af, acc[rr][m]);
         }
       }
+#pragma unroll
+      for (int m = 0; m < M; ++m) acc[i % R][m] = dot16(w, af[m], acc[i % R][m]);
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
-#pragma unroll
-      for (int rr = 0; rr < R; ++rr) wcur[u][rr] = wnext[u][rr];
-  }
+  };
+  int base = 0;
+  for (; base + D < total; base += D) pass(base, std::true_type());
+  pass(base, std::false_type());
 
-  // reduce over lanes; afterwards every lane holds every total and lane rr*M + m finishes output (m, n_base + rr)
+  // reduce over lanes (wave-uniform totals); lane rr*M + m keeps the one it finishes
   int mine = 0, my_asum = 0;
 #pragma unroll
   for (int m = 0; m < M; ++m) {
@@ -119,18 +147,17 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
     }
   }
   if (lane < R * M) {
-    const int rr = lane / M, m = lane - rr * M;
-    const int n = n_base + rr;
+    const int m = my_m, n = my_n;
     if (n < g.n) {
       uint32_t v = (uint32_t)mine;
-      if (rq.has_zw) v -= (uint32_t)my_asum * (uint32_t)rq.zw[n];
-      v += (uint32_t)rq.bias2[n];
-      const int32_t mult = rq.mult[n], e = rq.rshift[n];
+      if (rq.has_zw) v -= (uint32_t)my_asum * (uint32_t)p_zw;
+      v += (uint32_t)p_bias2;
+      const int32_t mult = p_mult, e = p_e;
       int32_t y;
       if (rq.fast) {
         y = rdiv_pot_fast(srdhm_nosat((int32_t)v, mult), e, (1 << e) >> 1);
       } else {
-        y = rdiv_pot(srdhm((int32_t)(v << rq.lshift[n]), mult), e);
+        y = rdiv_pot(srdhm((int32_t)(v << p_ls), mult), e);
       }
       y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
       y = y < rq.amax ? y : rq.amax;
@@ -140,11 +167,10 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
   }
 }
 
-template <int M, int R>
-static int launch_mr(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  constexpr int U = 2;
-  auto kern = gemv_i8_kernel<M, R, U>;
-  const int lds_bytes = M * g.kchunks * 16;
+template <int M, int R, int D>
+static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
+  auto kern = gemv_i8_kernel<M, R, D>;
+  const int lds_bytes = M * ((g.kchunks + 63) / 64) * 1024;
   if (lds_bytes > 64 * 1024) {
     static bool attr_set = false;
     if (!attr_set) {
@@ -162,9 +188,18 @@ static int launch_mr(const GemvArgs &g, const RequantParams &rq, hipStream_t str
 
 template <int M>
 static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  // fewer rows per wave when there are few output channels, so that every CU still gets several waves
-  if (g.n <= 8192) return launch_mr<M, 2>(g, rq, stream);
-  return launch_mr<M, 4>(g, rq, stream);
+  // Measured on MI355X: HBM streams fastest with many light waves that each have their whole share in flight at
+  // once (a wave that loops needs >= 8-16 resident waves per CU to keep up).  So pick the rows per wave so that a
+  // wave's R x ceil(K / 1 KiB) chunks fit the in-flight budget, and fall back to looping for very long rows.
+  const int nseg = (g.kchunks + 63) >> 6;
+  if (M >= 3) {  // register pressure grows with M: shorter queues, more rows per wave where there are many rows
+    if (g.n >= 8192 || nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
+    return launch_mrd<M, 2, 8>(g, rq, stream);
+  }
+  if (nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
+  if (nseg == 2) return launch_mrd<M, 4, 8>(g, rq, stream);
+  if (nseg <= 4 || M == 2) return launch_mrd<M, 2, 8>(g, rq, stream);
+  return launch_mrd<M, 1, 12>(g, rq, stream);
 }
 
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
@@ -175,7 +210,7 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t
   }
   if (m < 1 || m > kGemvMaxRows || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
       k_pad % kKPad != 0 || k_pad < k || (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
-      (int64_t)m * k > 160 * 1024 - 1024) {
+      (int64_t)m * round_up(k, 1024) > 160 * 1024 - 1024) {
     set_error("gemv: unsupported operand geometry m=%d n=%d k=%d lda=%lld", m, n, k, (long long)lda);
     return MI_PARAM_INVALID;
   }

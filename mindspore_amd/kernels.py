@@ -90,14 +90,20 @@ class MatmulInt8Kernel(_Handle):
         _lib.check(L.mi_matmul_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                       C.byref(self._h)), "mi_matmul_create")
 
-    def run(self, a):
+    def run(self, a, out=None):
+        """a: int8 [..., K] as a numpy array (host path) or a contiguous CUDA tensor (device path, current stream).
+        `out` (device path only) is a preallocated contiguous CUDA int8 tensor [..., N] to write into."""
         L = _lib.load()
         if _is_torch(a):
             import torch
             if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.shape[-1] != self.k:
                 raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % self.k)
             rows = a.numel() // self.k
-            out = torch.empty(a.shape[:-1] + (self.n,), dtype=torch.int8, device=a.device)
+            if out is None:
+                out = torch.empty(a.shape[:-1] + (self.n,), dtype=torch.int8, device=a.device)
+            elif (out.dtype != torch.int8 or not out.is_cuda or not out.is_contiguous()
+                  or out.numel() != rows * self.n):
+                raise ValueError("out must be a contiguous CUDA int8 tensor with %d elements" % (rows * self.n))
             _lib.check(L.mi_matmul_run(self._h, a.data_ptr(), rows, out.data_ptr(), _stream()), "mi_matmul_run")
             return out
         a = _host_i8(a)
