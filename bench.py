@@ -8,6 +8,7 @@ requantising epilogue); the decode GEMV (configuration 4, batch 1), DynamicQuant
 timed region.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm4096|gemm8192] [--no-cpu] [--no-extra]
+                    [--calibrate]
 """
 import argparse
 import json
@@ -21,9 +22,10 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA peak, TOP/s (5.0 POP/s)
 PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E peak, GB/s
 
-# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of this
-# script (summaries under profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {"gemm4096": None, "gemm8192": None}
+# HBM-side bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
+# this script, each scaled by what the same counter reads for the 256 MiB copy of --calibrate (FETCH_SIZE x 2.000,
+# WRITE_SIZE x 1.000; summary in profiles/gemm_direct_kernel_gemm4096.txt): (99515 + 16640) KiB.  None = not measured.
+MEASURED_TRAFFIC_BYTES = {"gemm4096": (99515 + 16640) * 1024, "gemm8192": None}
 
 
 def time_steps(fn, steps, warmup):
@@ -60,32 +62,49 @@ def bench_gemm(size, steps, warmup):
     return dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c)
 
 
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def bench_hbm_read(steps, warmup):
+    """What a kernel that only reads can reach on this device: the library's plain read stream over 48 MiB slices
+    (the size of one decode weight matrix) of a 3 GiB buffer, so no slice is still in the 256 MB Infinity Cache when
+    it is read again."""
+    import torch
+    from mindspore_amd import lib
+    L = lib.load()
+    slice_bytes, n_slices = 48 << 20, 64
+    buf = torch.ones(slice_bytes * n_slices, dtype=torch.int8, device="cuda")
+    state = {"i": 0}
+    def step():
+        i = state["i"] = (state["i"] + 1) % n_slices
+        lib.check(L.mi_diag_stream_read(buf.data_ptr() + i * slice_bytes, slice_bytes, _stream()), "mi_diag_stream_read")
+    ms, _ = time_steps(step, max(steps, 40), warmup)
+    del buf
+    return dict(bytes=slice_bytes, ms=ms, gbps=slice_bytes / (ms * 1e-3) / 1e9)
+
+
 def bench_gemv(steps, warmup, m=1):
-    """Decode step: the five 7B-class layer matrices, two layers' worth of distinct weights (404 MB) cycled so the
-    256 MB Infinity Cache cannot hold the working set."""
+    """Decode step: the five 7B-class layer matrices, three layers' worth of distinct weights (606 MB) cycled so the
+    256 MB Infinity Cache cannot hold the working set.  Outputs are preallocated; one step = 15 launches."""
     import torch
     from mindspore_amd import workloads as wl
-    kerns, acts, total_bytes = [], [], 0
-    for layer in range(2):
+    kerns, acts, outs, total_bytes = [], [], [], 0
+    for layer in range(3):
         for name, n, k in wl.DECODE_SHAPES:
             c = wl.gemv_c4(name, n, k, m, seed=layer)
             kerns.append(make_matmul(c))
             acts.append(torch.from_numpy(c["a"]).cuda())
+            outs.append(torch.empty((m, n), dtype=torch.int8, device="cuda"))
             total_bytes += n * k + m * k + m * n + 16 * n
     def step():
-        for kern, a in zip(kerns, acts):
-            kern.run(a)
+        for kern, a, o in zip(kerns, acts, outs):
+            kern.run(a, out=o)
     ev_ms, _ = time_steps(step, steps, warmup)
-    per_shape = {}
-    for i, (name, n, k) in enumerate(wl.DECODE_SHAPES):
-        if name in per_shape:
-            continue
-        kern, a = kerns[i], acts[i]
-        ms, _ = time_steps(lambda: kern.run(a), max(steps, 20), 3)
-        per_shape[name] = dict(n=n, k=k, ms_warm=ms, gbps_warm=(n * k + m * k + m * n + 16 * n) / (ms * 1e-3) / 1e9)
     gbps = total_bytes / (ev_ms * 1e-3) / 1e9
-    return dict(m=m, ms_per_decode_step_2_layers=ev_ms, bytes=total_bytes, gbps=gbps, frac_of_hbm_peak=gbps / PEAK_HBM_GBPS,
-                cache_warm_single_matrix=per_shape)
+    return dict(m=m, launches_per_step=len(kerns), ms_per_step=ev_ms, us_per_launch=ev_ms * 1e3 / len(kerns),
+                bytes_per_step=total_bytes, gbps=gbps, frac_of_hbm_peak=gbps / PEAK_HBM_GBPS)
 
 
 def bench_bert(steps, warmup):
@@ -146,6 +165,9 @@ def main():
     ap.add_argument("--workload", default="gemm4096", choices=["gemm4096", "gemm8192"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch the library's 256 MiB device copy three times (known traffic, for scaling "
+                         "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this hot path is a single-GPU path; only --gpus 1 is supported (got %d)" % args.gpus,
@@ -165,7 +187,9 @@ def main():
         other = 8192 if size == 4096 else 4096
         o = bench_gemm(other, max(3, args.steps // 5), 2)
         extra["gemm%d" % other] = dict(ms=o["ms"], tops=o["tops"], frac_of_int8_peak=o["tops"] / PEAK_INT8_TOPS)
+        extra["hbm_read_stream"] = bench_hbm_read(args.steps, 3)
         extra["gemv_decode_m1"] = bench_gemv(max(5, args.steps // 2), 3, 1)
+        extra["gemv_decode_m1"]["frac_of_read_stream"] = extra["gemv_decode_m1"]["gbps"] / extra["hbm_read_stream"]["gbps"]
         extra["gemv_decode_m8"] = bench_gemv(max(5, args.steps // 2), 3, 8)
         extra.update(bench_bert(max(5, args.steps // 2), 3))
     result = {
@@ -177,8 +201,15 @@ def main():
                                "int32 bias" % size},
         "roofline": {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
-                     "kernel": "gemm_i8_kernel<256,256,2,2,requant>", "ops_per_launch": g["ops"]},
+                     "kernel": "mi::gemm_direct_kernel<256, 256, 0, false, true>", "ops_per_launch": g["ops"]},
     }
+    if args.calibrate:
+        L = lib.load()
+        src = torch.ones(256 << 20, dtype=torch.int8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            lib.check(L.mi_diag_copy(dst.data_ptr(), src.data_ptr(), 256 << 20, _stream()), "mi_diag_copy")
+        torch.cuda.synchronize()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(g["case"], size)
     if extra:

@@ -193,6 +193,13 @@ int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in
                       float *c_host);
 void mi_dynmm_destroy(mi_dynmm *h);
 
+/* ---- measurement aids (no counterpart in the reference) ---------------------------------------------------------
+ * Two plain HBM movers with a known byte count, used by the benchmark: the read stream gives the bandwidth a
+ * kernel that only reads (the decode GEMV) can reach on this device, the copy calibrates the profiler's
+ * FETCH_SIZE / WRITE_SIZE counters.  bytes must be a multiple of 16, pointers 16-byte aligned. */
+int mi_diag_stream_read(const void *src_dev, int64_t bytes, void *stream);
+int mi_diag_copy(void *dst_dev, const void *src_dev, int64_t bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

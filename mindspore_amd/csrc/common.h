@@ -83,6 +83,10 @@ int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, in
 int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
                    const RequantParams &rq, int8_t *out, hipStream_t stream);
 
+// Measurement aids: read `bytes` and discard them / copy them, 16 bytes per lane.
+int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream);
+int launch_copy16(void *dst, const void *src, int64_t bytes, hipStream_t stream);
+
 // DynamicQuant: per-block min/max partials, then quantise (every block re-reduces the partials).
 constexpr int kDqMaxBlocks = 1024;
 int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, mi_dq_params *params, int8_t *q,

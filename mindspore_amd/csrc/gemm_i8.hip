@@ -272,16 +272,6 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
   }
 }
 
-#ifdef MI_EXP_TIMING
-__device__ unsigned long long mi_dbg[4096 * 8];
-extern "C" int mi_dbg_read(unsigned long long *dst, int n) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi_dbg), sizeof(unsigned long long) * n);
-}
-#define MI_T(...) __VA_ARGS__
-#else
-#define MI_T(...)
-#endif
-
 template <int TN, int TM>
 struct Frag {
   v4i w[TN], a[TM];
@@ -394,8 +384,6 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
 #pragma unroll
     for (int j = 0; j < TM; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * BKD);
   };
-
-  MI_T(unsigned long long t_vm = 0, t_bar = 0;)
   // One 64-byte K step on LDS stage `st` (tile kt).  On entry f0 holds sub-step 0 of this stage.
   //   sub-step 0 : MFMAs on f0 while f1 <- sub-step 1 of this stage
   //   barrier    : first wait until at most LPW of this wave's loads are outstanding (loads complete in order, so
@@ -409,11 +397,8 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
     hint_interleave_reads<TN, TM>();
     __builtin_amdgcn_sched_barrier(0);
-    MI_T(unsigned long long tb0 = clock64();)
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPW) : "memory");
-    MI_T(unsigned long long tb1 = clock64();)
     asm volatile("s_barrier" ::: "memory");
-    MI_T(unsigned long long tb2 = clock64(); t_vm += tb1 - tb0; t_bar += tb2 - tb1;)
     __builtin_amdgcn_sched_barrier(0);
     const int nxt = kt + 3 < ktiles ? kt + 3 : ktiles - 1;
     dma_tile((st + 3) & 3, nxt);
@@ -439,14 +424,11 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-
-  MI_T(unsigned long long t_start = clock64(), w_start = wall_clock64();)
   dma_tile(0, 0);
   dma_tile(1, 1);
   dma_tile(2, 2);
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LPW) : "memory");
   read_frag(f0, 0, 0);
-  MI_T(unsigned long long t_pro = clock64();)
   for (int kt = 0; kt < ktiles; kt += 4) {
     step(kt, 0);
     step(kt + 1, 1);
@@ -456,25 +438,10 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
   // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  MI_T(unsigned long long t_loop = clock64();)
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
                                                    lds + kEpiArrays * TILE_N * 4 + wave * 16384, n0, n0 + wn * WN,
                                                    m0 + wm * WM, r, h);
-#ifdef MI_EXP_TIMING
-  if (tid == 0 && blockIdx.x < 4096) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    unsigned long long t_end = clock64(), w_end = wall_clock64();
-    unsigned long long *d = mi_dbg + blockIdx.x * 8;
-    d[0] = t_pro - t_start;
-    d[1] = t_loop - t_pro;
-    d[2] = t_end - t_loop;
-    d[3] = w_start;
-    d[4] = w_end;
-    d[5] = t_vm;
-    d[6] = t_bar;
-  }
-#endif
 }
 
 // =====================================================================================================================
