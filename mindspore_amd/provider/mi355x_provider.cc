@@ -1,0 +1,304 @@
+// MindSpore Lite custom-provider kernels backed by libmi355x_int8.so.
+//
+// This translation unit is the reference-side half of the drop-in boundary: it subclasses mindspore::kernel::Kernel
+// (include/api/kernel.h:29-55) and registers creators through registry::RegisterKernel
+// (mindspore/lite/include/registry/register_kernel.h:57-74) for MatMulFusion, FullConnection, Conv2DFusion (int8) and
+// DynamicQuant (float32).  Everything below the Kernel objects is the C ABI of include/mi355x_int8.h.
+//
+// It needs a MindSpore Lite SDK to compile (register_kernel.h includes the flatc-generated schema/model_generated.h)
+// and is therefore not part of the library build:
+//   g++ -std=c++17 -fPIC -shared mi355x_provider.cc -I<lite-sdk>/runtime -I<repo>/include \
+//       -L<lite-sdk>/runtime/lib -lmindspore-lite -L<repo>/mindspore_amd -lmi355x_int8 -o libmi355x_provider.so
+// An application selects it with CPUDeviceInfo::SetProvider("mi355x") (+ SetProviderDevice("CPU")); the stock
+// benchmark tool with --provider=mi355x (it leaves the provider device empty, hence the second registration under "").
+//
+// Tensors are host-resident (arch "CPU": the kernels live in the ordinary CPU subgraph), so Execute() uses the
+// *_run_host entry points, which stage through pinned buffers.  A creator returns nullptr for everything the library
+// does not reproduce bit-exactly; the scheduler then falls back to the builtin CPU kernel
+// (mindspore/lite/src/litert/scheduler.cc:1173-1177).
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "include/api/kernel.h"
+#include "include/api/status.h"
+#include "include/api/types.h"
+#include "include/registry/register_kernel.h"
+#include "mi355x_int8.h"
+#include "schema/model_generated.h"
+
+namespace mindspore {
+namespace mi355x {
+namespace {
+constexpr int kWeightIndex = 1;
+constexpr int kBiasIndex = 2;
+
+bool LibraryReady() {
+  static const bool ok = (mi_init(0) == MI_OK);
+  return ok;
+}
+
+// Per-tensor activation quantisation is all the builtin kernels accept too (convolution_base.cc:334-342,368-375).
+bool PerTensor(const MSTensor &t) { return t.QuantParams().size() == 1; }
+
+void FilterQuant(const MSTensor &w, std::vector<double> *scales, std::vector<int32_t> *zps) {
+  for (const auto &q : w.QuantParams()) {
+    scales->push_back(q.scale);
+    zps->push_back(q.zero_point);
+  }
+}
+
+int ToStatus(int mi_code) { return mi_code == MI_OK ? static_cast<int>(kSuccess) : static_cast<int>(kLiteError); }
+
+int64_t RowsOf(const MSTensor &t) {
+  const auto shape = t.Shape();
+  int64_t rows = 1;
+  for (size_t i = 0; i + 1 < shape.size(); ++i) rows *= shape[i];
+  return rows;
+}
+}  // namespace
+
+// ---- MatMulFusion / FullConnection, int8 in -> int8 out (full quant) or fp32 out (dynamic quant) ----------------
+class MatmulKernel : public kernel::Kernel {
+ public:
+  MatmulKernel(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out, const schema::Primitive *prim,
+               const Context *ctx, bool b_transpose, int act)
+      : Kernel(in, out, prim, ctx), b_transpose_(b_transpose), act_(act) {}
+  ~MatmulKernel() override {
+    mi_matmul_destroy(full_);
+    mi_dynmm_destroy(dyn_);
+  }
+
+  int Prepare() override {
+    const MSTensor &w = inputs_[kWeightIndex];
+    const auto wshape = w.Shape();
+    if (wshape.size() != 2 || w.Data() == nullptr) return kLiteError;
+    const int32_t n = static_cast<int32_t>(b_transpose_ ? wshape[0] : wshape[1]);
+    const int32_t k = static_cast<int32_t>(b_transpose_ ? wshape[1] : wshape[0]);
+    std::vector<double> scales;
+    std::vector<int32_t> zps;
+    FilterQuant(w, &scales, &zps);
+    const void *bias = inputs_.size() > kBiasIndex ? inputs_[kBiasIndex].Data().get() : nullptr;
+    if (outputs_[0].DataType() == DataType::kNumberTypeInt8) {
+      const auto iq = inputs_[0].QuantParams().front();
+      const auto oq = outputs_[0].QuantParams().front();
+      mi_matmul_desc d{k, n, b_transpose_ ? 1 : 0, act_, iq.scale, iq.zero_point, oq.scale, oq.zero_point,
+                       static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
+      return ToStatus(mi_matmul_create(&d, static_cast<const int8_t *>(w.Data().get()),
+                                       static_cast<const int32_t *>(bias), &full_));
+    }
+    mi_dynmm_desc d{k, n, b_transpose_ ? 1 : 0, act_, static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
+    return ToStatus(
+      mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_));
+  }
+
+  int ReSize() override { return kSuccess; }  // the row count is read from the input tensor at every Execute
+
+  int Execute() override {
+    const auto *a = static_cast<const int8_t *>(inputs_[0].Data().get());
+    void *c = outputs_[0].MutableData();
+    if (a == nullptr || c == nullptr) return kLiteNullptr;
+    const int32_t rows = static_cast<int32_t>(RowsOf(inputs_[0]));
+    if (full_ != nullptr) return ToStatus(mi_matmul_run_host(full_, a, rows, static_cast<int8_t *>(c)));
+    // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
+    // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
+    const auto iq = inputs_[0].QuantParams().front();
+    return ToStatus(mi_dynmm_run_host(dyn_, a, rows, iq.scale, iq.zero_point, static_cast<float *>(c)));
+  }
+
+ private:
+  bool b_transpose_;
+  int act_;
+  mi_matmul *full_ = nullptr;
+  mi_dynmm *dyn_ = nullptr;
+};
+
+std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
+                                              const schema::Primitive *prim, const Context *ctx) {
+  if (!LibraryReady() || in.size() < 2 || out.size() != 1 || prim == nullptr) return nullptr;
+  bool b_transpose = true;
+  int act = 0;
+  if (const auto *fc = prim->value_as_FullConnection()) {  // weight is always [N, K] (fullconnection_int8.cc:33-34)
+    if (fc->use_axis()) return nullptr;
+    act = fc->activation_type();
+  } else if (const auto *mm = prim->value_as_MatMulFusion()) {
+    if (mm->transpose_a()) return nullptr;
+    b_transpose = mm->transpose_b();
+    act = mm->activation_type();
+  } else {
+    return nullptr;
+  }
+  const MSTensor &w = in[kWeightIndex];
+  const bool out_i8 = out[0].DataType() == DataType::kNumberTypeInt8;
+  const bool out_f32 = out[0].DataType() == DataType::kNumberTypeFloat32;
+  if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || w.Shape().size() != 2) return nullptr;
+  if (!(out_i8 || out_f32) || !PerTensor(in[0]) || (out_i8 && !PerTensor(out[0]))) return nullptr;
+  if (act != MI_ACT_NONE && act != MI_ACT_RELU && act != MI_ACT_RELU6) return nullptr;
+  if (in.size() > kBiasIndex) {
+    const auto want = out_i8 ? DataType::kNumberTypeInt32 : DataType::kNumberTypeFloat32;
+    if (!in[kBiasIndex].IsConst() || in[kBiasIndex].DataType() != want) return nullptr;
+  }
+  return std::make_shared<MatmulKernel>(in, out, prim, ctx, b_transpose, act);
+}
+
+// ---- Conv2DFusion int8 -------------------------------------------------------------------------------------------
+class ConvKernel : public kernel::Kernel {
+ public:
+  using Kernel::Kernel;
+  ~ConvKernel() override { mi_conv_destroy(conv_); }
+
+  int Prepare() override {
+    const auto *cv = primitive_->value_as_Conv2DFusion();
+    const MSTensor &w = inputs_[kWeightIndex];
+    const auto in_shape = inputs_[0].Shape();  // NHWC
+    mi_conv_desc d{};
+    d.in_channel = static_cast<int32_t>(cv->in_channel());
+    d.out_channel = static_cast<int32_t>(cv->out_channel());
+    d.kernel_h = static_cast<int32_t>(cv->kernel_size()->Get(0));
+    d.kernel_w = static_cast<int32_t>(cv->kernel_size()->Get(1));
+    d.stride_h = static_cast<int32_t>(cv->stride()->Get(0));
+    d.stride_w = static_cast<int32_t>(cv->stride()->Get(1));
+    d.dilation_h = static_cast<int32_t>(cv->dilation()->Get(0));
+    d.dilation_w = static_cast<int32_t>(cv->dilation()->Get(1));
+    d.group = static_cast<int32_t>(cv->group());
+    d.act_type = cv->activation_type();
+    if (cv->pad_mode() == schema::PadMode_SAME) {  // the builtin kernel gets these from shape inference
+      int32_t oh = 0, ow = 0;
+      mi_conv_same_pad(static_cast<int32_t>(in_shape[1]), d.kernel_h, d.stride_h, d.dilation_h, &d.pad_u, &d.pad_d,
+                       &oh);
+      mi_conv_same_pad(static_cast<int32_t>(in_shape[2]), d.kernel_w, d.stride_w, d.dilation_w, &d.pad_l, &d.pad_r,
+                       &ow);
+    } else if (cv->pad_mode() == schema::PadMode_PAD && cv->pad_list() != nullptr && cv->pad_list()->size() == 4) {
+      d.pad_u = static_cast<int32_t>(cv->pad_list()->Get(0));
+      d.pad_d = static_cast<int32_t>(cv->pad_list()->Get(1));
+      d.pad_l = static_cast<int32_t>(cv->pad_list()->Get(2));
+      d.pad_r = static_cast<int32_t>(cv->pad_list()->Get(3));
+    }
+    const auto iq = inputs_[0].QuantParams().front();
+    const auto oq = outputs_[0].QuantParams().front();
+    d.in_scale = iq.scale;
+    d.in_zp = iq.zero_point;
+    d.out_scale = oq.scale;
+    d.out_zp = oq.zero_point;
+    std::vector<double> scales;
+    std::vector<int32_t> zps;
+    FilterQuant(w, &scales, &zps);
+    d.filter_quant_num = static_cast<int32_t>(scales.size());
+    d.filter_scales = scales.data();
+    d.filter_zps = zps.data();
+    const void *bias = inputs_.size() > kBiasIndex ? inputs_[kBiasIndex].Data().get() : nullptr;
+    // MI_NOT_SUPPORT (3x3 stride-1 Winograd case, grouped convolution) surfaces here as an error; the creator
+    // below screens those cases out first so that the scheduler falls back instead
+    return ToStatus(
+      mi_conv_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const int32_t *>(bias), &conv_));
+  }
+
+  int ReSize() override { return kSuccess; }
+
+  int Execute() override {
+    const auto s = inputs_[0].Shape();
+    const auto *x = static_cast<const int8_t *>(inputs_[0].Data().get());
+    auto *y = static_cast<int8_t *>(outputs_[0].MutableData());
+    if (x == nullptr || y == nullptr || s.size() != 4) return kLiteNullptr;
+    return ToStatus(mi_conv_run_host(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]),
+                                     static_cast<int32_t>(s[2]), y));
+  }
+
+ private:
+  mi_conv *conv_ = nullptr;
+};
+
+std::shared_ptr<kernel::Kernel> ConvCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
+                                            const schema::Primitive *prim, const Context *ctx) {
+  if (!LibraryReady() || in.size() < 2 || out.size() != 1 || prim == nullptr) return nullptr;
+  const auto *cv = prim->value_as_Conv2DFusion();
+  if (cv == nullptr || cv->kernel_size() == nullptr || cv->stride() == nullptr || cv->dilation() == nullptr) {
+    return nullptr;
+  }
+  const MSTensor &w = in[kWeightIndex];
+  if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || out[0].DataType() != DataType::kNumberTypeInt8) {
+    return nullptr;
+  }
+  if (!PerTensor(in[0]) || !PerTensor(out[0])) return nullptr;
+  if (in.size() > kBiasIndex &&
+      (!in[kBiasIndex].IsConst() || in[kBiasIndex].DataType() != DataType::kNumberTypeInt32)) {
+    return nullptr;
+  }
+  const int64_t kh = cv->kernel_size()->Get(0), kw = cv->kernel_size()->Get(1);
+  const bool depthwise = cv->group() > 1 && cv->group() == cv->in_channel() && cv->group() == cv->out_channel();
+  if (cv->group() != 1 && !depthwise) return nullptr;
+  // on x86 the reference runs its integer Winograd for dense 3x3 stride-1 dilation-1 convolutions
+  // (convolution_int8_creator.cc:41-73), whose results are not those of the exact convolution: leave them to it
+  if (!depthwise && kh == 3 && kw == 3 && cv->stride()->Get(0) == 1 && cv->stride()->Get(1) == 1 &&
+      cv->dilation()->Get(0) == 1 && cv->dilation()->Get(1) == 1) {
+    return nullptr;
+  }
+  return std::make_shared<ConvKernel>(in, out, prim, ctx);
+}
+
+// ---- DynamicQuant, fp32 -> int8 per tensor -------------------------------------------------------------------------
+class DynamicQuantKernel : public kernel::Kernel {
+ public:
+  using Kernel::Kernel;
+  ~DynamicQuantKernel() override { mi_dynquant_destroy(dq_); }
+
+  int Prepare() override {
+    const auto *p = primitive_->value_as_DynamicQuant();
+    return ToStatus(mi_dynquant_create(p->symmetric() ? 1 : 0, &dq_));
+  }
+  int ReSize() override { return kSuccess; }
+  int Execute() override {
+    const auto *x = static_cast<const float *>(inputs_[0].Data().get());
+    auto *q = static_cast<int8_t *>(outputs_[0].MutableData());
+    if (x == nullptr || q == nullptr) return kLiteNullptr;
+    mi_dq_params p{};
+    const int rc = mi_dynquant_run_host(dq_, x, inputs_[0].ElementNum(), q, &p);
+    if (rc != MI_OK) return kLiteError;
+    // what DynamicQuantCPUKernel::CalculatePerlayerScaleZp publishes on the output tensor (dynamic_quant.cc:156-186)
+    QuantParam qp{};
+    qp.bit_num = 8;
+    qp.scale = p.scale;
+    qp.zero_point = p.zero_point;
+    qp.min = p.real_min;
+    qp.max = p.real_max;
+    outputs_[0].SetQuantParams({qp});
+    return kSuccess;
+  }
+
+ private:
+  mi_dynquant *dq_ = nullptr;
+};
+
+std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
+                                                    const schema::Primitive *prim, const Context *ctx) {
+  if (!LibraryReady() || in.size() != 1 || out.size() != 1 || prim == nullptr) return nullptr;
+  const auto *p = prim->value_as_DynamicQuant();
+  if (p == nullptr || p->activation_channel() || (p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0)) {
+    return nullptr;  // per-channel activation scales stay with the builtin kernel
+  }
+  if (p->dst_type() != static_cast<int64_t>(DataType::kNumberTypeInt8)) return nullptr;
+  if (in[0].DataType() != DataType::kNumberTypeFloat32 || out[0].DataType() != DataType::kNumberTypeInt8) {
+    return nullptr;
+  }
+  return std::make_shared<DynamicQuantKernel>(in, out, prim, ctx);
+}
+
+// ---- registration: arch "CPU" for applications, arch "" for the stock benchmark tool --------------------------------
+namespace {
+struct Registrar {
+  Registrar() {
+    for (const char *arch : {"CPU", ""}) {
+      registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeInt8, schema::PrimitiveType_MatMulFusion,
+                                          MatmulCreator);
+      registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeInt8,
+                                          schema::PrimitiveType_FullConnection, MatmulCreator);
+      registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeInt8, schema::PrimitiveType_Conv2DFusion,
+                                          ConvCreator);
+      registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeFloat32,
+                                          schema::PrimitiveType_DynamicQuant, DynamicQuantCreator);
+    }
+  }
+} g_registrar;
+}  // namespace
+}  // namespace mi355x
+}  // namespace mindspore

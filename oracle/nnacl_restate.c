@@ -306,7 +306,12 @@ int orc_conv_dw_int8(const int8_t *in, const int8_t *w, const int32_t *bias, int
         }
       }
       int qi = q.peroc ? c : 0;
-      out[(size_t)p * ch + c] = (int8_t)requant_to_i8(acc, q.mult[qi], q.ls[qi], q.rs[qi], q.zo, q.amin, q.amax);
+      /* ConvDwInt8Post clamps MSMAX(value, acc_min) first, then MSMIN(value, acc_max):
+       * NN/int8/conv_depthwise_int8.c:49-52 (the other order than MatmulInt8Opt; differs only if amin > amax) */
+      int32_t y = wadd(orc_mul_by_quant_mult(acc, q.mult[qi], q.ls[qi], q.rs[qi]), q.zo);
+      if (y < q.amin) y = q.amin;
+      if (y > q.amax) y = q.amax;
+      out[(size_t)p * ch + c] = (int8_t)y;
     }
   }
   requant_ctx_free(&q);
