@@ -94,6 +94,28 @@ def bench_hbm_read(steps, warmup):
     return dict(bytes=slice_bytes, ms=ms, gbps=slice_bytes / (ms * 1e-3) / 1e9)
 
 
+def bench_mfma_rate():
+    """The matrix pipe alone (register operands, no LDS, no memory) on all-zero operands and on operands drawn like
+    the GEMM's (uniform int8): the sustained shader clock, hence the rate, depends on the operand data."""
+    import numpy as np
+    import torch
+    from mindspore_amd import lib
+    L = lib.load()
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    out = {}
+    iters, wgs = 40000, 256
+    for name, data in (("zero_operands", np.zeros(32768, np.int8)),
+                       ("uniform_int8_operands", np.random.default_rng(0).integers(-128, 128, 32768, dtype=np.int8))):
+        ops = torch.from_numpy(data).cuda()
+        fn = lambda: lib.check(L.mi_diag_mfma_rate(ops.data_ptr(), iters, wgs, clocks.data_ptr(), _stream()),
+                               "mi_diag_mfma_rate")
+        ms, _ = time_steps(fn, 3, 1)
+        c = clocks.cpu().numpy()
+        out[name] = dict(tops=wgs * 4 * iters * 16 * 65536.0 / (ms * 1e-3) / 1e12, ms=ms,
+                         shader_clock_ghz=float(c[0]) / (float(c[1]) * 10.0))
+    return out
+
+
 def bench_gemv(steps, warmup, m=1):
     """Decode step: the five 7B-class layer matrices, three layers' worth of distinct weights (606 MB) cycled so the
     256 MB Infinity Cache cannot hold the working set.  Outputs are preallocated; one step = 15 launches."""
@@ -196,6 +218,8 @@ def main():
         other = 8192 if size == 4096 else 4096
         o = bench_gemm(other, max(3, args.steps // 5), 2)
         extra["gemm%d" % other] = dict(ms=o["ms"], tops=o["tops"], frac_of_int8_peak=o["tops"] / PEAK_INT8_TOPS)
+        extra["mfma_only"] = bench_mfma_rate()
+        extra["gemm%d_frac_of_mfma_only_same_data" % size] = g["tops"] / extra["mfma_only"]["uniform_int8_operands"]["tops"]
         extra["hbm_read_stream"] = bench_hbm_read(args.steps, 3)
         extra["gemv_decode_m1"] = bench_gemv(max(5, args.steps // 2), 3, 1)
         extra["gemv_decode_m1"]["frac_of_read_stream"] = extra["gemv_decode_m1"]["gbps"] / extra["hbm_read_stream"]["gbps"]

@@ -133,8 +133,9 @@ static int upload(DevBuf *b, const std::vector<T> &v) {
 
 // ---- shared "requantising GEMM operand" state: packed weights + per-channel epilogue arrays ------------------------
 struct RequantState {
-  int n = 0, k = 0, n_pad = 0, k_pad = 0;
+  int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
+  DevBuf w_blocked;  // built by the first run with 3..16 activation rows
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
   bool has_zw = false, fast = false;
@@ -161,6 +162,7 @@ struct RequantState {
     k = k_;
     n_pad = round_up(n, kNPad);
     k_pad = round_up(k, kKPad);
+    ldw = weight_row_stride(k_pad);
     zo = zo_;
     const bool peroc = nfilt > 1;
     h_mult.assign(n_pad, 0);
@@ -205,8 +207,8 @@ struct RequantState {
     if ((rc = upload(&lshift, h_ls)) != MI_OK) return rc;
     if ((rc = upload(&zw, zwv)) != MI_OK) return rc;
     if (pack_weights) {
-      std::vector<int8_t> packed((size_t)n_pad * k_pad, 0);
-      for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * k_pad, w_nk + (size_t)c * k, (size_t)k);
+      std::vector<int8_t> packed((size_t)n_pad * ldw, 0);
+      for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * ldw, w_nk + (size_t)c * k, (size_t)k);
       if ((rc = upload(&w, packed)) != MI_OK) return rc;
     }
     return MI_OK;
@@ -214,6 +216,7 @@ struct RequantState {
 
   void release() {
     w.release();
+    w_blocked.release();
     mult.release();
     bias2.release();
     rshift.release();
@@ -268,19 +271,32 @@ static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_
 
 // The GEMM kernels write rows with vector stores; when the caller's row length or base address does not allow that,
 // they write to a padded scratch output which is then compacted into the caller's tensor.
-static int run_requant_gemm(const RequantState &st, const int8_t *a, int64_t lda, int rows, int k16, int8_t *c,
+static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int rows, int k16, int8_t *c,
                             DevBuf *c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
-  const int8_t *w = static_cast<const int8_t *>(st.w.p);
-  if (rows <= kGemvMaxRows && (int64_t)rows * k16 <= 150 * 1024)
-    return launch_gemv_requant(a, lda, rows, k16, w, st.k_pad, st.n, rq, c, st.n, stream);
+  WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
+  if (rows <= kGemvMaxRows && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024)) {
+    if (rows > kGemvDotRows) {
+      if (st.w_blocked.p == nullptr) {
+        int rc = st.w_blocked.ensure((size_t)st.n_pad * st.k_pad);
+        if (rc != MI_OK) return rc;
+        rc = launch_block_weights(w.w, st.n_pad, st.k_pad, st.ldw, static_cast<int8_t *>(st.w_blocked.p), stream);
+        if (rc != MI_OK) {
+          st.w_blocked.release();
+          return rc;
+        }
+      }
+      w.blocked = static_cast<const int8_t *>(st.w_blocked.p);
+    }
+    return launch_gemv_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
+  }
   if ((st.n & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 3) == 0)
-    return launch_gemm_requant(a, lda, rows, k16, w, st.k_pad, st.n, rq, c, st.n, stream);
+    return launch_gemm_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
   const int n4 = round_up(st.n, 4);
   int rc = c_ws->ensure((size_t)rows * n4);
   if (rc != MI_OK) return rc;
   RequantParams rq_pad = rq;
-  rc = launch_gemm_requant(a, lda, rows, k16, w, st.k_pad, n4, rq_pad, static_cast<int8_t *>(c_ws->p), n4, stream);
+  rc = launch_gemm_requant(a, lda, rows, k16, w, n4, rq_pad, static_cast<int8_t *>(c_ws->p), n4, stream);
   if (rc != MI_OK) return rc;
   return launch_copy_rows(c_ws->p, n4, rows, st.n, c, st.n, stream);
 }
@@ -309,7 +325,7 @@ struct mi_dynquant {
 };
 
 struct mi_dynmm {
-  int n = 0, k = 0, n_pad = 0, k_pad = 0, act = 0;
+  int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0, act = 0;
   int32_t zw0 = 0;
   bool has_bias = false;
   DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out;
@@ -354,6 +370,17 @@ int mi_diag_copy(void *dst_dev, const void *src_dev, int64_t bytes, void *stream
     return MI_PARAM_INVALID;
   }
   return launch_copy16(dst_dev, src_dev, bytes, static_cast<hipStream_t>(stream));
+}
+
+int mi_diag_mfma_rate(const void *operands_dev, int32_t iters, int32_t workgroups, uint64_t *clocks_dev,
+                      void *stream) {
+  if (operands_dev == nullptr || clocks_dev == nullptr) return MI_NULL_PTR;
+  if (iters <= 0 || workgroups <= 0 || workgroups > 65536 || (reinterpret_cast<uintptr_t>(operands_dev) & 15) != 0) {
+    set_error("mi_diag_mfma_rate: bad iteration / workgroup count or unaligned operands");
+    return MI_PARAM_INVALID;
+  }
+  return launch_mfma_rate(operands_dev, iters, workgroups, reinterpret_cast<unsigned long long *>(clocks_dev),
+                          static_cast<hipStream_t>(stream));
 }
 
 const char *mi_last_error(void) { return g_err; }
@@ -736,15 +763,16 @@ int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const flo
   h->k = d->deep;
   h->n_pad = round_up(h->n, kNPad);
   h->k_pad = round_up(h->k, kKPad);
+  h->ldw = weight_row_stride(h->k_pad);
   h->act = d->act_type;
   h->zw0 = d->filter_zps[0];
   h->has_bias = bias_host != nullptr;
   const std::vector<int8_t> w_nk = to_nk(weight_host, h->n, h->k, d->b_transpose);
-  std::vector<int8_t> packed((size_t)h->n_pad * h->k_pad, 0);
+  std::vector<int8_t> packed((size_t)h->n_pad * h->ldw, 0);
   std::vector<float> ws(h->n_pad, 0.0f), bs(h->n_pad, 0.0f);
   std::vector<int32_t> wsum(h->n_pad, 0);
   for (int c = 0; c < h->n; ++c) {
-    memcpy(packed.data() + (size_t)c * h->k_pad, w_nk.data() + (size_t)c * h->k, (size_t)h->k);
+    memcpy(packed.data() + (size_t)c * h->ldw, w_nk.data() + (size_t)c * h->k, (size_t)h->k);
     int32_t s = 0;
     for (int i = 0; i < h->k; ++i) s += w_nk[(size_t)c * h->k + i];
     wsum[c] = s;
@@ -787,12 +815,12 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   dq.zw0 = h->zw0;
   dq.deep = h->k;
   dq.act = h->act;
-  const int8_t *w = static_cast<const int8_t *>(h->w.p);
+  const WeightView w{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw, nullptr};
   if ((h->n & 3) == 0 && (reinterpret_cast<uintptr_t>(c_dev) & 15) == 0)
-    return launch_gemm_dequant(a, lda, rows, k16, w, h->k_pad, h->n, dq, c_dev, h->n, s);
+    return launch_gemm_dequant(a, lda, rows, k16, w, h->n, dq, c_dev, h->n, s);
   const int n4 = round_up(h->n, 4);
   if ((rc = h->c_ws.ensure((size_t)rows * n4 * sizeof(float))) != MI_OK) return rc;
-  if ((rc = launch_gemm_dequant(a, lda, rows, k16, w, h->k_pad, n4, dq, static_cast<float *>(h->c_ws.p), n4, s)) != MI_OK)
+  if ((rc = launch_gemm_dequant(a, lda, rows, k16, w, n4, dq, static_cast<float *>(h->c_ws.p), n4, s)) != MI_OK)
     return rc;
   return launch_copy_rows(h->c_ws.p, (int64_t)n4 * 4, rows, h->n * 4, c_dev, (int64_t)h->n * 4, s);
 }

@@ -53,18 +53,36 @@ struct DequantParams {
   int32_t act;
 };
 
+// Packed weights: n_pad rows (output channels) of k_pad contraction bytes, zero filled past K, with row stride ldw.
+// The stride is skewed to an odd multiple of 256 bytes: the kernels fetch 16 rows x 64 bytes per wave instruction,
+// and with a power-of-two stride those 16 requests would all fall into the same memory channel.
+struct WeightView {
+  const int8_t *w;
+  int k_pad;
+  int ldw;
+  // Second copy for the matrix-core decode kernel (3..16 activation rows), or nullptr: the same bytes regrouped into
+  // 1 KiB blocks [row / 16][k / 64][row % 16][k % 64], so that the 16 rows x 64 bytes a wave instruction fetches are
+  // contiguous.  Built on the device on first use (launch_block_weights).
+  const int8_t *blocked;
+};
+inline int weight_row_stride(int k_pad) { return (k_pad / 256) % 2 == 0 ? k_pad + 256 : k_pad; }
+
 // A: int8 activations [M][lda] (lda in bytes, multiple of 16, base 16-byte aligned, K % 16 == 0);
-// W: packed weights [n_pad][k_pad]; C: [M][ldc] elements with n % 4 == 0, ldc % 4 == 0 and a 4-byte (int8) /
+// W: packed weights (above); C: [M][ldc] elements with n % 4 == 0, ldc % 4 == 0 and a 4-byte (int8) /
 // 16-byte (fp32) aligned base -- other output shapes go through a padded scratch buffer and launch_copy_rows.
-int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
-int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
 
 // Skinny-M path (m <= kGemvMaxRows): streams the weights once with 16-byte coalesced loads.
-constexpr int kGemvMaxRows = 8;
-int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+constexpr int kGemvMaxRows = 16;
+constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel (activations staged in LDS), above it the MFMA kernel
+int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
+
+// Regroups packed row-major weights into the blocked copy described at WeightView::blocked.
+int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t *blocked, hipStream_t stream);
 
 // Copies [rows][k] (row stride src_ld bytes) into a zero-padded [rows][k16] buffer, k16 = round_up(k, 16).
 int launch_pad_rows(const int8_t *src, int64_t src_ld, int rows, int k, int8_t *dst, int k16, hipStream_t stream);
@@ -86,6 +104,11 @@ int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, cons
 // Measurement aids: read `bytes` and discard them / copy them, 16 bytes per lane.
 int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream);
 int launch_copy16(void *dst, const void *src, int64_t bytes, hipStream_t stream);
+
+// Measurement aid: `iters` x 16 v_mfma_i32_32x32x32_i8 per wave on the given operand bytes (32 KiB), 4 waves per
+// workgroup; clocks[0..1] (device memory) receive shader cycles and 100 MHz ticks of the loop.
+int launch_mfma_rate(const void *operands, int iters, int workgroups, unsigned long long *clocks,
+                     hipStream_t stream);
 
 // DynamicQuant: per-block min/max partials, then quantise (every block re-reduces the partials).
 constexpr int kDqMaxBlocks = 1024;

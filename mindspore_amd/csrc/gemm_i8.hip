@@ -36,7 +36,8 @@ struct GemmArgs {
   int m;
   int k;  // bytes of K that may be read from A (multiple of 16)
   const int8_t *w;
-  int ldw;  // k_pad
+  int ldw;    // weight row stride in bytes
+  int k_pad;  // contraction extent of the packed weights (zero filled past K)
   int n;
   int tiles_m, tiles_n;
   void *c;
@@ -322,7 +323,7 @@ __device__ __forceinline__ void hint_interleave_reads() {
 // direct main loop: 4 LDS stages x 64 bytes of K, asynchronous global -> LDS loads three tiles ahead
 // =====================================================================================================================
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
-__global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
   constexpr int BKD = 64, NST = 4;
   constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
   constexpr int STAGE = (TILE_N + TILE_M) * BKD;
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
   const int r = lane & 31, h = lane >> 5;
-  const int ktiles = g.ldw / BKD;  // multiple of 4
+  const int ktiles = g.k_pad / BKD;  // multiple of 4
   EpiParams<TILE_N, EPI> epi;
   epi.fetch(rq, dq, n0, tid);
 
@@ -401,24 +402,30 @@ __global__ __launch_bounds__(256) void gemm_direct_kernel(GemmArgs g, RequantPar
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const int nxt = kt + 3 < ktiles ? kt + 3 : ktiles - 1;
-    dma_tile((st + 3) & 3, nxt);
     read_frag(f0, (st + 1) & 3, 0);
+    dma_tile((st + 3) & 3, nxt);
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
     {
-      constexpr int kMfma = TN * TM;
-      if constexpr (kMfma >= LPW) {
+      // operand reads first (the next sub-step waits for them), the loads of tile kt+3 behind them (they have
+      // almost three steps to land)
+      constexpr int kMfma = TN * TM, kReads = TN + TM;
+      if constexpr (kMfma >= kReads + LPW) {
+#pragma unroll
+        for (int i = 0; i < kReads; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        }
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
           __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
         }
       } else {
 #pragma unroll
         for (int i = 0; i < kMfma; ++i) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, LPW / kMfma, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, (TN + TM) / kMfma, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, (kReads + kMfma - 1) / kMfma, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, (LPW + kMfma - 1) / kMfma, 0);
         }
       }
     }
@@ -463,7 +470,7 @@ __global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
   const int r = lane & 31, h = lane >> 5;
-  const int ktiles = g.ldw / BK, kchunks = g.k >> 4;
+  const int ktiles = g.k_pad / BK, kchunks = g.k >> 4;
   EpiParams<TILE_N, EPI> epi;
   epi.fetch(rq, dq, n0, tid);
 
@@ -561,7 +568,7 @@ static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &
   g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
   const int blocks = g.tiles_m * g.tiles_n;
   // the asynchronous global->LDS loader cannot zero-fill, so it needs every 64-byte K step of A to be in bounds
-  if (g.k == g.ldw) {
+  if (g.k == g.k_pad) {
     hipLaunchKernelGGL((gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
                        rq, dq);
   } else {
@@ -582,14 +589,16 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
 
-static int check_args(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n, const void *c,
+static int check_args(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n, const void *c,
                       int64_t ldc, int c_align) {
+  const int8_t *w = wv.w;
+  const int k_pad = wv.k_pad;
   if (a == nullptr || w == nullptr || c == nullptr) {
     set_error("gemm: null pointer");
     return MI_NULL_PTR;
   }
   if (m <= 0 || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k || k_pad % kKPad != 0 || k_pad < k ||
-      (reinterpret_cast<uintptr_t>(a) & 15) != 0 || (n & 3) != 0 || (ldc & 3) != 0 || ldc < n ||
+      wv.ldw < k_pad || (wv.ldw & 15) != 0 || (reinterpret_cast<uintptr_t>(a) & 15) != 0 || (n & 3) != 0 || (ldc & 3) != 0 || ldc < n ||
       (reinterpret_cast<uintptr_t>(c) & (c_align - 1)) != 0) {
     set_error("gemm: unsupported operand geometry m=%d n=%d k=%d lda=%lld k_pad=%d ldc=%lld", m, n, k, (long long)lda,
               k_pad, (long long)ldc);
@@ -598,11 +607,11 @@ static int check_args(const int8_t *a, int64_t lda, int m, int k, const int8_t *
   return MI_OK;
 }
 
-int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
-  int rc = check_args(a, lda, m, k, w, k_pad, n, c, ldc, 4);
+  int rc = check_args(a, lda, m, k, w, n, c, ldc, 4);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k, w, k_pad, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
   DequantParams dq{};
   if (rq.has_zw) {
     return rq.fast ? launch_pick_tile<EPI_REQUANT, true, true>(g, rq, dq, stream)
@@ -612,14 +621,59 @@ int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t
                  : launch_pick_tile<EPI_REQUANT, false, false>(g, rq, dq, stream);
 }
 
-int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream) {
-  int rc = check_args(a, lda, m, k, w, k_pad, n, c, ldc, 16);
+  int rc = check_args(a, lda, m, k, w, n, c, ldc, 16);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k, w, k_pad, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
   RequantParams rq{};
   return dq.zw0 != 0 ? launch_pick_tile<EPI_DEQUANT, true, false>(g, rq, dq, stream)
                      : launch_pick_tile<EPI_DEQUANT, false, false>(g, rq, dq, stream);
+}
+
+// Measurement aid: nothing but back-to-back MFMAs on register operands taken from `operands` (256 threads x 8 x 16
+// bytes), one workgroup per CU, one wave per SIMD -- the rate the matrix pipe sustains for THAT operand data.  The
+// sustained shader clock depends on how many operand bits toggle, so the caller passes data like the GEMM's.
+// clocks[0] = shader cycles, clocks[1] = 100 MHz ticks spent in the loop by workgroup 0.
+__global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i *__restrict__ operands, int iters,
+                                                        unsigned long long *__restrict__ clocks,
+                                                        int *__restrict__ sink) {
+  v16i acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[i][e] = 0;
+  v4i fa[4], fb[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    fa[i] = operands[threadIdx.x * 8 + i];
+    fb[i] = operands[threadIdx.x * 8 + 4 + i];
+  }
+  const unsigned long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 3], fb[i >> 2], acc[i], 0, 0, 0);
+  }
+  const unsigned long long c1 = clock64(), w1 = wall_clock64();
+  int t = 0;
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) t += acc[i][e];
+  if (t == 0x5ca1ab1e && iters < 0) sink[0] = t;  // never true; keeps the accumulators alive
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    clocks[0] = c1 - c0;
+    clocks[1] = w1 - w0;
+  }
+}
+
+int launch_mfma_rate(const void *operands, int iters, int workgroups, unsigned long long *clocks,
+                     hipStream_t stream) {
+  hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(256), 0, stream, static_cast<const v4i *>(operands),
+                     iters, clocks, static_cast<int *>(nullptr));
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
 }
 
 }  // namespace mi

@@ -1,5 +1,5 @@
-// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 8 activation rows
-// against an [n_pad][k_pad] int8 weight matrix.  The kernel is HBM-bound on the weight stream, so the design goal
+// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 16 activation rows
+// against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw) (v_dot4 kernel for M <= 2, matrix-core kernel for 3 <= M <= 16).  The kernel is HBM-bound on the weight stream, so the design goal
 // is "every weight byte crosses HBM once, in 1 KiB coalesced wave loads, with enough loads in flight":
 //   - a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes);
 //   - it keeps D 16-byte loads per lane (D KiB per wave) in flight at all times, refilling a register slot as soon
@@ -40,7 +40,8 @@ struct GemvArgs {
   int64_t lda;
   int kchunks;  // K / 16
   const int8_t *w;
-  int ldw;  // k_pad
+  int ldw;    // weight row stride in bytes
+  int k_pad;  // contraction extent of a (zero padded) weight row
   int n;
   int8_t *c;
   int64_t ldc;
@@ -192,39 +193,197 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
   // once (a wave that loops needs >= 8-16 resident waves per CU to keep up).  So pick the rows per wave so that a
   // wave's R x ceil(K / 1 KiB) chunks fit the in-flight budget, and fall back to looping for very long rows.
   const int nseg = (g.kchunks + 63) >> 6;
-  if (M >= 3) {  // register pressure grows with M: shorter queues, more rows per wave where there are many rows
-    if (g.n >= 8192 || nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
-    return launch_mrd<M, 2, 8>(g, rq, stream);
-  }
   if (nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
   if (nseg == 2) return launch_mrd<M, 4, 8>(g, rq, stream);
   if (nseg <= 4 || M == 2) return launch_mrd<M, 2, 8>(g, rq, stream);
   return launch_mrd<M, 1, 12>(g, rq, stream);
 }
 
-int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const int8_t *w, int k_pad, int n,
+// =====================================================================================================================
+// 3 <= M <= 16 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
+// v_mfma_i32_16x16x64_i8 with the WEIGHTS as the 16-row operand: lane (g = lane / 16, i = lane % 16) supplies 16
+// contiguous K bytes of weight row i (K offset 16 g inside the 64-byte step) and the same 16 K bytes of activation row
+// i (zero for i >= M); the result register r of that lane is output (channel 4 g + r, activation row i).
+// The weights come from the blocked copy ([row / 16][k / 64][row % 16][k % 64]), so the 1 KiB a wave instruction fetches
+// is contiguous and a wave's consecutive steps walk consecutive KiB.
+// A workgroup of 8 waves owns RG x 16 channels; the waves split K into contiguous slices, each wave keeps D steps
+// (D x RG KiB of weights) in flight, and the partial sums meet in LDS.
+// =====================================================================================================================
+template <int RG, int D>
+__global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, RequantParams rq) {
+  constexpr int WAVES = 8;
+  __shared__ v4i red[WAVES][RG + 1][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane >> 4, idx = lane & 15;
+  const int n0 = blockIdx.x * (RG * 16);
+  const int k_bytes = g.kchunks * 16;
+  const int total = g.k_pad >> 6;  // 64-byte steps in a (zero padded) weight row
+  const int spw = (total + WAVES - 1) / WAVES;
+  const int s0 = wave * spw;
+  // blocked weights: 1 KiB block (row group, step) = 16 rows x 64 bytes; lane (grp, idx) takes row idx, chunk grp
+  const int8_t *wbase = g.w + (int64_t)(n0 >> 4) * total * 1024 + idx * 64 + grp * 16;
+  const int arow = idx < m_rows ? idx : m_rows - 1;
+  const int8_t *abase = g.a + (int64_t)arow * g.lda;
+
+  // the finishing lanes (first RG waves) fetch their channels' parameters while the weights stream
+  int32_t p_mult[4], p_e[4], p_ls[4], p_bias2[4], p_zw[4];
+  if (wave < RG) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = n0 + wave * 16 + 4 * grp + r;
+      p_mult[r] = rq.mult[n];
+      p_e[r] = rq.rshift[n];
+      p_ls[r] = rq.lshift[n];
+      p_bias2[r] = rq.bias2[n];
+      p_zw[r] = rq.zw[n];
+    }
+  }
+
+  auto load_w = [&](int j, int rg) -> v4i {
+    int s = s0 + j;
+    s = s < total ? s : total - 1;
+    return *reinterpret_cast<const v4i *>(wbase + ((int64_t)rg * total + s) * 1024);
+  };
+  auto load_x = [&](int j) -> v4i {
+    int off = (s0 + j) * 64 + grp * 16;
+    off = off < k_bytes ? off : k_bytes - 16;
+    return *reinterpret_cast<const v4i *>(abase + off);
+  };
+  v4i wbuf[D][RG], xbuf[D];
+#pragma unroll
+  for (int j = 0; j < D; ++j) {
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(j, rg);
+    xbuf[j] = load_x(j);
+  }
+
+  v4i acc[RG], asum = {0, 0, 0, 0};
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) acc[rg] = v4i{0, 0, 0, 0};
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+
+  auto pass = [&](int base, auto refill) {
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+      const int jj = base + j;
+      const bool live = idx < m_rows && jj < spw && s0 + jj < total && (s0 + jj) * 64 + grp * 16 < k_bytes;
+      v4i x = xbuf[j];
+      x.x = live ? x.x : 0;
+      x.y = live ? x.y : 0;
+      x.z = live ? x.z : 0;
+      x.w = live ? x.w : 0;
+      v4i w[RG];
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];
+      if (decltype(refill)::value) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(jj + D, rg);
+        xbuf[j] = load_x(jj + D);
+      }
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) acc[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x, acc[rg], 0, 0, 0);
+      if (rq.has_zw) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x, asum, 0, 0, 0);
+    }
+  };
+  int base = 0;
+  for (; base + D < spw; base += D) pass(base, std::true_type());
+  pass(base, std::false_type());
+
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) red[wave][rg][lane] = acc[rg];
+  red[wave][RG][lane] = asum;
+  __syncthreads();
+  if (wave < RG) {
+    v4i tot = {0, 0, 0, 0}, xs = {0, 0, 0, 0};
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      tot += red[w][wave][lane];
+      xs += red[w][RG][lane];
+    }
+    if (idx < m_rows) {
+      const int nb = n0 + wave * 16 + 4 * grp;
+      int8_t outv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        uint32_t v = (uint32_t)tot[r];
+        if (rq.has_zw) v -= (uint32_t)xs[0] * (uint32_t)p_zw[r];
+        v += (uint32_t)p_bias2[r];
+        int32_t y;
+        if (rq.fast) {
+          y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[r]), p_e[r], (1 << p_e[r]) >> 1);
+        } else {
+          y = rdiv_pot(srdhm((int32_t)(v << p_ls[r]), p_mult[r]), p_e[r]);
+        }
+        y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+        y = y < rq.amax ? y : rq.amax;
+        y = y > rq.amin ? y : rq.amin;
+        outv[r] = (int8_t)y;
+      }
+      int8_t *dst = g.c + (int64_t)idx * g.ldc + nb;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (nb + r < g.n) dst[r] = outv[r];
+    }
+  }
+}
+
+template <int RG, int D>
+static int launch_mfma(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  hipLaunchKernelGGL((gemv_mfma_kernel<RG, D>), dim3(blocks), dim3(512), 0, stream, g, m, rq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+__global__ __launch_bounds__(256) void block_weights_kernel(const int8_t *__restrict__ w, int ldw, int kblocks,
+                                                            int64_t chunks, int8_t *__restrict__ blocked) {
+  // one 16-byte chunk per thread; destination order, so the stores coalesce
+  for (int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * blockDim.x) {
+    const int in_block = (int)(c & 63);
+    const int64_t blk = c >> 6;
+    const int row = (int)(blk / kblocks) * 16 + (in_block >> 2);
+    const int kbyte = (int)(blk % kblocks) * 64 + (in_block & 3) * 16;
+    *reinterpret_cast<v4i *>(blocked + c * 16) = *reinterpret_cast<const v4i *>(w + (int64_t)row * ldw + kbyte);
+  }
+}
+
+int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t *blocked, hipStream_t stream) {
+  const int64_t chunks = (int64_t)n_pad * k_pad / 16;
+  const int64_t want = (chunks + 255) / 256;
+  hipLaunchKernelGGL(block_weights_kernel, dim3((unsigned)(want > 65536 ? 65536 : want)), dim3(256), 0, stream, w, ldw,
+                     k_pad / 64, chunks, blocked);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
+  const int8_t *w = wv.w;
+  const int k_pad = wv.k_pad;
   if (a == nullptr || w == nullptr || c == nullptr) {
     set_error("gemv: null pointer");
     return MI_NULL_PTR;
   }
   if (m < 1 || m > kGemvMaxRows || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
-      k_pad % kKPad != 0 || k_pad < k || (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
-      (int64_t)m * round_up(k, 1024) > 160 * 1024 - 1024) {
+      k_pad % kKPad != 0 || k_pad < k || wv.ldw < k_pad || (wv.ldw & 15) != 0 ||
+      (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
+      (m <= kGemvDotRows && (int64_t)m * round_up(k, 1024) > 160 * 1024 - 1024)) {
     set_error("gemv: unsupported operand geometry m=%d n=%d k=%d lda=%lld", m, n, k, (long long)lda);
     return MI_PARAM_INVALID;
   }
-  GemvArgs g{a, lda, k / 16, w, k_pad, n, c, ldc};
-  switch (m) {
-    case 1: return launch_m<1>(g, rq, stream);
-    case 2: return launch_m<2>(g, rq, stream);
-    case 3: return launch_m<3>(g, rq, stream);
-    case 4: return launch_m<4>(g, rq, stream);
-    case 5: return launch_m<5>(g, rq, stream);
-    case 6: return launch_m<6>(g, rq, stream);
-    case 7: return launch_m<7>(g, rq, stream);
-    default: return launch_m<8>(g, rq, stream);
+  GemvArgs g{a, lda, k / 16, w, wv.ldw, k_pad, n, c, ldc};
+  if (m > kGemvDotRows) {
+    if (wv.blocked == nullptr) {
+      set_error("gemv: the blocked weight copy is missing");
+      return MI_NULL_PTR;
+    }
+    g.w = wv.blocked;
+    // two 16-channel groups per workgroup (half the activation traffic) once there are enough channels to fill the
+    // device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4>(g, m, rq, stream);
+    return launch_mfma<1, 8>(g, m, rq, stream);
   }
+  return m == 1 ? launch_m<1>(g, rq, stream) : launch_m<2>(g, rq, stream);
 }
 
 }  // namespace mi

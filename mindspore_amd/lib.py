@@ -19,7 +19,7 @@ EXPORTS = [
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
     "mi_dynquant_run_host", "mi_dynquant_destroy",
     "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_destroy",
-    "mi_diag_stream_read", "mi_diag_copy",
+    "mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate",
 ]
 
 
@@ -114,6 +114,7 @@ def load():
     L.mi_dynmm_destroy.restype = None
     L.mi_diag_stream_read.argtypes = [vp, i64, vp]
     L.mi_diag_copy.argtypes = [vp, vp, i64, vp]
+    L.mi_diag_mfma_rate.argtypes = [vp, i32, i32, vp, vp]
     _lib = L
     return L
 
