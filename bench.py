@@ -163,6 +163,55 @@ def bench_bert(steps, warmup):
     return out
 
 
+def bench_small_configs(steps, warmup):
+    """Configuration 1 (FullConnection 128x768x768) and configuration 2 (MobileNetV2-style block, device-resident
+    chain of stem 3x3 s2, 1x1 expand, 3x3 depthwise, 1x1 project): latency per layer, algorithmic bytes moved."""
+    import torch
+    from mindspore_amd import kernels as K
+    from mindspore_amd import workloads as wl
+    out = {}
+    c = wl.fc_c1()
+    fc = make_matmul(c)
+    a = torch.from_numpy(c["a"]).cuda()
+    o = torch.empty((128, 768), dtype=torch.int8, device="cuda")
+    ms, _ = time_steps(lambda: fc.run(a, out=o), steps, warmup)
+    out["c1_fc_128x768x768"] = dict(us=ms * 1e3, tops=2.0 * 128 * 768 * 768 / (ms * 1e-3) / 1e12)
+    x, layers = wl.mobilenet_c2()
+    cur = torch.from_numpy(x).cuda()
+    kerns, ins = [], []
+    for L in layers:
+        qp = [K.QuantParam(float(sc), int(z)) for sc, z in zip(L["sw"], L["zw"])]
+        kern = K.ConvolutionInt8Kernel(L["w"], L["bias"], K.QuantParam(L["sx"], L["zx"]), qp,
+                                       K.QuantParam(L["so"], L["zo"]), (L["stride"],) * 2, (1, 1), L["pad"],
+                                       L["oc"] if L["kind"] == "dw" else 1, L["act"])
+        kerns.append(kern)
+        ins.append(cur)
+        cur = kern.run(cur)
+    outs = [kern.run(xin) for kern, xin in zip(kerns, ins)]
+    for L, kern, xin, yout in zip(layers, kerns, ins, outs):
+        ms, _ = time_steps(lambda: kern.run(xin, out=yout), steps, warmup)
+        nbytes = xin.numel() + yout.numel() + L["w"].size
+        out["c2_" + L["name"]] = dict(us_eager_call=ms * 1e3, in_shape=list(xin.shape), out_shape=list(yout.shape),
+                                      algorithmic_bytes=nbytes)
+    # the whole block as one captured HIP graph (five kernels), replayed: what the GPU needs once the host's
+    # per-call cost is out of the way
+    def chain():
+        cur = ins[0]
+        for kern, yout in zip(kerns, outs):
+            cur = kern.run(cur, out=yout)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        chain()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            chain()
+    torch.cuda.synchronize()
+    ms, _ = time_steps(graph.replay, steps, warmup)
+    total_us = ms * 1e3
+    out["c2_block_graph_us"] = total_us
+    return out
+
+
 def cpu_baseline(case, size):
     """nnacl's CPU path (compiled from the reference tree, oracle/_ref) -- or the restatement if that library did
     not travel -- on a bounded sample: the first `rows` activation rows of the same GEMM, all host cores."""
@@ -225,6 +274,7 @@ def main():
         extra["gemv_decode_m1"]["frac_of_read_stream"] = extra["gemv_decode_m1"]["gbps"] / extra["hbm_read_stream"]["gbps"]
         extra["gemv_decode_m8"] = bench_gemv(max(5, args.steps // 2), 3, 8)
         extra.update(bench_bert(max(5, args.steps // 2), 3))
+        extra.update(bench_small_configs(max(5, args.steps // 2), 3))
     result = {
         "metric": "int8 GEMM TOPS + % i8 MFMA peak; decode GEMV HBM GB/s; vs nnacl CPU",
         "value": g["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -200,12 +200,87 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const int8_t *__restrict__
   }
 }
 
+// Channel-vectorised variant for C % 16 == 0: one thread produces 16 consecutive channels of one output pixel, so
+// every tap is one 16-byte activation load and two 16-byte weight loads, and the store is one 16-byte row segment.
+__global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict__ in, ConvGeom g,
+                                                        const int16_t *__restrict__ w16,
+                                                        const int32_t *__restrict__ bias, int zx8, RequantParams rq,
+                                                        int8_t *__restrict__ out) {
+  const int ch = g.out_c, groups = ch >> 4;
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * groups;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t p = idx / groups;
+    const int c0 = (int)(idx - p * groups) << 4;
+    const int b = (int)(p / ((int64_t)g.out_h * g.out_w));
+    const int rem = (int)(p - (int64_t)b * g.out_h * g.out_w);
+    const int oh = rem / g.out_w, ow = rem - oh * g.out_w;
+    const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * ch + c0;
+    uint32_t acc[16];
+    {
+      const v4i *bp = reinterpret_cast<const v4i *>(bias + c0);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const v4i bv = bp[q];
+        acc[4 * q + 0] = (uint32_t)bv.x;
+        acc[4 * q + 1] = (uint32_t)bv.y;
+        acc[4 * q + 2] = (uint32_t)bv.z;
+        acc[4 * q + 3] = (uint32_t)bv.w;
+      }
+    }
+    for (int kh = 0; kh < g.kernel_h; ++kh) {
+      const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
+      if (ih < 0 || ih >= g.in_h) continue;
+      for (int kw = 0; kw < g.kernel_w; ++kw) {
+        const int iw = ow * g.stride_w - g.pad_l + kw * g.dilation_w;
+        if (iw < 0 || iw >= g.in_w) continue;
+        union {
+          v4i v;
+          int8_t b[16];
+        } xv;
+        union {
+          v4i v[2];
+          int16_t h[16];
+        } wv;
+        xv.v = *reinterpret_cast<const v4i *>(img + ((int64_t)ih * g.in_w + iw) * ch);
+        const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)(kh * g.kernel_w + kw) * ch + c0);
+        wv.v[0] = wp[0];
+        wv.v[1] = wp[1];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int32_t xs = (int16_t)((int)xv.b[j] - zx8);  // both factors fit 9 bits + sign: a 24-bit multiply
+          acc[j] += (uint32_t)(xs * (int32_t)wv.h[j]);
+        }
+      }
+    }
+    union {
+      v4i v;
+      int8_t b[16];
+    } o;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int c = c0 + j;
+      int32_t y = rdiv_pot(srdhm((int32_t)(acc[j] << rq.lshift[c]), rq.mult[c]), rq.rshift[c]);
+      y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+      y = y > rq.amin ? y : rq.amin;  // MSMAX first, then MSMIN (conv_depthwise_int8.c:49-50)
+      y = y < rq.amax ? y : rq.amax;
+      o.b[j] = (int8_t)y;
+    }
+    *reinterpret_cast<v4i *>(out + p * ch + c0) = o.v;
+  }
+}
+
 int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
                    const RequantParams &rq, int8_t *out, hipStream_t stream) {
-  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * g.out_c;
+  const bool vec = (g.out_c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * (vec ? g.out_c >> 4 : g.out_c);
   const int64_t want = (total + 255) / 256;
   const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
-  hipLaunchKernelGGL(conv_dw_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+  if (vec) {
+    hipLaunchKernelGGL(conv_dw16_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+  } else {
+    hipLaunchKernelGGL(conv_dw_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+  }
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }

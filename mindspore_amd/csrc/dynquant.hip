@@ -3,7 +3,7 @@
 //                         CalculateMinMaxFp32 (reference mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/
 //                         dynamic_quant_int8.c:19-27; a NaN is never selected), wavefront shuffle reduction, one
 //                         (min, max) partial per workgroup
-//   pass 2  dq_quantize : every workgroup re-reduces the <= 1024 partials (4 KiB, L2 resident), derives
+//   pass 2  dq_quantize : every workgroup re-reduces the <= 256 partials (2 KiB, L2 resident), derives
 //                         scale / zero point exactly as DynamicQuantCPUKernel::CalculatePerlayerScaleZp does
 //                         (mindspore/lite/src/litert/kernel/cpu/int8/dynamic_quant.cc:156-186: float range, float
 //                         division, zero point in double) and quantises its slice with the arithmetic of
@@ -59,7 +59,20 @@ __global__ __launch_bounds__(kDqThreads) void dq_minmax_kernel(const float *__re
   if ((reinterpret_cast<uintptr_t>(x) & 15) == 0) {
     const int64_t n4 = n >> 2;
     const v4f *x4 = reinterpret_cast<const v4f *>(x);
-    for (int64_t i = gtid; i < n4; i += stride) {
+    int64_t i = gtid;
+    for (; i + 3 * stride < n4; i += 4 * stride) {  // four independent 16-byte loads in flight per thread
+      v4f v[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = x4[i + j * stride];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        upd(v[j].x, lo, hi);
+        upd(v[j].y, lo, hi);
+        upd(v[j].z, lo, hi);
+        upd(v[j].w, lo, hi);
+      }
+    }
+    for (; i < n4; i += stride) {
       const v4f v = x4[i];
       upd(v.x, lo, hi);
       upd(v.y, lo, hi);
@@ -96,6 +109,21 @@ __global__ __launch_bounds__(kDqThreads) void dq_quantize_kernel(const float *__
                                                                  mi_dq_params *__restrict__ params,
                                                                  int8_t *__restrict__ q) {
   __shared__ float slo[kDqThreads / 64], shi[kDqThreads / 64];
+  // request this thread's 16 values first: they arrive while the partials are reduced and the scale is derived
+  const int64_t base = ((int64_t)blockIdx.x * kDqThreads + threadIdx.x) * kDqElemsPerThread;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0);
+  const bool fast = aligned && base + kDqElemsPerThread <= n;
+  v4f xv[4];
+  {
+    // never predicated: a thread without a full group of its own re-reads the first one (n >= 16 on this path)
+    const int64_t safe = fast ? base : 0;
+    const v4f *x4 = reinterpret_cast<const v4f *>(x + (aligned && n >= kDqElemsPerThread ? safe : 0));
+    if (aligned && n >= kDqElemsPerThread) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xv[j] = x4[j];
+    }
+  }
+
   float lo = FLT_MAX, hi = -FLT_MAX;
   for (int i = threadIdx.x; i < nparts; i += kDqThreads) {
     const float2 p = partials[i];
@@ -129,18 +157,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_quantize_kernel(const float *__
   const float inv = __fdiv_rn(1.0f, scale_f);
   const float zpf = (float)zp;
 
-  const int64_t base = ((int64_t)blockIdx.x * kDqThreads + threadIdx.x) * kDqElemsPerThread;
   if (base >= n) return;
-  const bool aligned = ((reinterpret_cast<uintptr_t>(x) & 15) == 0) && ((reinterpret_cast<uintptr_t>(q) & 15) == 0);
-  if (aligned && base + kDqElemsPerThread <= n) {
-    const v4f *x4 = reinterpret_cast<const v4f *>(x + base);
+  if (fast) {
     union {
       int4 v;
       int8_t b[16];
     } u;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const v4f v = x4[j];
+      const v4f v = xv[j];
       u.b[4 * j + 0] = quant_one(v.x, inv, zpf);
       u.b[4 * j + 1] = quant_one(v.y, inv, zpf);
       u.b[4 * j + 2] = quant_one(v.z, inv, zpf);
@@ -157,7 +182,9 @@ int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, 
                     hipStream_t stream) {
   const int64_t per_block = (int64_t)kDqThreads * kDqElemsPerThread;
   int64_t want = (n + per_block - 1) / per_block;
-  const int nparts = (int)(want < 1 ? 1 : (want > kDqMaxBlocks ? kDqMaxBlocks : want));
+  // pass 1: at most one workgroup per partial a thread of pass 2 reads in a single step
+  const int64_t want1 = (want + 2) / 3;
+  const int nparts = (int)(want1 < 1 ? 1 : (want1 > kDqThreads ? kDqThreads : want1));
   hipLaunchKernelGGL(dq_minmax_kernel, dim3(nparts), dim3(kDqThreads), 0, stream, x, n, partials);
   MI_HIP_CHECK(hipGetLastError());
   const int64_t qblocks = want < 1 ? 1 : want;

@@ -470,7 +470,7 @@ __global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
   const int r = lane & 31, h = lane >> 5;
-  const int ktiles = g.k_pad / BK, kchunks = g.k >> 4;
+  const int ktiles = (g.k + BK - 1) / BK, kchunks = g.k >> 4;  // the zero padding past K needs no MFMAs
   EpiParams<TILE_N, EPI> epi;
   epi.fetch(rq, dq, n0, tid);
 

@@ -169,7 +169,9 @@ class ConvolutionInt8Kernel(_Handle):
         _lib.check(_lib.load().mi_conv_out_shape(self._h, in_h, in_w, C.byref(oh), C.byref(ow)), "mi_conv_out_shape")
         return oh.value, ow.value
 
-    def run(self, x):
+    def run(self, x, out=None):
+        """x: int8 NHWC as a numpy array (host path) or a contiguous CUDA tensor (device path, current stream);
+        `out` (device path only) is a preallocated contiguous CUDA int8 tensor of the output shape."""
         L = _lib.load()
         if x.ndim != 4 or x.shape[3] != self.ic:
             raise ValueError("expected NHWC with %d channels, got %s" % (self.ic, tuple(x.shape)))
@@ -179,7 +181,11 @@ class ConvolutionInt8Kernel(_Handle):
             import torch
             if x.dtype != torch.int8 or not x.is_cuda or not x.is_contiguous():
                 raise ValueError("expected a contiguous CUDA int8 tensor")
-            out = torch.empty((b, oh, ow, self.oc), dtype=torch.int8, device=x.device)
+            if out is None:
+                out = torch.empty((b, oh, ow, self.oc), dtype=torch.int8, device=x.device)
+            elif (out.dtype != torch.int8 or not out.is_cuda or not out.is_contiguous()
+                  or out.numel() != b * oh * ow * self.oc):
+                raise ValueError("out must be a contiguous CUDA int8 tensor with %d elements" % (b * oh * ow * self.oc))
             _lib.check(L.mi_conv_run(self._h, x.data_ptr(), b, ih, iw, out.data_ptr(), _stream()), "mi_conv_run")
             return out
         x = _host_i8(x)
