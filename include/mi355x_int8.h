@@ -55,6 +55,13 @@ const char *mi_version(void);
 /* real multiplier -> (31-bit mantissa, left shift >= 0, right shift <= 0).
  * Replaces QuantizeRoundParameterWithDoublePrecision, NN/int8/quantize.c:39-51 (QuantizeMultiplier :113-161). */
 int mi_quantize_multiplier(double real_multiplier, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift);
+/* The alternative rounding the convolution wrappers select when a tensor's QuantParam.multiplier is 0
+ * (LK/base/convolution_base.cc:421-423,446-456).  Replaces QuantizeRoundParameterWithSinglePrecision,
+ * NN/int8/quantize.c:53-72, including its conversion of the double's value (not its bits) to uint32.  A provider
+ * kernel cannot see that field, so the create calls always use the double-precision method (the schema default);
+ * this entry point exists for callers that read the model themselves.  Domain 0 <= m < 2^32, else MI_PARAM_INVALID. */
+int mi_quantize_multiplier_single(double real_multiplier, int32_t *multiplier, int32_t *left_shift,
+                                  int32_t *right_shift);
 /* Clamp bounds of the fused activation in the quantised domain.
  * Replaces CalculateActivationRangeQuantized, NN/int8/quantize.c:78-94. */
 int mi_activation_range(int32_t act_type, int32_t out_zp, double out_scale, int32_t *act_min, int32_t *act_max);

@@ -392,6 +392,23 @@ int mi_quantize_multiplier(double real_multiplier, int32_t *multiplier, int32_t 
   return MI_OK;
 }
 
+int mi_quantize_multiplier_single(double real_multiplier, int32_t *multiplier, int32_t *left_shift,
+                                  int32_t *right_shift) {
+  if (multiplier == nullptr || left_shift == nullptr || right_shift == nullptr) return MI_NULL_PTR;
+  if (!(real_multiplier >= 0.0 && real_multiplier < 4294967296.0)) {
+    set_error("mi_quantize_multiplier_single: the multiplier must be in [0, 2^32)");
+    return MI_PARAM_INVALID;
+  }
+  // the reference converts the double's VALUE to uint32 here, so every multiplier below 1 gives
+  // (0x40000000, 0, -126); reproduced as it is
+  const uint32_t bits = (uint32_t)real_multiplier;
+  *multiplier = (int32_t)(((bits & 0x007FFFFFu) | 0x00800000u) << 7);
+  const int32_t shift = -(127 + 31 - 32 - (int32_t)(bits >> 23));
+  *left_shift = shift < 0 ? 0 : shift;
+  *right_shift = shift < 0 ? shift : 0;
+  return MI_OK;
+}
+
 int mi_activation_range(int32_t act_type, int32_t out_zp, double out_scale, int32_t *act_min, int32_t *act_max) {
   if (act_min == nullptr || act_max == nullptr) return MI_NULL_PTR;
   activation_range(act_type, out_zp, (float)out_scale, act_min, act_max);

@@ -12,7 +12,7 @@ MI_OK, MI_ERROR, MI_NULL_PTR, MI_PARAM_INVALID, MI_MEMORY_FAILED, MI_NOT_SUPPORT
 ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
 
 EXPORTS = [
-    "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_activation_range", "mi_requant_params",
+    "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_quantize_multiplier_single", "mi_activation_range", "mi_requant_params",
     "mi_multiply_by_quantized_multiplier",
     "mi_matmul_create", "mi_matmul_run", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
     "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_destroy",
@@ -81,6 +81,7 @@ def load():
     L.mi_last_error.restype = C.c_char_p
     L.mi_version.restype = C.c_char_p
     L.mi_quantize_multiplier.argtypes = [dbl, pi32, pi32, pi32]
+    L.mi_quantize_multiplier_single.argtypes = [dbl, pi32, pi32, pi32]
     L.mi_activation_range.argtypes = [i32, i32, dbl, pi32, pi32]
     L.mi_requant_params.argtypes = [dbl, C.POINTER(dbl), i32, dbl, pi32, pi32, pi32]
     L.mi_multiply_by_quantized_multiplier.argtypes = [i32, i32, i32, i32]

@@ -133,6 +133,22 @@ void orc_requant_params(double sx, const double *sw, int nfilt, double so, int32
   }
 }
 
+/* NN/int8/quantize.c:53-72.  The reference converts the double VALUE (not its bit pattern) to uint32, so every
+ * multiplier below 1 yields (0x40000000, 0, -126); kept as it is.  Domain: 0 <= m < 2^32. */
+void orc_round_param_single(double m, int32_t *mult, int32_t *ls, int32_t *rs) {
+  const uint32_t bits = (uint32_t)m;
+  *mult = (int32_t)(((bits & 0x007FFFFFu) | 0x00800000u) << 7);
+  int32_t shift = 127 + 31 - 32 - (int32_t)(bits >> 23);
+  shift = -shift;
+  if (shift < 0) {
+    *ls = 0;
+    *rs = shift;
+  } else {
+    *ls = shift;
+    *rs = 0;
+  }
+}
+
 static int32_t requant_to_i8(int32_t v, int32_t mult, int32_t ls, int32_t rs, int32_t zo, int32_t amin, int32_t amax) {
   int32_t y = wadd(orc_mul_by_quant_mult(v, mult, ls, rs), zo);
   if (y > amax) y = amax; /* MSMIN(maxi, value) first, then MSMAX(mini, value): NN/int8/matmul_int8.c:325-326 */

@@ -33,6 +33,7 @@ int32_t orc_mul_by_quant_mult(int32_t v, int32_t mult, int32_t ls, int32_t rs); 
 /* ---- quantize params (NN/int8/quantize.c) ---- */
 void orc_quantize_multiplier(double m, int32_t *mult, int32_t *shift);      /* :113-161 */
 void orc_round_param(double m, int32_t *mult, int32_t *ls, int32_t *rs);    /* :39-51 */
+void orc_round_param_single(double m, int32_t *mult, int32_t *ls, int32_t *rs); /* :53-72 */
 void orc_act_range(int relu, int relu6, int32_t zp, float scale, int32_t *mn, int32_t *mx); /* :76-94 */
 /* LK/int8/matmul_base_int8.cc:235-273 and LK/base/convolution_base.cc:416-427 */
 void orc_requant_params(double sx, const double *sw, int nfilt, double so, int32_t *mult, int32_t *ls, int32_t *rs);

@@ -172,6 +172,11 @@ class Oracle(_Base):
         self.lib.orc_round_param(C.c_double(m), C.byref(mult), C.byref(ls), C.byref(rs))
         return mult.value, ls.value, rs.value
 
+    def round_param_single(self, m):
+        mult, ls, rs = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        self.lib.orc_round_param_single(C.c_double(m), C.byref(mult), C.byref(ls), C.byref(rs))
+        return mult.value, ls.value, rs.value
+
     def act_range(self, relu, relu6, zp, scale):
         mn, mx = C.c_int32(0), C.c_int32(0)
         self.lib.orc_act_range(C.c_int(relu), C.c_int(relu6), C.c_int32(zp), C.c_float(scale), C.byref(mn),
@@ -242,6 +247,11 @@ class Reference(_Base):
     def round_param(self, m):
         mult, ls, rs = C.c_int32(0), C.c_int32(0), C.c_int32(0)
         self.lib.QuantizeRoundParameterWithDoublePrecision(C.c_double(m), C.byref(mult), C.byref(ls), C.byref(rs))
+        return mult.value, ls.value, rs.value
+
+    def round_param_single(self, m):
+        mult, ls, rs = C.c_int32(0), C.c_int32(0), C.c_int32(0)
+        self.lib.QuantizeRoundParameterWithSinglePrecision(C.c_double(m), C.byref(mult), C.byref(ls), C.byref(rs))
         return mult.value, ls.value, rs.value
 
     def act_range(self, relu, relu6, zp, scale):

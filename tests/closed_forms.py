@@ -70,6 +70,15 @@ def round_param(m):
     return (mult, 0, shift) if shift < 0 else (mult, shift, 0)
 
 
+def round_param_single(m):
+    """QuantizeRoundParameterWithSinglePrecision on 0 <= m < 2**32: the VALUE of m truncated to an integer plays the
+    role of the float's bit pattern (23-bit mantissa field, exponent field above it)."""
+    bits = int(m)  # truncation toward zero
+    mult = ((bits & 0x7FFFFF) | 0x800000) << 7
+    shift = -(126 - (bits >> 23))
+    return (mult, 0, shift) if shift < 0 else (mult, shift, 0)
+
+
 def round_half_away(x):
     """Vector round-half-away-from-zero on float64 (what C round() does)."""
     return np.sign(x) * np.floor(np.abs(x) + 0.5)

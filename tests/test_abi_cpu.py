@@ -41,6 +41,18 @@ def test_quantize_multiplier_matches_oracle(L, orc):
         assert (mult.value, ls.value, rs.value) == orc.round_param(m), m
 
 
+def test_quantize_multiplier_single_matches_oracle(L, orc):
+    rnd = random.Random(12)
+    vals = [0.0, 0.5, 1.0, 8388608.0, 8388613.0, 4294967295.0] + [rnd.uniform(0, 2.0 ** 32 - 1) for _ in range(2000)]
+    vals += [rnd.uniform(0, 3.0) for _ in range(500)]
+    for m in vals:
+        mult, ls, rs = C.c_int32(), C.c_int32(), C.c_int32()
+        assert L.mi_quantize_multiplier_single(m, C.byref(mult), C.byref(ls), C.byref(rs)) == 0
+        assert (mult.value, ls.value, rs.value) == orc.round_param_single(m), m
+    for bad in (-1.0, 2.0 ** 32, float("nan")):
+        assert L.mi_quantize_multiplier_single(bad, C.byref(mult), C.byref(ls), C.byref(rs)) == -3
+
+
 def test_requant_params_and_act_range_match_oracle(L, orc):
     rng = np.random.default_rng(12)
     sw = rng.uniform(1e-4, 1e-2, 1000)

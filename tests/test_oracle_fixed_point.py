@@ -77,6 +77,27 @@ def test_quantize_multiplier_exact(orc):
         assert orc.round_param(m) == cf.round_param(m)
 
 
+def test_round_param_single_known_answers(orc):
+    """Hand-computed: the mantissa field is the low 23 bits of trunc(m), the exponent field the bits above."""
+    assert orc.round_param_single(0.0) == (0x40000000, 0, -126)
+    assert orc.round_param_single(0.75) == (0x40000000, 0, -126)       # any multiplier below 1 truncates to 0
+    assert orc.round_param_single(1.0) == (0x40000080, 0, -126)        # mantissa field 1
+    assert orc.round_param_single(8388607.9) == (0x7FFFFF80, 0, -126)  # mantissa field all ones
+    assert orc.round_param_single(8388608.0) == (0x40000000, 0, -125)  # 2^23: exponent field 1
+    assert orc.round_param_single(126.0 * 8388608.0) == (0x40000000, 0, 0)
+    assert orc.round_param_single(127.0 * 8388608.0 + 3.0) == (0x40000180, 1, 0)
+    rnd = random.Random(4)
+    for _ in range(20000):
+        m = rnd.uniform(0.0, 2.0 ** 32 - 1.0)
+        assert orc.round_param_single(m) == cf.round_param_single(m), m
+
+
+def test_round_param_single_vs_nnacl(orc, ref):
+    rnd = random.Random(5)
+    for m in [0.0, 0.3, 1.0, 8388608.0, 4294967295.0] + [rnd.uniform(0.0, 2.0 ** 32 - 1.0) for _ in range(20000)]:
+        assert orc.round_param_single(m) == ref.round_param_single(m), m
+
+
 def test_quantize_multiplier_value(orc):
     # mult * 2^(shift-31) reproduces m to 31 bits
     for m in [0.0003, 0.02 * 0.005 / 0.05, 0.7, 1.0, 123.456]:
