@@ -171,6 +171,17 @@ int mi_dynquant_get_params(mi_dynquant *h, void *stream, mi_dq_params *params_ho
 /* Device address of the mi_dq_params block of the last run. */
 const mi_dq_params *mi_dynquant_device_params(const mi_dynquant *h);
 int mi_dynquant_run_host(mi_dynquant *h, const float *x_host, int64_t n, int8_t *q_host, mi_dq_params *params_host);
+/* DynamicQuant with preferred axes (per-channel activation scales; replaces the axis_num_ != 0 branch of
+ * DynamicQuantCPUKernel: ReSize LK/int8/dynamic_quant.cc:59-94, CalculateMinMax :118-143,
+ * CalculatePerChannelScaleZp :188-218, QuantData :236-246).  The tensor is given in the layout the reference works
+ * on after moving the preferred axes to the front: `segments` contiguous runs of `unit` elements, one
+ * {scale, zero point} each; for a MatMul activation [.., rows, K] that is the tensor as it stands (segments = rows,
+ * unit = K, insert_quant_node_manager.cc:138-160).  Layouts that need the transposition stay with the builtin kernel.
+ * params_dev / params_host: `segments` entries. */
+int mi_dynquant_run_segments(mi_dynquant *h, const float *x_dev, int64_t segments, int64_t unit, int8_t *q_dev,
+                             mi_dq_params *params_dev, void *stream);
+int mi_dynquant_run_segments_host(mi_dynquant *h, const float *x_host, int64_t segments, int64_t unit,
+                                  int8_t *q_host, mi_dq_params *params_host);
 void mi_dynquant_destroy(mi_dynquant *h);
 
 /* ---- dynamic-quant MatMul (int8 x int8 -> fp32) -------------------------------------------------------------- */
@@ -198,6 +209,14 @@ int mi_dynmm_run_chained(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const m
                          float *c_dev, void *stream);
 int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in_scale, int32_t in_zp,
                       float *c_host);
+/* One input scale per row (input_per_channel_, LK/int8/matmul_dynamic_base_int8.cc:152-171; NN/int8/
+ * dynamic_matmul_int8.c:126-128): row r uses row_params_dev[r].scale_f; the zero point is that of the first row
+ * (LK/int8/matmul_dynamic_int8.cc:61), as in the reference, whose converter only produces symmetric per-row
+ * quantisation.  row_params_dev is what mi_dynquant_run_segments wrote. */
+int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_dq_params *row_params_dev,
+                      float *c_dev, void *stream);
+int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
+                           float *c_host);
 void mi_dynmm_destroy(mi_dynmm *h);
 
 /* ---- measurement aids (no counterpart in the reference) ---------------------------------------------------------

@@ -321,14 +321,14 @@ struct mi_conv {
 
 struct mi_dynquant {
   int symmetric = 0;
-  DevBuf partials, params, h_in, h_out;
+  DevBuf partials, params, h_in, h_out, h_params;
 };
 
 struct mi_dynmm {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0, act = 0;
   int32_t zw0 = 0;
   bool has_bias = false;
-  DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out;
+  DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out, h_params;
 };
 
 extern "C" {
@@ -729,6 +729,44 @@ int mi_dynquant_get_params(mi_dynquant *h, void *stream, mi_dq_params *params_ho
   return MI_OK;
 }
 
+int mi_dynquant_run_segments(mi_dynquant *h, const float *x_dev, int64_t segments, int64_t unit, int8_t *q_dev,
+                             mi_dq_params *params_dev, void *stream) {
+  if (h == nullptr || x_dev == nullptr || q_dev == nullptr || params_dev == nullptr) {
+    set_error("mi_dynquant_run_segments: null argument");
+    return MI_NULL_PTR;
+  }
+  if (segments < 1 || unit < 1) {
+    set_error("mi_dynquant_run_segments: segments and unit must be positive");
+    return MI_PARAM_INVALID;
+  }
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  return launch_dynquant_segments(x_dev, segments, unit, h->symmetric, params_dev, q_dev,
+                                  static_cast<hipStream_t>(stream));
+}
+
+int mi_dynquant_run_segments_host(mi_dynquant *h, const float *x_host, int64_t segments, int64_t unit, int8_t *q_host,
+                                  mi_dq_params *params_host) {
+  if (h == nullptr || x_host == nullptr || q_host == nullptr || params_host == nullptr) {
+    set_error("mi_dynquant_run_segments_host: null argument");
+    return MI_NULL_PTR;
+  }
+  if (segments < 1 || unit < 1) return MI_PARAM_INVALID;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  const size_t n = (size_t)segments * (size_t)unit;
+  if ((rc = h->h_in.ensure(n * 4 + 16)) != MI_OK || (rc = h->h_out.ensure(n + 16)) != MI_OK ||
+      (rc = h->h_params.ensure(sizeof(mi_dq_params) * (size_t)segments)) != MI_OK)
+    return rc;
+  MI_HIP_CHECK(hipMemcpy(h->h_in.p, x_host, n * 4, hipMemcpyHostToDevice));
+  rc = mi_dynquant_run_segments(h, static_cast<const float *>(h->h_in.p), segments, unit,
+                                static_cast<int8_t *>(h->h_out.p), static_cast<mi_dq_params *>(h->h_params.p), nullptr);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(q_host, h->h_out.p, n, hipMemcpyDeviceToHost));
+  MI_HIP_CHECK(hipMemcpy(params_host, h->h_params.p, sizeof(mi_dq_params) * (size_t)segments, hipMemcpyDeviceToHost));
+  return MI_OK;
+}
+
 const mi_dq_params *mi_dynquant_device_params(const mi_dynquant *h) {
   return h == nullptr ? nullptr : static_cast<const mi_dq_params *>(h->params.p);
 }
@@ -756,6 +794,7 @@ void mi_dynquant_destroy(mi_dynquant *h) {
   h->params.release();
   h->h_in.release();
   h->h_out.release();
+  h->h_params.release();
   delete h;
 }
 
@@ -809,7 +848,7 @@ int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const flo
 }
 
 static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float sx, int32_t zx,
-                          const mi_dq_params *qp_dev, float *c_dev, hipStream_t s) {
+                          const mi_dq_params *qp_dev, float *c_dev, hipStream_t s, bool per_row = false) {
   if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
     set_error("mi_dynmm_run: null argument");
     return MI_NULL_PTR;
@@ -830,6 +869,7 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   dq.sx = sx;
   dq.zx = zx;
   dq.zw0 = h->zw0;
+  dq.per_row = per_row ? 1 : 0;
   dq.deep = h->k;
   dq.act = h->act;
   const WeightView w{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw, nullptr};
@@ -854,6 +894,45 @@ int mi_dynmm_run_chained(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const m
     return MI_NULL_PTR;
   }
   return dynmm_run_impl(h, a_dev, rows, 0.0f, 0, params_dev, c_dev, static_cast<hipStream_t>(stream));
+}
+
+int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_dq_params *row_params_dev, float *c_dev,
+                      void *stream) {
+  if (row_params_dev == nullptr) {
+    set_error("mi_dynmm_run_rows: row_params_dev is null");
+    return MI_NULL_PTR;
+  }
+  return dynmm_run_impl(h, a_dev, rows, 0.0f, 0, row_params_dev, c_dev, static_cast<hipStream_t>(stream), true);
+}
+
+int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
+                           float *c_host) {
+  if (h == nullptr || a_host == nullptr || c_host == nullptr || in_scales == nullptr) {
+    set_error("mi_dynmm_run_rows_host: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) return MI_PARAM_INVALID;
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  const size_t in_bytes = (size_t)rows * h->k, out_bytes = (size_t)rows * h->n * sizeof(float);
+  if ((rc = h->h_in.ensure(in_bytes)) != MI_OK || (rc = h->h_out.ensure(out_bytes)) != MI_OK ||
+      (rc = h->h_params.ensure(sizeof(mi_dq_params) * (size_t)rows)) != MI_OK)
+    return rc;
+  std::vector<mi_dq_params> p((size_t)rows);
+  for (int r = 0; r < rows; ++r) {
+    p[r].scale = in_scales[r];
+    p[r].scale_f = (float)in_scales[r];  // the wrapper narrows every input scale to float (matmul_dynamic_base_int8.cc:168-171)
+    p[r].zero_point = in_zp;
+    p[r].real_min = p[r].real_max = 0.0f;
+  }
+  MI_HIP_CHECK(hipMemcpy(h->h_params.p, p.data(), sizeof(mi_dq_params) * (size_t)rows, hipMemcpyHostToDevice));
+  MI_HIP_CHECK(hipMemcpy(h->h_in.p, a_host, in_bytes, hipMemcpyHostToDevice));
+  rc = mi_dynmm_run_rows(h, static_cast<const int8_t *>(h->h_in.p), rows,
+                         static_cast<const mi_dq_params *>(h->h_params.p), static_cast<float *>(h->h_out.p), nullptr);
+  if (rc != MI_OK) return rc;
+  MI_HIP_CHECK(hipMemcpy(c_host, h->h_out.p, out_bytes, hipMemcpyDeviceToHost));
+  return MI_OK;
 }
 
 int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in_scale, int32_t in_zp, float *c_host) {
@@ -885,6 +964,7 @@ void mi_dynmm_destroy(mi_dynmm *h) {
   h->c_ws.release();
   h->h_in.release();
   h->h_out.release();
+  h->h_params.release();
   delete h;
 }
 

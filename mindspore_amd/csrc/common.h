@@ -51,6 +51,7 @@ struct DequantParams {
   int32_t zw0;
   int32_t deep;  // true K
   int32_t act;
+  int32_t per_row;  // input scale of row r is qp_dev[r].scale_f; the zero point is qp_dev[0].zero_point
 };
 
 // Packed weights: n_pad rows (output channels) of k_pad contraction bytes, zero filled past K, with row stride ldw.
@@ -114,5 +115,8 @@ int launch_mfma_rate(const void *operands, int iters, int workgroups, unsigned l
 constexpr int kDqMaxBlocks = 1024;
 int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, mi_dq_params *params, int8_t *q,
                     hipStream_t stream);
+// One {scale, zero point} per contiguous run of `unit` elements; params has `segments` entries.
+int launch_dynquant_segments(const float *x, int64_t segments, int64_t unit, int symmetric, mi_dq_params *params,
+                             int8_t *q, hipStream_t stream);
 
 }  // namespace mi

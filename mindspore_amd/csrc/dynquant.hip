@@ -178,6 +178,91 @@ __global__ __launch_bounds__(kDqThreads) void dq_quantize_kernel(const float *__
   }
 }
 
+// DynamicQuant with preferred axes (one scale / zero point per segment): after the preferred axes lead, the tensor is
+// `segments` contiguous runs of `unit` elements (DynamicQuantCPUKernel::ReSize / CalculateMinMax / QuantData,
+// mindspore/lite/src/litert/kernel/cpu/int8/dynamic_quant.cc:59-94,118-143,236-246; scale and zero point per segment
+// as CalculatePerChannelScaleZp :188-218, the same formulas as the per-tensor case).  One wave per segment: first
+// sweep min/max, second sweep (the run is L1/L2 resident by then) quantises.
+__global__ __launch_bounds__(kDqThreads) void dq_segments_kernel(const float *__restrict__ x, int64_t segments,
+                                                                 int64_t unit, int symmetric,
+                                                                 mi_dq_params *__restrict__ params,
+                                                                 int8_t *__restrict__ q) {
+  const int lane = threadIdx.x & 63;
+  const int64_t seg = (int64_t)blockIdx.x * (kDqThreads / 64) + (threadIdx.x >> 6);
+  if (seg >= segments) return;
+  const float *xs = x + seg * unit;
+  int8_t *qs = q + seg * unit;
+  const bool vec = ((reinterpret_cast<uintptr_t>(xs) & 15) == 0) && ((reinterpret_cast<uintptr_t>(qs) & 3) == 0);
+  const int64_t n4 = vec ? unit >> 2 : 0;
+  float lo = FLT_MAX, hi = -FLT_MAX;
+  const v4f *x4 = reinterpret_cast<const v4f *>(xs);
+  for (int64_t i = lane; i < n4; i += 64) {
+    const v4f v = x4[i];
+    upd(v.x, lo, hi);
+    upd(v.y, lo, hi);
+    upd(v.z, lo, hi);
+    upd(v.w, lo, hi);
+  }
+  for (int64_t i = (n4 << 2) + lane; i < unit; i += 64) upd(xs[i], lo, hi);
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float l2 = __shfl_xor(lo, off), h2 = __shfl_xor(hi, off);
+    lo = l2 < lo ? l2 : lo;
+    hi = h2 > hi ? h2 : hi;
+  }
+  float scale_f;
+  double scale_d;
+  int zp = 0;
+  if (!symmetric) {
+    float range = __fsub_rn(hi, lo);
+    if (range <= 0) range = 0.01f;
+    scale_f = __fdiv_rn(range, 255.0f);
+    scale_d = (double)scale_f;
+    zp = double_to_int_x86(round(-128.0 - (double)lo / scale_d));
+  } else {
+    const float a = fabsf(hi), b = fabsf(lo);
+    const float big = (a < b) ? b : a;
+    scale_f = __fdiv_rn(__fmul_rn(2.0f, big), 254.0f);
+    scale_d = (double)scale_f;
+  }
+  if (lane == 0) {
+    mi_dq_params *p = params + seg;
+    p->scale = scale_d;
+    p->scale_f = scale_f;
+    p->zero_point = zp;
+    p->real_min = lo;
+    p->real_max = hi;
+  }
+  const float inv = __fdiv_rn(1.0f, scale_f);
+  const float zpf = (float)zp;
+  for (int64_t i = lane; i < n4; i += 64) {
+    const v4f v = x4[i];
+    union {
+      int w;
+      int8_t b[4];
+    } u;
+    u.b[0] = quant_one(v.x, inv, zpf);
+    u.b[1] = quant_one(v.y, inv, zpf);
+    u.b[2] = quant_one(v.z, inv, zpf);
+    u.b[3] = quant_one(v.w, inv, zpf);
+    *reinterpret_cast<int *>(qs + 4 * i) = u.w;
+  }
+  for (int64_t i = (n4 << 2) + lane; i < unit; i += 64) qs[i] = quant_one(xs[i], inv, zpf);
+}
+
+int launch_dynquant_segments(const float *x, int64_t segments, int64_t unit, int symmetric, mi_dq_params *params,
+                             int8_t *q, hipStream_t stream) {
+  const int64_t blocks = (segments + kDqThreads / 64 - 1) / (kDqThreads / 64);
+  if (blocks > 0x7fffffff) {
+    set_error("dynquant: too many segments");
+    return MI_PARAM_INVALID;
+  }
+  hipLaunchKernelGGL(dq_segments_kernel, dim3((unsigned)blocks), dim3(kDqThreads), 0, stream, x, segments, unit,
+                     symmetric, params, q);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, mi_dq_params *params, int8_t *q,
                     hipStream_t stream) {
   const int64_t per_block = (int64_t)kDqThreads * kDqElemsPerThread;

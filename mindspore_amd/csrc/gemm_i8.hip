@@ -231,6 +231,14 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
       zx = dq.qp_dev->zero_point;
     }
     const uint32_t kzz = (uint32_t)dq.deep * (uint32_t)zx * (uint32_t)dq.zw0;
+    // input_per_channel_: one input scale per row (NN/int8/dynamic_matmul_int8.c:126-128)
+    float sxr[TM];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      int m = m_w + j * 32 + r;
+      m = m < g.m ? m : g.m - 1;
+      sxr[j] = dq.per_row ? dq.qp_dev[m].scale_f : sx;
+    }
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
 #pragma unroll
@@ -241,13 +249,9 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         const v4f ws4 = *reinterpret_cast<const v4f *>(pl);
         const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
         const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
-        float ms[4];
         uint32_t corr[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          ms[e] = __fmul_rn(sx, ws4[e]);
-          corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e];
-        }
+        for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e];
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
           const int m = m_w + j * 32 + r;
@@ -256,7 +260,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
           for (int e = 0; e < 4; ++e) {
             uint32_t v = (uint32_t)acc[i][j][q * 4 + e] + corr[e];
             if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
-            float d = __fmul_rn(ms[e], (float)(int32_t)v);
+            float d = __fmul_rn(__fmul_rn(sxr[j], ws4[e]), (float)(int32_t)v);
             if (dq.bias != nullptr) d = __fadd_rn(d, b4[e]);
             if (dq.act == MI_ACT_RELU) {
               d = (0.0f > d) ? 0.0f : d;

@@ -231,6 +231,33 @@ class DynamicQuantKernel(_Handle):
     def device_params(self):
         return _lib.load().mi_dynquant_device_params(self._h)
 
+    def run_rows(self, x):
+        """Per-channel activation scales as the converter asks for them for a MatMul input (prefer_axes = every axis
+        but the last): x [..., K] -> (q, [QuantParam per row]).  numpy in: host path, list of QuantParam out.
+        CUDA tensor in: device path, returns (q, params) with params a CUDA uint8 tensor of `rows` parameter
+        blocks to hand to MatmulDynamicInt8Kernel.run(..., row_params=params)."""
+        L = _lib.load()
+        unit = x.shape[-1]
+        if _is_torch(x):
+            import torch
+            if x.dtype != torch.float32 or not x.is_cuda or not x.is_contiguous():
+                raise ValueError("expected a contiguous CUDA float32 tensor")
+            rows = x.numel() // unit
+            q = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+            params = torch.empty(rows * C.sizeof(_lib.DqParams), dtype=torch.uint8, device=x.device)
+            _lib.check(L.mi_dynquant_run_segments(self._h, x.data_ptr(), rows, unit, q.data_ptr(), params.data_ptr(),
+                                                  _stream()), "mi_dynquant_run_segments")
+            return q, params
+        x = np.ascontiguousarray(x)
+        if x.dtype != np.float32:
+            raise TypeError("DynamicQuant needs a float32 input")
+        rows = x.size // unit
+        q = np.empty(x.shape, np.int8)
+        p = (_lib.DqParams * rows)()
+        _lib.check(L.mi_dynquant_run_segments_host(self._h, x.ctypes.data, rows, unit, q.ctypes.data, p),
+                   "mi_dynquant_run_segments_host")
+        return q, [QuantParam(e.scale, e.zero_point) for e in p]
+
 
 class MatmulDynamicInt8Kernel(_Handle):
     """Dynamic-quant MatMul: int8 activations (scale / zero point supplied at every run) x int8 weights -> fp32."""
@@ -252,7 +279,10 @@ class MatmulDynamicInt8Kernel(_Handle):
         _lib.check(L.mi_dynmm_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                      C.byref(self._h)), "mi_dynmm_create")
 
-    def run(self, a, in_quant=None, params_dev=None):
+    def run(self, a, in_quant=None, params_dev=None, row_params=None):
+        """in_quant: one QuantParam (per-tensor input) or a list with one per row (per-channel input; the zero point
+        used is the first one, as in the reference).  Device path alternatives: params_dev (address of the block a
+        DynamicQuantKernel.run left on the device) or row_params (the tensor DynamicQuantKernel.run_rows returned)."""
         L = _lib.load()
         if _is_torch(a):
             import torch
@@ -260,7 +290,12 @@ class MatmulDynamicInt8Kernel(_Handle):
                 raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % self.k)
             rows = a.numel() // self.k
             out = torch.empty(a.shape[:-1] + (self.n,), dtype=torch.float32, device=a.device)
-            if params_dev is not None:
+            if row_params is not None:
+                if row_params.numel() != rows * C.sizeof(_lib.DqParams):
+                    raise ValueError("row_params does not hold %d parameter blocks" % rows)
+                _lib.check(L.mi_dynmm_run_rows(self._h, a.data_ptr(), rows, row_params.data_ptr(), out.data_ptr(),
+                                               _stream()), "mi_dynmm_run_rows")
+            elif params_dev is not None:
                 _lib.check(L.mi_dynmm_run_chained(self._h, a.data_ptr(), rows, params_dev, out.data_ptr(), _stream()),
                            "mi_dynmm_run_chained")
             else:
@@ -270,6 +305,14 @@ class MatmulDynamicInt8Kernel(_Handle):
         a = _host_i8(a)
         rows = a.size // self.k
         out = np.empty(a.shape[:-1] + (self.n,), np.float32)
+        if not isinstance(in_quant, QuantParam):  # a sequence: one QuantParam per row
+            in_quant = list(in_quant)
+            if len(in_quant) != rows:
+                raise ValueError("need one input QuantParam per row (%d), got %d" % (rows, len(in_quant)))
+            scales = (C.c_double * rows)(*[float(qp.scale) for qp in in_quant])
+            _lib.check(L.mi_dynmm_run_rows_host(self._h, a.ctypes.data, rows, scales, int(in_quant[0].zero_point),
+                                                out.ctypes.data), "mi_dynmm_run_rows_host")
+            return out
         _lib.check(L.mi_dynmm_run_host(self._h, a.ctypes.data, rows, float(in_quant.scale), int(in_quant.zero_point),
                                        out.ctypes.data), "mi_dynmm_run_host")
         return out

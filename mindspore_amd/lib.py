@@ -17,8 +17,9 @@ EXPORTS = [
     "mi_matmul_create", "mi_matmul_run", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
     "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_destroy",
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
-    "mi_dynquant_run_host", "mi_dynquant_destroy",
-    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_destroy",
+    "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
+    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host",
+    "mi_dynmm_destroy",
     "mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate",
 ]
 
@@ -105,12 +106,16 @@ def load():
     L.mi_dynquant_device_params.argtypes = [vp]
     L.mi_dynquant_device_params.restype = vp
     L.mi_dynquant_run_host.argtypes = [vp, vp, i64, vp, C.POINTER(DqParams)]
+    L.mi_dynquant_run_segments.argtypes = [vp, vp, i64, i64, vp, vp, vp]
+    L.mi_dynquant_run_segments_host.argtypes = [vp, vp, i64, i64, vp, vp]
     L.mi_dynquant_destroy.argtypes = [vp]
     L.mi_dynquant_destroy.restype = None
     L.mi_dynmm_create.argtypes = [C.POINTER(DynmmDesc), vp, vp, C.POINTER(vp)]
     L.mi_dynmm_run.argtypes = [vp, vp, i32, dbl, i32, vp, vp]
     L.mi_dynmm_run_chained.argtypes = [vp, vp, i32, vp, vp, vp]
     L.mi_dynmm_run_host.argtypes = [vp, vp, i32, dbl, i32, vp]
+    L.mi_dynmm_run_rows.argtypes = [vp, vp, i32, vp, vp, vp]
+    L.mi_dynmm_run_rows_host.argtypes = [vp, vp, i32, C.POINTER(dbl), i32, vp]
     L.mi_dynmm_destroy.argtypes = [vp]
     L.mi_dynmm_destroy.restype = None
     L.mi_diag_stream_read.argtypes = [vp, i64, vp]

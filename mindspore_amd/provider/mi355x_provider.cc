@@ -13,7 +13,7 @@
 // benchmark tool with --provider=mi355x (it leaves the provider device empty, hence the second registration under "").
 //
 // Tensors are host-resident (arch "CPU": the kernels live in the ordinary CPU subgraph), so Execute() uses the
-// *_run_host entry points, which stage through pinned buffers.  A creator returns nullptr for everything the library
+// *_run_host entry points, which copy into and out of device buffers the handle owns.  A creator returns nullptr for everything the library
 // does not reproduce bit-exactly; the scheduler then falls back to the builtin CPU kernel
 // (mindspore/lite/src/litert/scheduler.cc:1173-1177).
 #include <memory>
@@ -102,8 +102,16 @@ class MatmulKernel : public kernel::Kernel {
     if (full_ != nullptr) return ToStatus(mi_matmul_run_host(full_, a, rows, static_cast<int8_t *>(c)));
     // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
     // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
-    const auto iq = inputs_[0].QuantParams().front();
-    return ToStatus(mi_dynmm_run_host(dyn_, a, rows, iq.scale, iq.zero_point, static_cast<float *>(c)));
+    const auto iqs = inputs_[0].QuantParams();
+    if (iqs.size() == 1) {
+      return ToStatus(mi_dynmm_run_host(dyn_, a, rows, iqs[0].scale, iqs[0].zero_point, static_cast<float *>(c)));
+    }
+    // one scale per row (input_per_channel_, :152-171); the zero point used is the first one (matmul_dynamic_int8.cc:61)
+    if (iqs.size() != static_cast<size_t>(rows)) return kLiteError;
+    std::vector<double> scales(iqs.size());
+    for (size_t i = 0; i < iqs.size(); ++i) scales[i] = iqs[i].scale;
+    return ToStatus(
+      mi_dynmm_run_rows_host(dyn_, a, rows, scales.data(), iqs[0].zero_point, static_cast<float *>(c)));
   }
 
  private:
@@ -132,7 +140,8 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
   const bool out_i8 = out[0].DataType() == DataType::kNumberTypeInt8;
   const bool out_f32 = out[0].DataType() == DataType::kNumberTypeFloat32;
   if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || w.Shape().size() != 2) return nullptr;
-  if (!(out_i8 || out_f32) || !PerTensor(in[0]) || (out_i8 && !PerTensor(out[0]))) return nullptr;
+  // full quant needs per-tensor activations; the dynamic MatMul also takes one input scale per row
+  if (!(out_i8 || out_f32) || (out_i8 && (!PerTensor(in[0]) || !PerTensor(out[0])))) return nullptr;
   if (act != MI_ACT_NONE && act != MI_ACT_RELU && act != MI_ACT_RELU6) return nullptr;
   if (in.size() > kBiasIndex) {
     const auto want = out_i8 ? DataType::kNumberTypeInt32 : DataType::kNumberTypeFloat32;
@@ -244,6 +253,7 @@ class DynamicQuantKernel : public kernel::Kernel {
 
   int Prepare() override {
     const auto *p = primitive_->value_as_DynamicQuant();
+    per_row_ = p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0;
     return ToStatus(mi_dynquant_create(p->symmetric() ? 1 : 0, &dq_));
   }
   int ReSize() override { return kSuccess; }
@@ -251,6 +261,22 @@ class DynamicQuantKernel : public kernel::Kernel {
     const auto *x = static_cast<const float *>(inputs_[0].Data().get());
     auto *q = static_cast<int8_t *>(outputs_[0].MutableData());
     if (x == nullptr || q == nullptr) return kLiteNullptr;
+    if (per_row_) {  // the creator admitted only "every axis but the last": one run per row of the last axis
+      const int64_t unit = inputs_[0].Shape().back();
+      const int64_t segments = inputs_[0].ElementNum() / unit;
+      std::vector<mi_dq_params> ps(static_cast<size_t>(segments));
+      if (mi_dynquant_run_segments_host(dq_, x, segments, unit, q, ps.data()) != MI_OK) return kLiteError;
+      std::vector<QuantParam> qps(ps.size());
+      for (size_t i = 0; i < ps.size(); ++i) {
+        qps[i].bit_num = 8;
+        qps[i].scale = ps[i].scale;
+        qps[i].zero_point = ps[i].zero_point;
+        qps[i].min = ps[i].real_min;
+        qps[i].max = ps[i].real_max;
+      }
+      outputs_[0].SetQuantParams(qps);
+      return kSuccess;
+    }
     mi_dq_params p{};
     const int rc = mi_dynquant_run_host(dq_, x, inputs_[0].ElementNum(), q, &p);
     if (rc != MI_OK) return kLiteError;
@@ -267,14 +293,24 @@ class DynamicQuantKernel : public kernel::Kernel {
 
  private:
   mi_dynquant *dq_ = nullptr;
+  bool per_row_ = false;
 };
 
 std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
                                                     const schema::Primitive *prim, const Context *ctx) {
   if (!LibraryReady() || in.size() != 1 || out.size() != 1 || prim == nullptr) return nullptr;
   const auto *p = prim->value_as_DynamicQuant();
-  if (p == nullptr || p->activation_channel() || (p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0)) {
-    return nullptr;  // per-channel activation scales stay with the builtin kernel
+  if (p == nullptr) return nullptr;
+  if (p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0) {
+    // per-channel activation scales: taken when the preferred axes are exactly the leading rank-1 axes (what the
+    // converter emits for a MatMul input without transpose_a, insert_quant_node_manager.cc:138-160), so that no
+    // transposition is involved; everything else stays with the builtin kernel
+    const size_t rank = in[0].Shape().size();
+    if (rank < 2 || p->prefer_axes()->size() != rank - 1) return nullptr;
+    for (size_t i = 0; i + 1 < rank; ++i) {
+      const int axis = p->prefer_axes()->Get(i);
+      if ((axis < 0 ? axis + static_cast<int>(rank) : axis) != static_cast<int>(i)) return nullptr;
+    }
   }
   if (p->dst_type() != static_cast<int64_t>(DataType::kNumberTypeInt8)) return nullptr;
   if (in[0].DataType() != DataType::kNumberTypeFloat32 || out[0].DataType() != DataType::kNumberTypeInt8) {

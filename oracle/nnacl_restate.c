@@ -410,12 +410,47 @@ int orc_dynamic_quant(const float *x, int64_t n, int symmetric, int8_t *q, doubl
  * value = sum(a*b) - zw*sum(a) - zx*sum(b) + K*zx*zw in wrapping int32 over the true K; the per-channel case still
  * uses the single zero point zw[0] (matmul_dynamic_int8.cc:52).  dst = (sx*sw) * (float)value, then + bias, then
  * the activation -- three separately rounded float operations. */
+/* DynamicQuantCPUKernel with prefer_axes (LK/int8/dynamic_quant.cc:59-94 ReSize, :118-143 CalculateMinMax, :188-218
+ * CalculatePerChannelScaleZp, :236-246 QuantData): after the preferred axes lead, the tensor is `segments` contiguous
+ * runs of `unit` elements, each with its own min/max, scale and zero point.  The scale / zero-point formulas are
+ * those of the per-tensor case. */
+int orc_dynamic_quant_segments(const float *x, int64_t segments, int64_t unit, int symmetric, int8_t *q,
+                               double *scales, int32_t *zps) {
+  if (segments < 1 || unit < 1) return -1;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t s = 0; s < segments; ++s) {
+    float mn = FLT_MAX, mx = -FLT_MAX;
+    orc_minmax_fp32(x + s * unit, unit, &mn, &mx);
+    orc_dynquant_params(mn, mx, symmetric, &scales[s], &zps[s]);
+    orc_quantize_fp32_int8(x + s * unit, q + s * unit, (float)scales[s], zps[s], unit);
+  }
+  return 0;
+}
+
+static int dyn_mm(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k, int b_transpose,
+                  float fsx, const float *sx_rows, int zx, const double *sw, const int32_t *zw, int nfilt,
+                  int act_type);
+
 int orc_dynamic_matmul(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
                        int b_transpose, double sx, int zx, const double *sw, const int32_t *zw, int nfilt,
                        int act_type) {
+  return dyn_mm(a, w, bias, c, m, n, k, b_transpose, (float)sx, NULL, zx, sw, zw, nfilt, act_type);
+}
+
+/* input_per_channel_: one input scale per row, a single input zero point -- the first one
+ * (LK/int8/matmul_dynamic_int8.cc:61-62, NN/int8/dynamic_matmul_int8.c:126-128) */
+int orc_dynamic_matmul_rows(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
+                            int b_transpose, const float *sx_rows, int zx, const double *sw, const int32_t *zw,
+                            int nfilt, int act_type) {
+  if (sx_rows == NULL) return -1;
+  return dyn_mm(a, w, bias, c, m, n, k, b_transpose, 0.0f, sx_rows, zx, sw, zw, nfilt, act_type);
+}
+
+static int dyn_mm(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k, int b_transpose,
+                  float fsx, const float *sx_rows, int zx, const double *sw, const int32_t *zw, int nfilt,
+                  int act_type) {
   if (nfilt < 1 || (nfilt > 1 && nfilt != n)) return -1;
   const int peroc = nfilt > 1;
-  const float fsx = (float)sx;
   const int32_t z = zw[0];
   int8_t *wt = NULL;
   const int8_t *wnk = w;
@@ -444,7 +479,7 @@ int orc_dynamic_matmul(const int8_t *a, const int8_t *w, const float *bias, floa
       for (int kk = 0; kk < k; ++kk) s0 += (int32_t)ar[kk] * (int32_t)wr[kk];
       int32_t s1 = wmul(z, asum), s2 = wmul(zx, wsum[cc]), s3 = wmul(wmul(k, zx), z);
       int32_t value = wadd(wsub(wsub(s0, s1), s2), s3);
-      volatile float ms = fsx * (float)sw[peroc ? cc : 0];
+      volatile float ms = (sx_rows ? sx_rows[r] : fsx) * (float)sw[peroc ? cc : 0];
       volatile float d = ms * (float)value;
       if (bias) d = d + bias[cc];
       float o = d;

@@ -68,6 +68,11 @@ void orc_quantize_fp32_int8(const float *x, int8_t *q, float scale, int32_t zp, 
 int orc_dynamic_quant(const float *x, int64_t n, int symmetric, int8_t *q, double *scale, int32_t *zp);
 
 /* ---- dynamic-quant MatMul (LK/int8/matmul_dynamic_int8.cc + NN/int8/dynamic_matmul_int8.c:99-143) ---- */
+int orc_dynamic_quant_segments(const float *x, int64_t segments, int64_t unit, int symmetric, int8_t *q,
+                               double *scales, int32_t *zps);
+int orc_dynamic_matmul_rows(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
+                            int b_transpose, const float *sx_rows, int zx, const double *sw, const int32_t *zw,
+                            int nfilt, int act_type);
 int orc_dynamic_matmul(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
                        int b_transpose, double sx, int zx, const double *sw, const int32_t *zw, int nfilt,
                        int act_type);

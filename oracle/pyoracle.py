@@ -120,6 +120,35 @@ class _Base:
         self._done(rc, "dynamic_quant")
         return q, scale.value, zp.value
 
+    def dynamic_quant_segments(self, x, symmetric=False):
+        """x: [segments, unit] fp32 (the layout after the preferred axes lead) -> (q, scales[segments], zps)."""
+        x = _f32(x)
+        segments, unit = x.shape
+        q = np.empty(x.shape, np.int8)
+        scales, zps = np.empty(segments, np.float64), np.empty(segments, np.int32)
+        f = getattr(self.lib, self.prefix + "dynamic_quant_segments")
+        f.restype = C.c_int
+        it = C.c_int if self.extra else C.c_int64
+        rc = f(_p(x, C.c_float), it(segments), it(unit), C.c_int(1 if symmetric else 0), _p(q, C.c_int8),
+               _p(scales, C.c_double), _p(zps, C.c_int32), *self._tail())
+        self._done(rc, "dynamic_quant_segments")
+        return q, scales, zps
+
+    def dynamic_matmul_rows(self, a, w, bias, sx_rows, zx, sw, zw, act=ACT_NONE, b_transpose=True):
+        """Per-row input scales (float32 [rows]), one input zero point."""
+        a, w, bias, sx_rows = _i8(a), _i8(w), _f32(bias), _f32(sx_rows)
+        m, k = a.shape
+        n = w.shape[0] if b_transpose else w.shape[1]
+        sw, zw = _f64(sw), _i32(np.atleast_1d(zw))
+        out = np.empty((m, n), np.float32)
+        f = getattr(self.lib, self.prefix + "dynamic_matmul_rows")
+        f.restype = C.c_int
+        rc = f(_p(a, C.c_int8), _p(w, C.c_int8), _p(bias, C.c_float), _p(out, C.c_float), C.c_int(m), C.c_int(n),
+               C.c_int(k), C.c_int(1 if b_transpose else 0), _p(sx_rows, C.c_float), C.c_int(zx), _p(sw, C.c_double),
+               _p(zw, C.c_int32), C.c_int(len(sw)), C.c_int(act), *self._tail())
+        self._done(rc, "dynamic_matmul_rows")
+        return out
+
     def dynamic_matmul(self, a, w, bias, sx, zx, sw, zw, act=ACT_NONE, b_transpose=True):
         a, w, bias = _i8(a), _i8(w), _f32(bias)
         m, k = a.shape

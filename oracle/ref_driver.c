@@ -588,6 +588,37 @@ int ref_dynamic_quant(const float *x, int n, int symmetric, int8_t *q, double *s
 /* ------------------------------------------------------------------------------------------------------------
  * Dynamic-quant MatMul: LK/int8/matmul_dynamic_int8.cc:40-65,86-147; base LK/int8/matmul_dynamic_base_int8.cc
  * ------------------------------------------------------------------------------------------------------------ */
+/* DynamicQuantCPUKernel with prefer_axes: CalculateMinMaxFp32 and DoQuantizeFp32ToInt8 per segment, scale and zero
+ * point per segment as CalculatePerChannelScaleZp derives them (LK/int8/dynamic_quant.cc:188-218).  Single thread per
+ * segment, as in the wrapper. */
+int ref_dynamic_quant_segments(const float *x, int segments, int unit, int symmetric, int8_t *q, double *scales,
+                               int32_t *zps, int threads, double *run_seconds) {
+  (void)threads;
+  if (segments < 1 || unit < 1) return -1;
+  double t0 = now_s();
+  for (int s = 0; s < segments; ++s) {
+    float real_min = FLT_MAX, real_max = -FLT_MAX;
+    CalculateMinMaxFp32(x + (size_t)s * unit, unit, &real_min, &real_max);
+    double scale;
+    int zp = 0;
+    if (!symmetric) {
+      float range = real_max - real_min;
+      if (range <= 0) range = 0.01f;
+      scale = range / 255;
+      zp = (int)round(INT8_MIN - real_min / scale);
+    } else {
+      float amax = fabsf(real_max), amin = fabsf(real_min);
+      float mx = amax < amin ? amin : amax;
+      scale = 2 * mx / 254;
+    }
+    scales[s] = scale;
+    zps[s] = zp;
+    DoQuantizeFp32ToInt8(x + (size_t)s * unit, q + (size_t)s * unit, (float)scale, zp, unit, INT8_MIN, INT8_MAX);
+  }
+  if (run_seconds) *run_seconds = now_s() - t0;
+  return 0;
+}
+
 typedef struct dm_ctx {
   const int8_t *pack_a, *pack_b;
   const float *bias;
@@ -597,6 +628,7 @@ typedef struct dm_ctx {
   const float *sx;
   const float *swf;
   int zw0, peroc, act_type;
+  int per_row; /* input_per_channel_: sx has one entry per row */
 } dm_ctx;
 
 static void dm_task(void *p, int task) {
@@ -608,13 +640,31 @@ static void dm_task(void *p, int task) {
   const float *b = x->bias ? x->bias + cur_stride : NULL;
   const float *fs = x->peroc ? x->swf + cur_stride : x->swf;
   DynamicMatmul4x16x4AIWI(x->pack_a, x->pack_b + (size_t)cur_stride * x->deep16, b, x->c + cur_stride, x->row, cur_oc,
-                          x->deep, x->deep16, (size_t)x->col, x->zx, x->sx, fs, x->zw0, false, x->peroc,
+                          x->deep, x->deep16, (size_t)x->col, x->zx, x->sx, fs, x->zw0, x->per_row != 0, x->peroc,
                           (int64_t)x->act_type);
 }
+
+static int ref_dyn_mm(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
+                      int b_transpose, double sx, const float *sx_rows, int zx, const double *sw, const int32_t *zw,
+                      int nfilt, int act_type, int threads, double *run_seconds);
 
 int ref_dynamic_matmul(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
                        int b_transpose, double sx, int zx, const double *sw, const int32_t *zw, int nfilt,
                        int act_type, int threads, double *run_seconds) {
+  return ref_dyn_mm(a, w, bias, c, m, n, k, b_transpose, sx, NULL, zx, sw, zw, nfilt, act_type, threads, run_seconds);
+}
+
+int ref_dynamic_matmul_rows(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
+                            int b_transpose, const float *sx_rows, int zx, const double *sw, const int32_t *zw,
+                            int nfilt, int act_type, int threads, double *run_seconds) {
+  if (sx_rows == NULL) return -1;
+  return ref_dyn_mm(a, w, bias, c, m, n, k, b_transpose, 0.0, sx_rows, zx, sw, zw, nfilt, act_type, threads,
+                    run_seconds);
+}
+
+static int ref_dyn_mm(const int8_t *a, const int8_t *w, const float *bias, float *c, int m, int n, int k,
+                      int b_transpose, double sx, const float *sx_rows, int zx, const double *sw, const int32_t *zw,
+                      int nfilt, int act_type, int threads, double *run_seconds) {
   if (nfilt < 1 || (nfilt > 1 && nfilt != n)) return -1;
   if (threads < 1) threads = 1;
   const int peroc = nfilt > 1;
@@ -634,7 +684,8 @@ int ref_dynamic_matmul(const int8_t *a, const int8_t *w, const float *bias, floa
   int8_t *pack_a = malloc((size_t)row4 * deep16 + 1); /* InitMatrixABuffer, per Run */
   memset(pack_a, zx, (size_t)row4 * deep16);
   RowMajor2Row16x4MajorInt8(a, pack_a, m, k);
-  dm_ctx x = {pack_a, pack_b, bias, c, m, n, k, deep16, thread_stride * C4NUM, zx, &sxf, swf, zw[0], peroc, act_type};
+  dm_ctx x = {pack_a,  pack_b, bias,  c,        m, n, k, deep16, thread_stride * C4NUM, zx, sx_rows ? sx_rows : &sxf,
+              swf,     zw[0],  peroc, act_type, sx_rows != NULL};
   parallel_launch(dm_task, &x, thread_num);
   free(pack_a);
   if (run_seconds) *run_seconds = now_s() - t0;

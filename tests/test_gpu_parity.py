@@ -295,6 +295,39 @@ def test_dynamic_quant_chained_into_matmul(orc):
     assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("rows,k", [(1, 16), (5, 7), (37, 100), (64, 768), (130, 1030), (3, 5000)])
+def test_dynamic_quant_per_row_and_matmul(orc, rows, k):
+    """Per-channel activation quantisation (one scale per row) feeding the dynamic MatMul with per-row input scales,
+    host path and device-chained path, symmetric (what the converter emits) and asymmetric."""
+    import torch
+    rng = np.random.default_rng(rows * 1000 + k)
+    x = rng.normal(0, 1, (rows, k)).astype(np.float32)
+    x[rng.random((rows, k)) < 0.01] *= 8
+    if rows > 2:
+        x[1] = 0.25          # constant row: range 0 -> the 0.01 fallback
+        x[2, 0] = np.inf     # +inf dominates the row's max
+    n = 24
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
+    bias = rng.normal(0, 0.1, n).astype(np.float32)
+    mm = K.MatmulDynamicInt8Kernel(w, bias, _qps(sw, np.zeros(n, np.int32)))
+    for symmetric in (True, False):
+        want_q, want_s, want_z = orc.dynamic_quant_segments(x, symmetric)
+        dq = K.DynamicQuantKernel(symmetric)
+        got_q, qps = dq.run_rows(x)
+        assert np.array_equal(got_q, want_q)
+        assert [p.scale for p in qps] == list(want_s) and [p.zero_point for p in qps] == list(want_z)
+        want_c = orc.dynamic_matmul_rows(want_q, w, bias, want_s.astype(np.float32), int(want_z[0]), sw,
+                                         np.zeros(n, np.int32))
+        got_c = mm.run(got_q, qps)
+        assert np.array_equal(got_c.view(np.uint32), want_c.view(np.uint32))
+        xq, params = dq.run_rows(torch.from_numpy(x).cuda())
+        got_dev = mm.run(xq, row_params=params)
+        torch.cuda.synchronize()
+        assert np.array_equal(xq.cpu().numpy(), want_q)
+        assert np.array_equal(got_dev.cpu().numpy().view(np.uint32), want_c.view(np.uint32))
+
+
 def test_error_paths():
     L = K._lib.init()
     assert L.mi_matmul_run(None, None, 1, None, None) == K._lib.MI_NULL_PTR

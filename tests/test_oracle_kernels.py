@@ -249,6 +249,47 @@ def test_dynamic_quant_vs_nnacl(orc, ref):
             assert np.array_equal(q, q2)
 
 
+def test_dynamic_quant_segments_closed_form_and_nnacl(orc, ref):
+    """One {scale, zero point} per contiguous run: every run must equal the per-tensor closed form applied to that run
+    alone (a mistake in the run boundaries or a shared min/max fails), and the compiled nnacl sequence."""
+    rng = np.random.default_rng(310)
+    for segments, unit in [(1, 50), (7, 1), (37, 91), (16, 768), (3, 5000)]:
+        x = (rng.standard_normal((segments, unit)) * rng.uniform(0.1, 20, (segments, 1))).astype(np.float32)
+        if segments > 2 and unit > 1:
+            x[1] = -3.5                 # constant run
+            x[2, unit // 2] = np.nan    # never selected (a run of nothing but NaN is outside the closed form)
+        for sym in (False, True):
+            q, scales, zps = orc.dynamic_quant_segments(x, sym)
+            for i in range(segments):
+                s2, z2 = cf.dynquant_params(x[i], sym)
+                assert (scales[i], zps[i]) == (s2, z2), (segments, unit, i)
+                assert np.array_equal(q[i], cf.quantize_fp32_int8(x[i], np.float32(scales[i]), int(zps[i])))
+            q2, sc2, zp2 = ref.dynamic_quant_segments(x, sym)
+            assert np.array_equal(q, q2) and np.array_equal(scales, sc2) and np.array_equal(zps, zp2)
+
+
+def test_dynamic_matmul_rows_closed_form_and_nnacl(orc, ref):
+    """Per-row input scales: row r of the result equals the per-tensor closed form evaluated with that row's scale
+    (so using scale[0] everywhere, or indexing by column, fails); one input zero point for all rows."""
+    rng = np.random.default_rng(410)
+    for it in range(24):
+        m, n, k = int(rng.integers(1, 30)), int(rng.integers(1, 30)), int(rng.integers(1, 100))
+        case, w_nk = _dm_case(rng, m, n, k, bool(it & 1), 0 if it & 2 else int(rng.integers(-5, 6)), bool(it & 4),
+                              [0, 1, 3][it % 3], bool(it & 8))
+        sx_rows = rng.uniform(0.01, 0.1, m).astype(np.float32)
+        zx = case["zx"] if it & 16 else 0
+        got = orc.dynamic_matmul_rows(case["a"], case["w"], case["bias"], sx_rows, zx, case["sw"], case["zw"],
+                                      case["act"], case["b_transpose"])
+        for r in range(m):
+            want = cf.dynamic_matmul(case["a"][r:r + 1], w_nk, case["bias"], sx_rows[r], zx, case["sw"],
+                                     int(case["zw"][0]), case["act"])
+            assert np.array_equal(got[r:r + 1].view(np.uint32), want.view(np.uint32)), (it, r)
+        ref.threads = 1 + it % 3
+        got2 = ref.dynamic_matmul_rows(case["a"], case["w"], case["bias"], sx_rows, zx, case["sw"], case["zw"],
+                                       case["act"], case["b_transpose"])
+        assert np.array_equal(got.view(np.uint32), got2.view(np.uint32)), it
+
+
 def test_minmax(orc, ref):
     rng = np.random.default_rng(301)
     x = rng.standard_normal(10007).astype(np.float32)
