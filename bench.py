@@ -237,6 +237,63 @@ def cpu_baseline(case, size):
                        "column stripes on %d threads)" % (rows, size, size, cores))
 
 
+def cpu_side_by_side():
+    """The reference's CPU path on the other configurations (same engine and thread count as cpu_baseline), a few
+    seconds in total: decode GEMV (QKV matrix, one row), DynamicQuant 4096x768, the BERT QKV dynamic MatMul on its
+    first 256 rows, configuration 1, and the four layers of configuration 2."""
+    from oracle import pyoracle
+    from mindspore_amd import workloads as wl
+    cores = min(16, os.cpu_count() or 1)
+    if pyoracle.Reference.available():
+        eng, kind = pyoracle.reference(), "reference"
+        eng.threads = cores
+    else:
+        eng, kind = pyoracle.oracle(), "port"
+        eng.set_threads(cores)
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return eng.last_seconds if kind == "reference" else time.perf_counter() - t0
+
+    out = {"kind": kind, "cores": cores}
+    name, n, k = wl.DECODE_SHAPES[0]
+    c = wl.gemv_c4(name, n, k, 1, seed=0)
+    secs = timed(lambda: eng.matmul_int8(**{kk: c[kk] for kk in ("a", "w", "bias", "sx", "zx", "sw", "zw", "so", "zo", "act")}))
+    out["gemv_%s_m1" % name] = dict(ms=secs * 1e3, gbps=(n * k + k + n + 16 * n) / secs / 1e9)
+    x = wl.bert_c3_activation(768)
+    secs = timed(lambda: eng.dynamic_quant(x))
+    out["dynquant_4096x768"] = dict(ms=secs * 1e3, gbps=x.size * 5 / secs / 1e9)
+    q, sx, zx = eng.dynamic_quant(x)
+    bname, bn, bk = wl.BERT_SHAPES[0]
+    wt = wl.bert_c3_weights(bname, bn, bk)
+    rows = 256
+    secs = timed(lambda: eng.dynamic_matmul(q[:rows], wt["w"], wt["bias"], sx, zx, wt["sw"], np_zeros(bn)))
+    out["dynmm_%s_first_%d_rows" % (bname, rows)] = dict(ms=secs * 1e3, tops=2.0 * rows * bn * bk / secs / 1e12)
+    c1 = wl.fc_c1()
+    secs = timed(lambda: eng.matmul_int8(**{kk: c1[kk] for kk in ("a", "w", "bias", "sx", "zx", "sw", "zw", "so", "zo", "act")}))
+    out["c1_fc_128x768x768"] = dict(us=secs * 1e6)
+    xin, layers = wl.mobilenet_c2()
+    cur, total = xin, 0.0
+    for L in layers:
+        shape = pyoracle.conv_shape(cur.shape[0], cur.shape[1], cur.shape[2], L["ic"], L["oc"], (L["kernel"],) * 2,
+                                    (L["stride"],) * 2, (1, 1), L["pad"])
+        fn = eng.conv_dw_int8 if L["kind"] == "dw" else eng.conv_int8
+        res = {}
+        secs = timed(lambda: res.setdefault("y", fn(cur, L["w"], L["bias"], shape, L["sx"], L["zx"], L["sw"], L["zw"],
+                                                    L["so"], L["zo"], L["act"])))
+        out["c2_" + L["name"]] = dict(us=secs * 1e6)
+        total += secs
+        cur = res["y"]
+    out["c2_block_us"] = total * 1e6
+    return out
+
+
+def np_zeros(n):
+    import numpy as np
+    return np.zeros(n, np.int32)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -295,6 +352,8 @@ def main():
         torch.cuda.synchronize()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(g["case"], size)
+        if not args.no_extra:
+            extra["cpu_side_by_side"] = cpu_side_by_side()
     if "host_path_ms" in g:
         extra["gemm%d_host_tensors" % size] = dict(ms=g["host_path_ms"], tops=g["ops"] / (g["host_path_ms"] * 1e-3) / 1e12,
                                                    note="mi_matmul_run_host: H2D + kernel + D2H, PCIe inclusive")

@@ -85,6 +85,10 @@ __device__ __forceinline__ uint32_t pack4(int y0, int y1, int y2, int y3) {
 //      Per-channel parameters are read from LDS (array p of kEpiArrays x TILE_N ints, filled by EpiParams below):
 //      global loads here would share the vmcnt counter with the output stores and serialise on them. ----
 constexpr int kEpiArrays = 5;
+constexpr int kDeqStageRowBytes = 144;  // fp32 output staging: 32 columns (128 B) + 16 B so that rows shift banks
+// bytes of the wave-private output staging tile behind the parameter arrays
+template <int EPI, int TM>
+constexpr int epi_stage_bytes() { return EPI == EPI_REQUANT ? 16384 : TM * 32 * kDeqStageRowBytes; }
 
 // The workgroup's per-channel epilogue parameters: thread t holds channel n0 + t of each array (fetched at kernel
 // start, so the latency is hidden by the main loop) and drops them into LDS once the main loop is done.
@@ -239,12 +243,18 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
       m = m < g.m ? m : g.m - 1;
       sxr[j] = dq.per_row ? dq.qp_dev[m].scale_f : sx;
     }
+    // As for the int8 output, the accumulator layout (a lane holds 4 consecutive columns of 32 different rows) is
+    // turned into whole 128-byte row segments before it meets global memory: per 32-column block the wave's
+    // TM x 32 rows go through a wave-private LDS tile (row stride 144 bytes: the 16-byte writes of 8 consecutive
+    // rows and the 16-byte reads along a row are both bank-conflict free) and leave as 8 rows x 128 B per store.
+    constexpr int kRowB = kDeqStageRowBytes;
+    const int lane = h * 32 + r;
+    const int lr = lane >> 3, lc = lane & 7;
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int nb = n_w + i * 32 + q * 8 + h * 4;
-        if (nb >= g.n) continue;
         const int *pl = p + (nb - n_tile);
         const v4f ws4 = *reinterpret_cast<const v4f *>(pl);
         const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
@@ -254,7 +264,6 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e];
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
-          const int m = m_w + j * 32 + r;
           v4f o;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -270,8 +279,16 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
             }
             o[e] = d;
           }
-          if (m < g.m) *reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + nb) = o;
+          *reinterpret_cast<v4f *>(cstage + (j * 32 + r) * kRowB + (q * 8 + h * 4) * 4) = o;
         }
+      }
+      const int n = n_w + i * 32 + lc * 4;
+#pragma unroll
+      for (int t = 0; t < TM * 4; ++t) {
+        const int row = t * 8 + lr;
+        const v4f v = *reinterpret_cast<const v4f *>(cstage + row * kRowB + lc * 16);
+        const int m = m_w + row;
+        if (m < g.m && n < g.n) *reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + n) = v;
       }
     }
   }
@@ -451,7 +468,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
-                                                   lds + kEpiArrays * TILE_N * 4 + wave * 16384, n0, n0 + wn * WN,
+                                                   lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
                                                    m0 + wm * WM, r, h);
 }
 
@@ -561,7 +578,7 @@ __global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantPar
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
-                                                   lds + kEpiArrays * TILE_N * 4 + wave * 16384, n0, n0 + wn * WN,
+                                                   lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
                                                    m0 + wm * WM, r, h);
 }
 

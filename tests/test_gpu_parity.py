@@ -194,6 +194,8 @@ DW_CASES = [
     (1, 9, 9, 3, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2)),
     (1, 56, 56, 96, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),
     (1, 15, 18, 16, (5, 5), (1, 2), (1, 1), (2, 2, 2, 2)),
+    (2, 11, 9, 32, (3, 3), (2, 1), (2, 2), (2, 2, 2, 2)),
+    (1, 4, 4, 48, (3, 3), (1, 1), (1, 1), (2, 2, 2, 2)),
 ]
 
 
