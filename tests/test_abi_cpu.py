@@ -99,6 +99,13 @@ def test_device_entry_points_fail_cleanly_without_init(L):
     assert L.mi_conv_run(None, None, 1, 4, 4, None, None) == lib.MI_NULL_PTR
     assert L.mi_dynmm_run(None, None, 1, 0.1, 0, None, None) == lib.MI_NULL_PTR
     assert L.mi_dynquant_run(None, None, 4, None, None) == lib.MI_NULL_PTR
+    assert L.mi_dynquant_run_segments(None, None, 4, 4, None, None, None) == lib.MI_NULL_PTR
+    assert L.mi_dynquant_run_segments_host(None, None, 4, 4, None, None) == lib.MI_NULL_PTR
+    assert L.mi_dynmm_run_rows(None, None, 1, None, None, None) == lib.MI_NULL_PTR
+    assert L.mi_dynmm_run_rows_host(None, None, 1, None, 0, None) == lib.MI_NULL_PTR
+    assert L.mi_diag_stream_read(None, 16, None) == lib.MI_NULL_PTR
+    assert L.mi_diag_copy(None, None, 16, None) == lib.MI_NULL_PTR
+    assert L.mi_diag_mfma_rate(None, 1, 1, None, None) == lib.MI_NULL_PTR
     h = C.c_void_p()
     assert L.mi_matmul_create(None, None, None, C.byref(h)) == lib.MI_NULL_PTR
     import torch
