@@ -116,6 +116,20 @@ def bench_mfma_rate():
     return out
 
 
+def bench_vendor_int_mm(size, steps):
+    """Yardstick only (not part of the product path): the vendor GEMM library behind torch._int_mm on the same
+    operand distribution -- int8 x int8 -> int32, no requantisation, 16.8 MB less output compression work than the
+    kernel under test.  Shows what a tuned library reaches on this box under the same data-dependent clock."""
+    import torch
+    try:
+        a = torch.randint(-128, 128, (size, size), dtype=torch.int8, device="cuda")
+        b = torch.randint(-128, 128, (size, size), dtype=torch.int8, device="cuda")
+        ms, _ = time_steps(lambda: torch._int_mm(a, b), steps, 3)
+    except Exception as ex:  # noqa: BLE001 -- an optional yardstick must never fail the benchmark
+        return dict(error=str(ex)[:200])
+    return dict(ms=ms, tops=2.0 * size ** 3 / (ms * 1e-3) / 1e12, what="torch._int_mm, int32 output, uniform int8")
+
+
 def bench_gemv(steps, warmup, m=1):
     """Decode step: the five 7B-class layer matrices, three layers' worth of distinct weights (606 MB) cycled so the
     256 MB Infinity Cache cannot hold the working set.  Outputs are preallocated; one step = 15 launches."""
@@ -326,6 +340,7 @@ def main():
         extra["gemm%d" % other] = dict(ms=o["ms"], tops=o["tops"], frac_of_int8_peak=o["tops"] / PEAK_INT8_TOPS)
         extra["mfma_only"] = bench_mfma_rate()
         extra["gemm%d_frac_of_mfma_only_same_data" % size] = g["tops"] / extra["mfma_only"]["uniform_int8_operands"]["tops"]
+        extra["vendor_library_gemm%d" % size] = bench_vendor_int_mm(size, max(10, args.steps // 2))
         extra["hbm_read_stream"] = bench_hbm_read(args.steps, 3)
         extra["gemv_decode_m1"] = bench_gemv(max(5, args.steps // 2), 3, 1)
         extra["gemv_decode_m1"]["frac_of_read_stream"] = extra["gemv_decode_m1"]["gbps"] / extra["hbm_read_stream"]["gbps"]
