@@ -5,6 +5,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355x_int8.so")
+NATIVE_BENCH = os.path.join(HERE, "native_bench")
 SOURCES = ["capi.hip", "gemm_i8.hip", "gemv_i8.hip", "conv_i8.hip", "dynquant.hip"]
 # -ffp-contract=off: the float steps of DynamicQuant / dynamic MatMul and the host-side multiplier derivation are
 # separately rounded operations in the reference and must not be fused.
@@ -29,6 +30,10 @@ def build_library(verbose=False):
             raise RuntimeError("hipcc failed for %s" % cmd[-3])
     link = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs
     subprocess.check_call(link)
+    # the native benchmark host (a C++ caller of the C ABI, like a provider kernel)
+    subprocess.check_call(["hipcc", "-O2", "-std=c++17", "-x", "hip", "--offload-arch=gfx950", "-Wno-unused-result",
+                           os.path.join(CSRC, "native_bench.cc"), "-o", NATIVE_BENCH, "-L" + HERE, "-lmi355x_int8",
+                           "-Wl,-rpath,$ORIGIN"])
     return LIB
 
 

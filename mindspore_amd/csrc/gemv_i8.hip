@@ -54,7 +54,7 @@ struct GemvArgs {
 // No weight load is predicated (a predicated load makes the compiler wait for earlier loads before issuing later
 // ones): lanes past the end of a row re-read its last 16 bytes and chunks past the end of the stream re-read the
 // last chunk; both meet a zero activation fragment or are not accumulated.
-template <int M, int R, int D>
+template <int M, int R, int D, bool DIRECT>
 __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
   static_assert(D % R == 0, "the slot -> row mapping must be static");
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -84,16 +84,35 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
   const int32_t p_mult = rq.mult[my_n], p_e = rq.rshift[my_n], p_ls = rq.lshift[my_n], p_bias2 = rq.bias2[my_n];
   const int32_t p_zw = rq.zw[my_n];
 
-  // stage the activations (the weight loads above are already in flight)
+  // DIRECT (the whole share of the wave is in flight, total <= D): every wave fetches its own activation fragments
+  // straight into registers -- no LDS, no workgroup barrier.  Otherwise the workgroup stages the activations in LDS
+  // once (the weight loads above are already in flight either way).
+  v4i apre[DIRECT ? D / R : 1][M];
+  if (DIRECT) {
 #pragma unroll
-  for (int m = 0; m < M; ++m) {
-    const v4i *arow = reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda);
-    for (int ch = tid; ch < kc_pad; ch += 256) {
-      v4i z = {0, 0, 0, 0};
-      sa[m * kc_pad + ch] = ch < g.kchunks ? arow[ch] : z;
+    for (int sgi = 0; sgi < D / R; ++sgi)
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const int chunk = sgi * 64 + lane;
+        const int cc = chunk < g.kchunks ? chunk : g.kchunks - 1;
+        const v4i v = reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda)[cc];
+        const bool live = chunk < g.kchunks;
+        apre[sgi][m].x = live ? v.x : 0;
+        apre[sgi][m].y = live ? v.y : 0;
+        apre[sgi][m].z = live ? v.z : 0;
+        apre[sgi][m].w = live ? v.w : 0;
+      }
+  } else {
+#pragma unroll
+    for (int m = 0; m < M; ++m) {
+      const v4i *arow = reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda);
+      for (int ch = tid; ch < kc_pad; ch += 256) {
+        v4i z = {0, 0, 0, 0};
+        sa[m * kc_pad + ch] = ch < g.kchunks ? arow[ch] : z;
+      }
     }
+    __syncthreads();
   }
-  __syncthreads();
 
   int acc[R][M];
   int asum[M];
@@ -117,7 +136,11 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
 #pragma unroll
         for (int m = 0; m < M; ++m) {
           v4i z = {0, 0, 0, 0};
-          af[m] = seg < nseg ? sa[m * kc_pad + seg * 64 + lane] : z;
+          if (DIRECT) {
+            af[m] = apre[i / R][m];
+          } else {
+            af[m] = seg < nseg ? sa[m * kc_pad + seg * 64 + lane] : z;
+          }
           if (rq.has_zw) {
             v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
             asum[m] = dot16(af[m], ones, asum[m]);
@@ -168,10 +191,10 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
   }
 }
 
-template <int M, int R, int D>
-static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  auto kern = gemv_i8_kernel<M, R, D>;
-  const int lds_bytes = M * ((g.kchunks + 63) / 64) * 1024;
+template <int M, int R, int D, bool DIRECT>
+static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
+  auto kern = gemv_i8_kernel<M, R, D, DIRECT>;
+  const int lds_bytes = DIRECT ? 0 : M * ((g.kchunks + 63) / 64) * 1024;
   if (lds_bytes > 64 * 1024) {
     static bool attr_set = false;
     if (!attr_set) {
@@ -187,6 +210,12 @@ static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t st
   return MI_OK;
 }
 
+template <int M, int R, int D>
+static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
+  const int total = ((g.kchunks + 63) >> 6) * R;
+  return total <= D ? launch_mrdx<M, R, D, true>(g, rq, stream) : launch_mrdx<M, R, D, false>(g, rq, stream);
+}
+
 template <int M>
 static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
   // Measured on MI355X: HBM streams fastest with many light waves that each have their whole share in flight at
@@ -195,7 +224,7 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
   const int nseg = (g.kchunks + 63) >> 6;
   if (nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
   if (nseg == 2) return launch_mrd<M, 4, 8>(g, rq, stream);
-  if (nseg <= 4 || M == 2) return launch_mrd<M, 2, 8>(g, rq, stream);
+  if (nseg <= 4) return launch_mrd<M, 2, 8>(g, rq, stream);
   return launch_mrd<M, 1, 12>(g, rq, stream);
 }
 

@@ -1,0 +1,171 @@
+// Native host for the launch-latency-sensitive parts of the benchmark: a C++ caller of the C ABI, which is what a
+// MindSpore Lite provider kernel is.  (A Python caller spends about as long per call as a decode GEMV runs, so it
+// measures the interpreter, not the kernel.)  Prints one JSON object.
+//   native_bench decode <rows> <layers> <steps> <warmup>   the five 7B-class layer matrices x layers, cycled
+//   native_bench read <mib> <steps> <warmup>               the library's plain read stream over slices of 3 GiB
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "../../include/mi355x_int8.h"
+
+#define CHECK_HIP(x)                                                          \
+  do {                                                                        \
+    hipError_t e_ = (x);                                                      \
+    if (e_ != hipSuccess) {                                                   \
+      fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));                 \
+      return 1;                                                               \
+    }                                                                         \
+  } while (0)
+#define CHECK_MI(x)                                                           \
+  do {                                                                        \
+    int rc_ = (x);                                                            \
+    if (rc_ != MI_OK) {                                                       \
+      fprintf(stderr, "%s failed: %d (%s)\n", #x, rc_, mi_last_error());      \
+      return 1;                                                               \
+    }                                                                         \
+  } while (0)
+
+namespace {
+struct Rng {  // SplitMix64
+  uint64_t s;
+  uint64_t next() {
+    uint64_t z = (s += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+  }
+  double uniform() { return (double)(next() >> 11) * (1.0 / 9007199254740992.0); }
+};
+
+// weights ~ clip(round(N(0,1) * 32), +-127): sum of 12 uniforms as the normal
+int8_t normal_weight(Rng *r) {
+  double acc = -6.0;
+  const uint64_t a = r->next(), b = r->next();
+  for (int i = 0; i < 6; ++i) acc += (double)((a >> (10 * i)) & 1023) / 1024.0;
+  for (int i = 0; i < 6; ++i) acc += (double)((b >> (10 * i)) & 1023) / 1024.0;
+  double v = std::round(acc * 32.0);
+  v = v > 127 ? 127 : (v < -127 ? -127 : v);
+  return (int8_t)v;
+}
+
+struct Shape {
+  const char *name;
+  int n, k;
+};
+const Shape kDecode[5] = {{"qkv", 12288, 4096}, {"o", 4096, 4096}, {"gate", 11008, 4096}, {"up", 11008, 4096},
+                          {"down", 4096, 11008}};
+}  // namespace
+
+static int run_decode(int rows, int layers, int steps, int warmup) {
+  std::vector<mi_matmul *> handles;
+  std::vector<int8_t *> acts, outs;
+  std::vector<int> which;
+  double bytes = 0;
+  Rng rng{12345};
+  for (int l = 0; l < layers; ++l) {
+    for (int s = 0; s < 5; ++s) {
+      const int n = kDecode[s].n, k = kDecode[s].k;
+      std::vector<int8_t> w((size_t)n * k);
+      for (auto &x : w) x = normal_weight(&rng);
+      std::vector<double> scales(n);
+      std::vector<int32_t> zps(n, 0), bias(n);
+      for (int c = 0; c < n; ++c) {
+        scales[c] = 0.001 + 0.009 * rng.uniform();
+        bias[c] = (int32_t)(rng.next() % 10001) - 5000;
+      }
+      mi_matmul_desc d{};
+      d.deep = k;
+      d.col = n;
+      d.b_transpose = 1;
+      d.act_type = MI_ACT_NONE;
+      d.in_scale = 0.02;
+      d.in_zp = (int32_t)(rng.next() % 17) - 8;
+      d.out_scale = 0.02 * 0.0055 * std::sqrt((double)k) * 40.0;
+      d.out_zp = 0;
+      d.filter_quant_num = n;
+      d.filter_scales = scales.data();
+      d.filter_zps = zps.data();
+      mi_matmul *h = nullptr;
+      CHECK_MI(mi_matmul_create(&d, w.data(), bias.data(), &h));
+      handles.push_back(h);
+      which.push_back(s);
+      std::vector<int8_t> a((size_t)rows * k);
+      for (auto &x : a) x = (int8_t)(rng.next() & 0xff);
+      int8_t *ad = nullptr, *od = nullptr;
+      CHECK_HIP(hipMalloc(&ad, a.size()));
+      CHECK_HIP(hipMalloc(&od, (size_t)rows * n));
+      CHECK_HIP(hipMemcpy(ad, a.data(), a.size(), hipMemcpyHostToDevice));
+      acts.push_back(ad);
+      outs.push_back(od);
+      bytes += (double)n * k + (double)rows * k + (double)rows * n + 16.0 * n;
+    }
+  }
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  auto step = [&]() -> int {
+    for (size_t i = 0; i < handles.size(); ++i) CHECK_MI(mi_matmul_run(handles[i], acts[i], rows, outs[i], st));
+    return 0;
+  };
+  for (int i = 0; i < warmup; ++i)
+    if (step()) return 1;
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i)
+    if (step()) return 1;
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+  const double ms_step = ms / steps;
+  printf("{\"mode\": \"decode\", \"m\": %d, \"launches_per_step\": %zu, \"ms_per_step\": %.6f, \"us_per_launch\": %.3f, "
+         "\"bytes_per_step\": %.0f, \"gbps\": %.1f}\n",
+         rows, handles.size(), ms_step, ms_step * 1e3 / handles.size(), bytes, bytes / (ms_step * 1e-3) / 1e9);
+  for (auto *h : handles) mi_matmul_destroy(h);
+  return 0;
+}
+
+static int run_read(int mib, int steps, int warmup) {
+  const size_t total = (size_t)3 << 30, slice = (size_t)mib << 20;
+  const int nslices = (int)(total / slice);
+  char *buf = nullptr;
+  CHECK_HIP(hipMalloc(&buf, total));
+  CHECK_HIP(hipMemset(buf, 1, total));
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  for (int i = 0; i < warmup; ++i) CHECK_MI(mi_diag_stream_read(buf + (size_t)(i % nslices) * slice, (int64_t)slice, st));
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i)
+    CHECK_MI(mi_diag_stream_read(buf + (size_t)((i + warmup) % nslices) * slice, (int64_t)slice, st));
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+  printf("{\"mode\": \"read\", \"bytes\": %zu, \"ms\": %.6f, \"gbps\": %.1f}\n", slice, ms / steps,
+         (double)slice / (ms / steps * 1e-3) / 1e9);
+  return 0;
+}
+
+int main(int argc, char **argv) {
+  if (argc < 2) {
+    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | read <mib> <steps> <warmup>\n");
+    return 2;
+  }
+  CHECK_MI(mi_init(0));
+  if (strcmp(argv[1], "decode") == 0 && argc >= 6) return run_decode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
+  if (strcmp(argv[1], "read") == 0 && argc >= 5) return run_read(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
+  fprintf(stderr, "bad arguments\n");
+  return 2;
+}
