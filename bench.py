@@ -391,6 +391,12 @@ def main():
         for _ in range(3):
             lib.check(L.mi_diag_copy(dst.data_ptr(), src.data_ptr(), 256 << 20, _stream()), "mi_diag_copy")
         torch.cuda.synchronize()
+    if "mfma_only" in extra:
+        # the matrix pipe alone on operands drawn like this GEMM's: the shader clock it sustains depends on the data
+        lim = extra["mfma_only"]["uniform_int8_operands"]
+        result["roofline"]["peak_on_this_data"] = lim["tops"]
+        result["roofline"]["peak_on_this_data_clock_ghz"] = lim["shader_clock_ghz"]
+        result["roofline"]["frac_of_peak_on_this_data"] = g["tops"] / lim["tops"]
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(g["case"], size)
         if not args.no_extra:
