@@ -313,10 +313,10 @@ struct mi_matmul {
 
 struct mi_conv {
   mi_conv_desc d;
-  bool depthwise = false, direct_1x1 = false;
+  bool depthwise = false, direct_1x1 = false, dw_fast = false;
   int fill = 0;
   RequantState st;
-  DevBuf w16, dw_bias, col_ws, c_ws, h_in, h_out;
+  DevBuf w16, dw_bias, dw_bias_folded, col_ws, c_ws, h_in, h_out;
 };
 
 struct mi_dynquant {
@@ -581,8 +581,27 @@ int mi_conv_create(const mi_conv_desc *d, const int8_t *weight_host, const int32
     }
     std::vector<int32_t> b(oc, 0);
     if (bias_host != nullptr) memcpy(b.data(), bias_host, (size_t)oc * sizeof(int32_t));
+    // For the channel-vectorised kernel: a tap outside the image reads as the input zero point, so that
+    // (x - zx) * w vanishes there, and -zx * sum_t(w) moves into the bias once: bias' = bias - zx8 * sum_t w16[t][c].
+    // Identical to the reference's sum over the valid taps modulo 2^32.
+    const int32_t zx8 = (int32_t)(int8_t)d->in_zp;
+    std::vector<int32_t> bf(oc, 0);
+    h->dw_fast = h->st.amin <= h->st.amax;
+    for (int c = 0; c < oc; ++c) {
+      uint32_t wsum = 0;
+      for (int t = 0; t < plane; ++t) wsum += (uint32_t)(int32_t)w16[(size_t)t * oc + c];
+      bf[c] = (int32_t)((uint32_t)b[c] - (uint32_t)zx8 * wsum);
+      // the cheap rounding form needs: no left shift, 1 <= e <= 30, no saturating product, nothing leaves int32
+      const int32_t mult = h->st.h_mult[c], e = std::min(31, -h->st.h_rs[c]);
+      const int64_t vmax = (int64_t)plane * 255 * 255 + llabs((long long)b[c]);
+      const int64_t xmax = ((vmax * llabs((long long)mult)) >> 31) + 1;
+      if (h->st.h_ls[c] != 0 || e < 1 || e > 30 || mult == INT32_MIN || vmax >= ((int64_t)1 << 31) ||
+          xmax + ((int64_t)1 << (e - 1)) + llabs((long long)d->out_zp) + 1 > INT32_MAX)
+        h->dw_fast = false;
+    }
     if (rc == MI_OK) rc = upload(&h->w16, w16);
     if (rc == MI_OK) rc = upload(&h->dw_bias, b);
+    if (rc == MI_OK) rc = upload(&h->dw_bias_folded, bf);
   } else {
     const int kdim = d->kernel_h * d->kernel_w * d->in_channel;
     const bool is_1x1 = d->kernel_h == 1 && d->kernel_w == 1;
@@ -636,8 +655,10 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
     return MI_PARAM_INVALID;
   }
   if (h->depthwise) {
+    RequantParams rq = h->st.params();
+    rq.fast = h->dw_fast ? 1 : 0;
     return launch_conv_dw(in_dev, g, static_cast<const int16_t *>(h->w16.p), static_cast<const int32_t *>(h->dw_bias.p),
-                          (int)(int8_t)d.in_zp, h->st.params(), out_dev, s);
+                          static_cast<const int32_t *>(h->dw_bias_folded.p), (int)(int8_t)d.in_zp, rq, out_dev, s);
   }
   const int k = h->st.k;
   const int8_t *a = nullptr;
@@ -682,6 +703,7 @@ void mi_conv_destroy(mi_conv *h) {
   h->st.release();
   h->w16.release();
   h->dw_bias.release();
+  h->dw_bias_folded.release();
   h->col_ws.release();
   h->c_ws.release();
   h->h_in.release();

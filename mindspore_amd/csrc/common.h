@@ -98,9 +98,11 @@ struct ConvGeom {
 };
 // im2col into [batch*out_h*out_w][k16] with K order (kh, kw, ic); out-of-image taps are `fill`, the K tail is zero.
 int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, int k16, hipStream_t stream);
-// Depthwise conv + requantisation, weights pre-offset to int16 [KH*KW][C].
-int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
-                   const RequantParams &rq, int8_t *out, hipStream_t stream);
+// Depthwise conv + requantisation, weights pre-offset to int16 [KH*KW][C].  bias_folded = bias - zx8 * sum_t w16[t][c]
+// (used by the channel-vectorised kernel, which reads out-of-image taps as zx8); rq.fast: the host proved the cheap
+// rounding form exact for every channel.
+int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias,
+                   const int32_t *bias_folded, int zx8, const RequantParams &rq, int8_t *out, hipStream_t stream);
 
 // Measurement aids: read `bytes` and discard them / copy them, 16 bytes per lane.
 int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream);

@@ -202,16 +202,17 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const int8_t *__restrict__
 
 // Channel-vectorised variant for C % 16 == 0: one thread produces 16 consecutive channels of one output pixel, so
 // every tap is one 16-byte activation load and two 16-byte weight loads, and the store is one 16-byte row segment.
-// TAPS > 0 (kernel_h * kernel_w known at compile time): the loads of all taps are issued before the first
-// multiply; a tap outside the image reads a clamped address and contributes nothing.  TAPS == 0: any kernel size,
-// tap by tap.
+// A tap outside the image reads as the input zero point (the matching -zx * w is already in bias_folded), so the
+// inner product is sum_t x_t * w_t with no subtraction.  TAPS > 0 (kernel_h * kernel_w known at compile time): the
+// loads of all taps are issued before the first multiply.  TAPS == 0: any kernel size, tap by tap.
 template <int TAPS>
 __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict__ in, ConvGeom g,
                                                         const int16_t *__restrict__ w16,
-                                                        const int32_t *__restrict__ bias, int zx8, RequantParams rq,
-                                                        int8_t *__restrict__ out) {
+                                                        const int32_t *__restrict__ bias_folded, int zx8,
+                                                        RequantParams rq, int8_t *__restrict__ out) {
   const int ch = g.out_c, groups = ch >> 4;
   const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * groups;
+  const int zsplat = (zx8 & 0xff) * 0x01010101;
   union XV {
     v4i v;
     int8_t b[16];
@@ -230,7 +231,7 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
     const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * ch + c0;
     uint32_t acc[16];
     {
-      const v4i *bp = reinterpret_cast<const v4i *>(bias + c0);
+      const v4i *bp = reinterpret_cast<const v4i *>(bias_folded + c0);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const v4i bv = bp[q];
@@ -240,13 +241,21 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
         acc[4 * q + 3] = (uint32_t)bv.w;
       }
     }
-    auto mac = [&](const XV &xv, const WV &wv, bool inside) {
+    auto mac = [&](XV xv, const WV &wv, bool inside) {
+      xv.v.x = inside ? xv.v.x : zsplat;
+      xv.v.y = inside ? xv.v.y : zsplat;
+      xv.v.z = inside ? xv.v.z : zsplat;
+      xv.v.w = inside ? xv.v.w : zsplat;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        // both factors fit 9 bits + sign: a 24-bit multiply; a tap outside the image adds nothing
-        const int32_t xs = inside ? (int32_t)(int16_t)((int)xv.b[j] - zx8) : 0;
-        acc[j] += (uint32_t)(xs * (int32_t)wv.h[j]);
-      }
+      for (int j = 0; j < 16; ++j) acc[j] += (uint32_t)((int32_t)xv.b[j] * (int32_t)wv.h[j]);  // 8 bit x 10 bit
+    };
+    auto tap_address = [&](int kh, int kw, bool *inside) -> const int8_t * {
+      const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
+      const int iw = ow * g.stride_w - g.pad_l + kw * g.dilation_w;
+      *inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+      const int ihc = ih < 0 ? 0 : (ih >= g.in_h ? g.in_h - 1 : ih);
+      const int iwc = iw < 0 ? 0 : (iw >= g.in_w ? g.in_w - 1 : iw);
+      return img + ((int64_t)ihc * g.in_w + iwc) * ch;
     };
     if (TAPS > 0) {
       XV xv[TAPS > 0 ? TAPS : 1];
@@ -255,12 +264,7 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) {
         const int kh = t / g.kernel_w, kw = t - kh * g.kernel_w;
-        const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
-        const int iw = ow * g.stride_w - g.pad_l + kw * g.dilation_w;
-        inside[t] = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
-        const int ihc = ih < 0 ? 0 : (ih >= g.in_h ? g.in_h - 1 : ih);
-        const int iwc = iw < 0 ? 0 : (iw >= g.in_w ? g.in_w - 1 : iw);
-        xv[t].v = *reinterpret_cast<const v4i *>(img + ((int64_t)ihc * g.in_w + iwc) * ch);
+        xv[t].v = *reinterpret_cast<const v4i *>(tap_address(kh, kw, &inside[t]));
         const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)t * ch + c0);
         wv[t].v[0] = wp[0];
         wv[t].v[1] = wp[1];
@@ -268,21 +272,17 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) mac(xv[t], wv[t], inside[t]);
     } else {
-      for (int kh = 0; kh < g.kernel_h; ++kh) {
-        const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
-        if (ih < 0 || ih >= g.in_h) continue;
+      for (int kh = 0; kh < g.kernel_h; ++kh)
         for (int kw = 0; kw < g.kernel_w; ++kw) {
-          const int iw = ow * g.stride_w - g.pad_l + kw * g.dilation_w;
-          if (iw < 0 || iw >= g.in_w) continue;
           XV xv;
           WV wv;
-          xv.v = *reinterpret_cast<const v4i *>(img + ((int64_t)ih * g.in_w + iw) * ch);
+          bool inside;
+          xv.v = *reinterpret_cast<const v4i *>(tap_address(kh, kw, &inside));
           const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)(kh * g.kernel_w + kw) * ch + c0);
           wv.v[0] = wp[0];
           wv.v[1] = wp[1];
-          mac(xv, wv, true);
+          mac(xv, wv, inside);
         }
-      }
     }
     union {
       v4i v;
@@ -295,7 +295,12 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
       const v4i rs4 = *reinterpret_cast<const v4i *>(rq.rshift + c0 + 4 * q);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        int32_t y = rdiv_pot(srdhm((int32_t)(acc[4 * q + e] << ls4[e]), m4[e]), rs4[e]);
+        int32_t y;
+        if (rq.fast) {
+          y = rdiv_pot_fast(srdhm_nosat((int32_t)acc[4 * q + e], m4[e]), rs4[e], (1 << rs4[e]) >> 1);
+        } else {
+          y = rdiv_pot(srdhm((int32_t)(acc[4 * q + e] << ls4[e]), m4[e]), rs4[e]);
+        }
         y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
         y = y > rq.amin ? y : rq.amin;  // MSMAX first, then MSMIN (conv_depthwise_int8.c:49-50)
         y = y < rq.amax ? y : rq.amax;
@@ -306,16 +311,16 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
   }
 }
 
-int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias, int zx8,
-                   const RequantParams &rq, int8_t *out, hipStream_t stream) {
+int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias,
+                   const int32_t *bias_folded, int zx8, const RequantParams &rq, int8_t *out, hipStream_t stream) {
   const bool vec = (g.out_c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
   const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * (vec ? g.out_c >> 4 : g.out_c);
   const int64_t want = (total + 255) / 256;
   const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
   if (vec && g.kernel_h * g.kernel_w == 9) {
-    hipLaunchKernelGGL(conv_dw16_kernel<9>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+    hipLaunchKernelGGL(conv_dw16_kernel<9>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded, zx8, rq, out);
   } else if (vec) {
-    hipLaunchKernelGGL(conv_dw16_kernel<0>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
+    hipLaunchKernelGGL(conv_dw16_kernel<0>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded, zx8, rq, out);
   } else {
     hipLaunchKernelGGL(conv_dw_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
   }
