@@ -375,7 +375,7 @@ def main():
         nread = native_bench("read", 48, 64, 4)
         if nread and "gbps" in nread:
             extra["hbm_read_stream_native_host"] = nread
-        for m in (1, 8):
+        for m in (1, 8, 32):
             nat = native_bench("decode", m, 3, max(10, args.steps // 2), 3)
             py = section("gemv_decode_m%d_python_host" % m, lambda: bench_gemv(max(5, args.steps // 2), 3, m))
             if nat and "gbps" in nat:

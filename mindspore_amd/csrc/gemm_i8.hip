@@ -341,11 +341,14 @@ __device__ __forceinline__ void hint_interleave_reads() {
 }
 
 // =====================================================================================================================
-// direct main loop: 4 LDS stages x 64 bytes of K, asynchronous global -> LDS loads three tiles ahead
+// direct main loop: NST LDS stages x 64 bytes of K, asynchronous global -> LDS loads NST - 1 tiles ahead.
+// NST = 4 for the compute-bound shapes; NST = 16 with 64 x 64 tiles for a few (<= 64) activation rows, where the
+// kernel is a weight stream and what counts is the number of bytes in flight per CU.
 // =====================================================================================================================
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
-  constexpr int BKD = 64, NST = 4;
+  constexpr int BKD = 64, PD = NST - 1;  // PD: prefetch distance in K steps
+  static_assert((NST & (NST - 1)) == 0 && NST >= 4, "stage count must be a power of two");
   constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
   constexpr int STAGE = (TILE_N + TILE_M) * BKD;
   constexpr int WPW = TILE_N / 16 / 4, APW = TILE_M / 16 / 4, LPW = WPW + APW;  // 1 KiB blocks per wave and tile
@@ -408,10 +411,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
   // One 64-byte K step on LDS stage `st` (tile kt).  On entry f0 holds sub-step 0 of this stage.
   //   sub-step 0 : MFMAs on f0 while f1 <- sub-step 1 of this stage
-  //   barrier    : first wait until at most LPW of this wave's loads are outstanding (loads complete in order, so
-  //                that is "tile kt+1 has landed, tile kt+2 may still be in flight"), then meet the other waves:
-  //                now tile kt+1 is complete in LDS and nobody reads stage (st+3)&3 (tile kt-1) any more
-  //   sub-step 1 : refill that stage with tile kt+3, f0 <- sub-step 0 of tile kt+1, MFMAs on f1
+  //   barrier    : first wait until at most (PD - 2) * LPW of this wave's loads are outstanding (loads complete in
+  //                order, so that is "tile kt+1 has landed, later tiles may still be in flight"), then meet the other
+  //                waves: now tile kt+1 is complete in LDS and nobody reads stage st-1 (tile kt-1) any more
+  //   sub-step 1 : refill that stage with tile kt+PD, f0 <- sub-step 0 of tile kt+1, MFMAs on f1
   // Past the end of K the loads re-fetch the last tile into a stage nobody reads again, which keeps the
   // outstanding-load count the same in every step.
   auto step = [&](int kt, int st) {
@@ -419,12 +422,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
     hint_interleave_reads<TN, TM>();
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LPW) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PD - 2) * LPW) : "memory");
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    const int nxt = kt + 3 < ktiles ? kt + 3 : ktiles - 1;
-    read_frag(f0, (st + 1) & 3, 0);
-    dma_tile((st + 3) & 3, nxt);
+    const int nxt = kt + PD < ktiles ? kt + PD : ktiles - 1;
+    read_frag(f0, (st + 1) & (NST - 1), 0);
+    dma_tile((st + PD) & (NST - 1), nxt);
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
     {
       // operand reads first (the next sub-step waits for them), the loads of tile kt+3 behind them (they have
@@ -452,16 +455,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  dma_tile(0, 0);
-  dma_tile(1, 1);
-  dma_tile(2, 2);
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LPW) : "memory");
+#pragma unroll
+  for (int t = 0; t < PD; ++t) dma_tile(t, t < ktiles ? t : ktiles - 1);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PD - 1) * LPW) : "memory");
   read_frag(f0, 0, 0);
   for (int kt = 0; kt < ktiles; kt += 4) {
-    step(kt, 0);
-    step(kt + 1, 1);
-    step(kt + 2, 2);
-    step(kt + 3, 3);
+    const int st = NST == 4 ? 0 : (kt & (NST - 1));  // ktiles is a multiple of 4, NST a multiple of 4
+    step(kt, st);
+    step(kt + 1, st + 1);
+    step(kt + 2, st + 2);
+    step(kt + 3, st + 3);
   }
   // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -583,15 +586,15 @@ __global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantPar
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
   g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
   g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
   const int blocks = g.tiles_m * g.tiles_n;
   // the asynchronous global->LDS loader cannot zero-fill, so it needs every 64-byte K step of A to be in bounds
   if (g.k == g.k_pad) {
-    hipLaunchKernelGGL((gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
-                       rq, dq);
+    auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST>;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, g, rq, dq);
   } else {
     hipLaunchKernelGGL((gemm_staged_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
                        rq, dq);
@@ -605,6 +608,9 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
                             hipStream_t stream) {
   const int64_t tiles_l = (int64_t)((g.m + 255) / 256) * ((g.n + 255) / 256);
   const int64_t tiles_m = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
+  // a few activation rows against a big weight matrix: one row of 64 x 64 tiles, deep prefetch (HBM-bound)
+  if (g.m <= 64 && g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 16>(g, rq, dq, stream);
+  if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
   if (tiles_l >= 192) return launch_cfg<256, 256, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);

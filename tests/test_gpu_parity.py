@@ -46,7 +46,10 @@ def _gpu_matmul(case, device_tensors=False):
 
 MM_SHAPES = [(1, 1, 1), (1, 64, 16), (2, 5, 7), (3, 100, 15), (4, 256, 128), (5, 260, 129), (7, 33, 1000), (8, 512, 768),
              (9, 64, 64), (31, 31, 31), (64, 64, 128), (65, 65, 130), (128, 768, 768), (129, 257, 513),
-             (300, 100, 17), (500, 1030, 96), (1000, 3, 256), (2049, 1100, 64)]
+             (300, 100, 17), (500, 1030, 96), (1000, 3, 256), (2049, 1100, 64),
+             # few rows against long weight rows: the deep-prefetch tile configuration (16 LDS stages)
+             (17, 100, 1024), (33, 260, 2048), (64, 512, 4096), (40, 64, 1280), (20, 36, 5120),
+             (65, 100, 1024), (128, 260, 2048), (100, 64, 1280)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
