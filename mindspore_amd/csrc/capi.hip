@@ -331,6 +331,20 @@ struct mi_dynmm {
   DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out, h_params;
 };
 
+// No C++ exception may cross the C ABI: host allocations in the create calls can throw.
+template <typename F>
+static int guarded(const char *what, F &&f) {
+  try {
+    return f();
+  } catch (const std::bad_alloc &) {
+    set_error("%s: out of host memory", what);
+    return MI_MEMORY_FAILED;
+  } catch (...) {
+    set_error("%s: unexpected exception", what);
+    return MI_ERROR;
+  }
+}
+
 extern "C" {
 
 int mi_init(int device) {
@@ -430,7 +444,7 @@ int32_t mi_multiply_by_quantized_multiplier(int32_t value, int32_t multiplier, i
 }
 
 // ---------------------------------------------------------------------------------------------------------- matmul
-int mi_matmul_create(const mi_matmul_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_matmul **out) {
+static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_matmul **out) {
   if (d == nullptr || weight_host == nullptr || out == nullptr) {
     set_error("mi_matmul_create: null argument");
     return MI_NULL_PTR;
@@ -455,6 +469,10 @@ int mi_matmul_create(const mi_matmul_desc *d, const int8_t *weight_host, const i
   }
   *out = h;
   return MI_OK;
+}
+
+int mi_matmul_create(const mi_matmul_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_matmul **out) {
+  return guarded("mi_matmul_create", [&] { return mi_matmul_create_impl(d, weight_host, bias_host, out); });
 }
 
 int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream) {
@@ -535,7 +553,7 @@ int mi_conv_same_pad(int32_t in, int32_t kernel, int32_t stride, int32_t dilatio
   return MI_OK;
 }
 
-int mi_conv_create(const mi_conv_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_conv **out) {
+static int mi_conv_create_impl(const mi_conv_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_conv **out) {
   if (d == nullptr || weight_host == nullptr || out == nullptr) {
     set_error("mi_conv_create: null argument");
     return MI_NULL_PTR;
@@ -618,6 +636,10 @@ int mi_conv_create(const mi_conv_desc *d, const int8_t *weight_host, const int32
   }
   *out = h;
   return MI_OK;
+}
+
+int mi_conv_create(const mi_conv_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_conv **out) {
+  return guarded("mi_conv_create", [&] { return mi_conv_create_impl(d, weight_host, bias_host, out); });
 }
 
 int mi_conv_out_shape(const mi_conv *h, int32_t in_h, int32_t in_w, int32_t *out_h, int32_t *out_w) {
@@ -821,7 +843,7 @@ void mi_dynquant_destroy(mi_dynquant *h) {
 }
 
 // ---------------------------------------------------------------------------------------------------------- dynmm
-int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {
+static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {
   if (d == nullptr || weight_host == nullptr || out == nullptr) {
     set_error("mi_dynmm_create: null argument");
     return MI_NULL_PTR;
@@ -867,6 +889,10 @@ int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const flo
   }
   *out = h;
   return MI_OK;
+}
+
+int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {
+  return guarded("mi_dynmm_create", [&] { return mi_dynmm_create_impl(d, weight_host, bias_host, out); });
 }
 
 static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float sx, int32_t zx,
@@ -927,7 +953,7 @@ int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_d
   return dynmm_run_impl(h, a_dev, rows, 0.0f, 0, row_params_dev, c_dev, static_cast<hipStream_t>(stream), true);
 }
 
-int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
+static int mi_dynmm_run_rows_host_impl(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
                            float *c_host) {
   if (h == nullptr || a_host == nullptr || c_host == nullptr || in_scales == nullptr) {
     set_error("mi_dynmm_run_rows_host: null argument");
@@ -955,6 +981,11 @@ int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, cons
   if (rc != MI_OK) return rc;
   MI_HIP_CHECK(hipMemcpy(c_host, h->h_out.p, out_bytes, hipMemcpyDeviceToHost));
   return MI_OK;
+}
+
+int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
+                           float *c_host) {
+  return guarded("mi_dynmm_run_rows_host", [&] { return mi_dynmm_run_rows_host_impl(h, a_host, rows, in_scales, in_zp, c_host); });
 }
 
 int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in_scale, int32_t in_zp, float *c_host) {
