@@ -285,6 +285,8 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
           st.w_blocked.release();
           return rc;
         }
+        // one-time: later runs may come in on other streams and must find the copy complete
+        MI_HIP_CHECK(hipStreamSynchronize(stream));
       }
       w.blocked = static_cast<const int8_t *>(st.w_blocked.p);
     }
