@@ -11,12 +11,10 @@
 // one output row: the epilogue packs them into one 32-bit store, per-channel parameters are 16-byte loads, and
 // the input-row sum a lane needs is the one it accumulated itself (v_dot4 against 0x01010101).
 //
-// Two main loops share the epilogue:
-//   direct : K % 256 == 0.  Tiles travel global -> LDS with asynchronous 16-byte-per-lane loads
-//            (global_load_lds_dwordx4), four LDS stages of 64 bytes of K, three tiles in flight, one barrier per
-//            stage; operand fragments for K sub-step s+1 are read from LDS while the MFMAs of sub-step s run.
-//   staged : any K % 16 == 0.  Tiles travel global -> registers -> LDS (the tail of K is zero-filled in
-//            registers), two LDS stages of 128 bytes of K.
+// Main loop: tiles travel global -> LDS with asynchronous 16-byte-per-lane loads (global_load_lds_dwordx4), NST
+// LDS stages of 64 bytes of K, NST - 1 tiles in flight, one barrier per stage; operand fragments for K sub-step
+// s+1 are read from LDS while the MFMAs of sub-step s run.  Any K that is a multiple of 16: the weights are zero
+// padded, so an activation chunk past K only has to be a valid read (it re-reads the row's last chunk).
 // LDS rows are XOR-swizzled in units of 16 bytes so that 8 consecutive lanes of a 16-byte access always cover
 // all 32 banks.
 #include "common.h"
@@ -300,15 +298,17 @@ struct Frag {
 };
 
 template <int TN, int TM, bool HAS_ZW>
-__device__ __forceinline__ void mma_frag(v16i (&acc)[TN][TM], int (&rowsum)[TM], const Frag<TN, TM> &f) {
+__device__ __forceinline__ void mma_frag(v16i (&acc)[TN][TM], int (&rowsum)[TM], const Frag<TN, TM> &f, int ones) {
+  // ones: 0x01010101, or 0 when this lane's 16 activation bytes lie past K (they are then a re-read of valid
+  // bytes, harmless for the products because the weights are zero there, but they must not enter the row sums)
   if (HAS_ZW) {
 #pragma unroll
     for (int j = 0; j < TM; ++j) {
       int t = rowsum[j];
-      t = __builtin_amdgcn_sdot4(f.a[j].x, 0x01010101, t, false);
-      t = __builtin_amdgcn_sdot4(f.a[j].y, 0x01010101, t, false);
-      t = __builtin_amdgcn_sdot4(f.a[j].z, 0x01010101, t, false);
-      t = __builtin_amdgcn_sdot4(f.a[j].w, 0x01010101, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].x, ones, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].y, ones, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].z, ones, t, false);
+      t = __builtin_amdgcn_sdot4(f.a[j].w, ones, t, false);
       rowsum[j] = t;
     }
   }
@@ -362,7 +362,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
   const int r = lane & 31, h = lane >> 5;
-  const int ktiles = g.k_pad / BKD;  // multiple of 4
+  const int ktiles = (g.k + BKD - 1) / BKD;  // the zero padding of the weights past K needs no MFMAs
+  const int kchunks = g.k >> 4;
   EpiParams<TILE_N, EPI> epi;
   epi.fetch(rq, dq, n0, tid);
 
@@ -376,15 +377,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int i = 0; i < APW; ++i) {
     int m = m0 + (wave * APW + i) * 16 + drow;
     m = m < g.m ? m : g.m - 1;
-    asrc[i] = g.a + (int64_t)m * g.lda + dchunk * 16;
+    asrc[i] = g.a + (int64_t)m * g.lda;
   }
+  // A has exactly K valid bytes per row (the weights are zero padded, A is the caller's): a 16-byte chunk past K is
+  // fetched from the row's last chunk instead
+  const int a_last = (kchunks - 1) * 16;
   auto dma_tile = [&](int stage, int kt) {
     char *sw = lds + stage * STAGE + wave * WPW * 1024;
     char *sa = lds + stage * STAGE + TILE_N * BKD + wave * APW * 1024;
 #pragma unroll
     for (int i = 0; i < WPW; ++i) async_copy16(wsrc + (int64_t)i * 16 * g.ldw + kt * BKD, sw + i * 1024);
+    int koff = kt * BKD + dchunk * 16;
+    koff = koff < a_last ? koff : a_last;
 #pragma unroll
-    for (int i = 0; i < APW; ++i) async_copy16(asrc[i] + kt * BKD, sa + i * 1024);
+    for (int i = 0; i < APW; ++i) async_copy16(asrc[i] + koff, sa + i * 1024);
   };
 
   v16i acc[TN][TM];
@@ -419,7 +425,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // outstanding-load count the same in every step.
   auto step = [&](int kt, int st) {
     read_frag(f1, st, 1);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0, (kt * 4 + h < kchunks) ? 0x01010101 : 0);
     hint_interleave_reads<TN, TM>();
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((PD - 2) * LPW) : "memory");
@@ -428,7 +434,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int nxt = kt + PD < ktiles ? kt + PD : ktiles - 1;
     read_frag(f0, (st + 1) & (NST - 1), 0);
     dma_tile((st + PD) & (NST - 1), nxt);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
+    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1, (kt * 4 + 2 + h < kchunks) ? 0x01010101 : 0);
     {
       // operand reads first (the next sub-step waits for them), the loads of tile kt+3 behind them (they have
       // almost three steps to land)
@@ -459,125 +465,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int t = 0; t < PD; ++t) dma_tile(t, t < ktiles ? t : ktiles - 1);
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PD - 1) * LPW) : "memory");
   read_frag(f0, 0, 0);
-  for (int kt = 0; kt < ktiles; kt += 4) {
-    const int st = NST == 4 ? 0 : (kt & (NST - 1));  // ktiles is a multiple of 4, NST a multiple of 4
-    step(kt, st);
-    step(kt + 1, st + 1);
-    step(kt + 2, st + 2);
-    step(kt + 3, st + 3);
-  }
+  for (int kt = 0; kt < ktiles; ++kt) step(kt, kt & (NST - 1));
   // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  epi.to_lds(reinterpret_cast<int *>(lds), tid);
-  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
-                                                   lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
-                                                   m0 + wm * WM, r, h);
-}
-
-// =====================================================================================================================
-// staged main loop: 2 LDS stages x 128 bytes of K, global -> registers -> LDS, zero fill past K
-// =====================================================================================================================
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST>
-__global__ __launch_bounds__(256) void gemm_staged_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
-  constexpr int BK = 128, THREADS = 256;
-  constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
-  constexpr int STAGE = (TILE_N + TILE_M) * BK;
-  constexpr int W_CHUNKS = TILE_N * 8 / THREADS, A_CHUNKS = TILE_M * 8 / THREADS;
-  constexpr int ROWS_PER_PASS = THREADS / 8;
-  __shared__ __attribute__((aligned(1024))) char lds[2 * STAGE];
-
-  int tile_m, tile_n;
-  tile_coords(g, &tile_m, &tile_n);
-  const int m0 = tile_m * TILE_M, n0 = tile_n * TILE_N;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 1, wm = wave >> 1;
-  const int r = lane & 31, h = lane >> 5;
-  const int ktiles = (g.k + BK - 1) / BK, kchunks = g.k >> 4;  // the zero padding past K needs no MFMAs
-  EpiParams<TILE_N, EPI> epi;
-  epi.fetch(rq, dq, n0, tid);
-
-  // loader: thread t moves chunk (t & 7) of rows (t >> 3) + i * ROWS_PER_PASS; chunk c of row R is stored at slot
-  // c ^ (R & 7)
-  const int lc = tid & 7, lrow = tid >> 3;
-  v4i wreg[W_CHUNKS], areg[A_CHUNKS];
-  const int8_t *wsrc = g.w + (int64_t)(n0 + lrow) * g.ldw + lc * 16;
-  const int8_t *asrc[A_CHUNKS];
-#pragma unroll
-  for (int i = 0; i < A_CHUNKS; ++i) {
-    int m = m0 + lrow + i * ROWS_PER_PASS;
-    m = m < g.m ? m : g.m - 1;
-    asrc[i] = g.a + (int64_t)m * g.lda + lc * 16;
-  }
-  auto load_tile = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < W_CHUNKS; ++i)
-      wreg[i] = *reinterpret_cast<const v4i *>(wsrc + (int64_t)i * ROWS_PER_PASS * g.ldw + kt * BK);
-    const bool valid = kt * 8 + lc < kchunks;
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      v4i z = {0, 0, 0, 0};
-      areg[i] = valid ? *reinterpret_cast<const v4i *>(asrc[i] + kt * BK) : z;
-    }
-  };
-  auto store_tile = [&](int stage) {
-    char *sw = lds + stage * STAGE;
-    char *sa = sw + TILE_N * BK;
-#pragma unroll
-    for (int i = 0; i < W_CHUNKS; ++i) {
-      const int row = lrow + i * ROWS_PER_PASS;
-      *reinterpret_cast<v4i *>(sw + row * BK + ((lc ^ (row & 7)) << 4)) = wreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < A_CHUNKS; ++i) {
-      const int row = lrow + i * ROWS_PER_PASS;
-      *reinterpret_cast<v4i *>(sa + row * BK + ((lc ^ (row & 7)) << 4)) = areg[i];
-    }
-  };
-
-  v16i acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-  int rowsum[TM];
-#pragma unroll
-  for (int j = 0; j < TM; ++j) rowsum[j] = 0;
-
-  const int frag_swz = r & 7;
-  const int w_off = (wn * WN + r) * BK, a_off = TILE_N * BK + (wm * WM + r) * BK;
-  Frag<TN, TM> f0, f1;
-  auto read_frag = [&](Frag<TN, TM> &f, int stage, int s) {
-    const char *base = lds + stage * STAGE + (((2 * s + h) ^ frag_swz) << 4);
-#pragma unroll
-    for (int i = 0; i < TN; ++i) f.w[i] = *reinterpret_cast<const v4i *>(base + w_off + i * 32 * BK);
-#pragma unroll
-    for (int j = 0; j < TM; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * BK);
-  };
-
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-  read_frag(f0, 0, 0);
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const int st = kt & 1;
-    const bool more = kt + 1 < ktiles;
-    if (more) load_tile(kt + 1);
-    read_frag(f1, st, 1);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
-    read_frag(f0, st, 2);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
-    read_frag(f1, st, 3);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0);
-    if (more) store_tile(st ^ 1);
-    __syncthreads();
-    if (more) read_frag(f0, st ^ 1, 0);
-    mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1);
-  }
-
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
@@ -591,14 +481,8 @@ static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &
   g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
   g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
   const int blocks = g.tiles_m * g.tiles_n;
-  // the asynchronous global->LDS loader cannot zero-fill, so it needs every 64-byte K step of A to be in bounds
-  if (g.k == g.k_pad) {
-    auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST>;
-    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, g, rq, dq);
-  } else {
-    hipLaunchKernelGGL((gemm_staged_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST>), dim3(blocks), dim3(256), 0, stream, g,
-                       rq, dq);
-  }
+  auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST>;
+  hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, g, rq, dq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
