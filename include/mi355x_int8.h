@@ -36,6 +36,8 @@ extern "C" {
 #define MI_PARAM_INVALID (-3) /* RET_PARAM_INVALID: shape/quant-parameter mismatch, nothing was launched */
 #define MI_MEMORY_FAILED (-6) /* RET_MEMORY_FAILED */
 #define MI_NOT_SUPPORT (-7)   /* RET_NOT_SUPPORT: the creator should decline and let the builtin CPU kernel run */
+#define MI_INFER_ERR (-500)     /* RET_INFER_ERR: the operand shapes do not fit the operator */
+#define MI_INFER_INVALID (-501) /* RET_INFER_INVALID: an input dimension is still unknown (negative); infer again later */
 
 #define MI_ACT_NONE 0
 #define MI_ACT_RELU 1
@@ -218,6 +220,45 @@ int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_d
 int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
                            float *c_host);
 void mi_dynmm_destroy(mi_dynmm *h);
+
+/* ---- shape inference (host arithmetic, no GPU needed) --------------------------------------------------------------
+ * What a provider's kernel::KernelInterface::Infer (mindspore/lite/include/kernel_interface.h:42-59) computes for the
+ * operators of this path; Lite calls it in place of its builtin inference when one is registered
+ * (mindspore/lite/src/litert/infer_manager.cc:90-145).  Shapes are int32 arrays of at most MI_MAX_DIMS entries;
+ * out_shape must have room for MI_MAX_DIMS.  MI_INFER_INVALID when any input dimension is negative (the reference's
+ * InferFlag, NN/infer/common_infer.c:274-295), MI_INFER_ERR when the shapes do not fit, as Lite maps every other nnacl
+ * error (infer_manager.cc:147-160).  DynamicQuant needs no entry point: its output has the input's shape
+ * (NN/infer/dynamic_quant_infer.c:21-40). */
+#define MI_MAX_DIMS 8
+
+/* MatMulFusion.  Replaces MatmulInferShape / SetShape / CheckMatmulInputShape, NN/infer/matmul_infer.c:23-124: the
+ * shorter shape is left-padded with 1s, a pair of 1-D operands is treated as [1,K]x[K,1] and collapses to a scalar
+ * (out_dims 0), leading dimensions broadcast when one divides the other.  bias_dims 0 = no bias tensor. */
+int mi_infer_matmul(const int32_t *a_shape, int32_t a_dims, const int32_t *b_shape, int32_t b_dims,
+                    const int32_t *bias_shape, int32_t bias_dims, int32_t transpose_a, int32_t transpose_b,
+                    int32_t *out_shape, int32_t *out_dims);
+/* FullConnection.  Replaces FullConnectionInferShape, NN/infer/full_connection_infer.c:20-89.  w_shape is [N, K];
+ * bias_dims 0 = no bias tensor, which must agree with has_bias; with use_axis the input's dimensions from `axis` on
+ * are folded into K and the output keeps the leading ones, otherwise the output is [elements / K, N]. */
+int mi_infer_fullconnection(const int32_t *a_shape, int32_t a_dims, const int32_t *w_shape, int32_t w_dims,
+                            const int32_t *bias_shape, int32_t bias_dims, int32_t has_bias, int32_t use_axis,
+                            int32_t axis, int32_t *out_shape, int32_t *out_dims);
+
+#define MI_PAD_EXPLICIT 0 /* schema PadMode PAD */
+#define MI_PAD_SAME 1
+#define MI_PAD_VALID 2
+typedef struct mi_conv_infer {
+  int32_t kernel_h, kernel_w; /* -1: taken from the weight shape */
+  int32_t stride_h, stride_w, dilation_h, dilation_w;
+  int32_t pad_mode;
+  int32_t pad_u, pad_d, pad_l, pad_r; /* in: explicit padding; out: what SAME mode derived */
+  int32_t group;                      /* 0: taken from the weight shape (depthwise) */
+} mi_conv_infer;
+/* Conv2DFusion on an NHWC input [N,H,W,C] and a weight [OC,KH,KW,IC].  Replaces Conv2dInferShape / ConvInferShape /
+ * CheckConvAttr, NN/infer/conv2d_infer.c:20-166, including the float ceil of VALID mode and the clamp of a negative
+ * output extent to 1.  Updates p (kernel size, group, SAME-mode pads) as the reference updates its ConvParameter. */
+int mi_infer_conv2d(const int32_t *in_shape, int32_t in_dims, const int32_t *w_shape, int32_t w_dims,
+                    mi_conv_infer *p, int32_t *out_shape, int32_t *out_dims);
 
 /* ---- measurement aids (no counterpart in the reference) ---------------------------------------------------------
  * Two plain HBM movers with a known byte count and a matrix-pipe exerciser, used by the benchmark: the read stream gives the bandwidth a

@@ -6,7 +6,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355x_int8.so")
 NATIVE_BENCH = os.path.join(HERE, "native_bench")
-SOURCES = ["capi.hip", "gemm_i8.hip", "gemv_i8.hip", "conv_i8.hip", "dynquant.hip"]
+SOURCES = ["capi.hip", "gemm_i8.hip", "gemv_i8.hip", "conv_i8.hip", "dynquant.hip", "infer_shape.hip"]
 # -ffp-contract=off: the float steps of DynamicQuant / dynamic MatMul and the host-side multiplier derivation are
 # separately rounded operations in the reference and must not be fused.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",

@@ -316,3 +316,57 @@ class MatmulDynamicInt8Kernel(_Handle):
         _lib.check(L.mi_dynmm_run_host(self._h, a.ctypes.data, rows, float(in_quant.scale), int(in_quant.zero_point),
                                        out.ctypes.data), "mi_dynmm_run_host")
         return out
+
+
+# ---- shape inference (host arithmetic; what a provider's KernelInterface::Infer answers) ----
+
+def _shape_arg(shape):
+    shape = [] if shape is None else [int(d) for d in shape]
+    return (C.c_int32 * max(len(shape), 1))(*shape), len(shape)
+
+
+def _shape_result(code, what, out, out_dims):
+    _lib.check(code, what)
+    return [out[i] for i in range(out_dims.value)]
+
+
+def infer_matmul_shape(a_shape, b_shape, bias_shape=None, transpose_a=False, transpose_b=False):
+    """Output shape of MatMulFusion as ``MatmulInferShape`` derives it; raises ``MiError`` with code -501 while an
+    input dimension is unknown and -500 when the shapes do not fit."""
+    L = _lib.load()
+    a, an = _shape_arg(a_shape)
+    b, bn = _shape_arg(b_shape)
+    bias, biasn = _shape_arg(bias_shape)
+    out, out_dims = (C.c_int32 * 8)(), C.c_int32(0)
+    code = L.mi_infer_matmul(a, an, b, bn, bias, biasn, int(transpose_a), int(transpose_b), out, C.byref(out_dims))
+    return _shape_result(code, "mi_infer_matmul", out, out_dims)
+
+
+def infer_fullconnection_shape(a_shape, w_shape, bias_shape=None, has_bias=None, use_axis=False, axis=0):
+    """Output shape of FullConnection as ``FullConnectionInferShape`` derives it."""
+    L = _lib.load()
+    a, an = _shape_arg(a_shape)
+    w, wn = _shape_arg(w_shape)
+    bias, biasn = _shape_arg(bias_shape)
+    if has_bias is None:
+        has_bias = bias_shape is not None
+    out, out_dims = (C.c_int32 * 8)(), C.c_int32(0)
+    code = L.mi_infer_fullconnection(a, an, w, wn, bias, biasn, int(has_bias), int(use_axis), int(axis), out,
+                                     C.byref(out_dims))
+    return _shape_result(code, "mi_infer_fullconnection", out, out_dims)
+
+
+def infer_conv2d_shape(in_shape, w_shape, kernel=(-1, -1), stride=(1, 1), dilation=(1, 1), pad_mode=0,
+                       pads=(0, 0, 0, 0), group=1):
+    """Output shape of Conv2DFusion as ``Conv2dInferShape`` derives it, and the parameters it settles: returns
+    ``(out_shape, (pad_u, pad_d, pad_l, pad_r), (kernel_h, kernel_w), group)``.  pad_mode: 0 explicit, 1 SAME,
+    2 VALID."""
+    L = _lib.load()
+    x, xn = _shape_arg(in_shape)
+    w, wn = _shape_arg(w_shape)
+    p = _lib.ConvInfer(kernel[0], kernel[1], stride[0], stride[1], dilation[0], dilation[1], pad_mode,
+                       pads[0], pads[1], pads[2], pads[3], group)
+    out, out_dims = (C.c_int32 * 8)(), C.c_int32(0)
+    code = L.mi_infer_conv2d(x, xn, w, wn, C.byref(p), out, C.byref(out_dims))
+    shape = _shape_result(code, "mi_infer_conv2d", out, out_dims)
+    return shape, (p.pad_u, p.pad_d, p.pad_l, p.pad_r), (p.kernel_h, p.kernel_w), p.group

@@ -20,6 +20,7 @@ EXPORTS = [
     "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
     "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host",
     "mi_dynmm_destroy",
+    "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
     "mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate",
 ]
 
@@ -44,6 +45,12 @@ class DynmmDesc(C.Structure):
     _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
                 ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
                 ("filter_zps", C.POINTER(C.c_int32))]
+
+
+class ConvInfer(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in (
+        "kernel_h", "kernel_w", "stride_h", "stride_w", "dilation_h", "dilation_w", "pad_mode",
+        "pad_u", "pad_d", "pad_l", "pad_r", "group")]
 
 
 class DqParams(C.Structure):
@@ -118,6 +125,9 @@ def load():
     L.mi_dynmm_run_rows_host.argtypes = [vp, vp, i32, C.POINTER(dbl), i32, vp]
     L.mi_dynmm_destroy.argtypes = [vp]
     L.mi_dynmm_destroy.restype = None
+    L.mi_infer_matmul.argtypes = [pi32, i32, pi32, i32, pi32, i32, i32, i32, pi32, pi32]
+    L.mi_infer_fullconnection.argtypes = [pi32, i32, pi32, i32, pi32, i32, i32, i32, i32, pi32, pi32]
+    L.mi_infer_conv2d.argtypes = [pi32, i32, pi32, i32, C.POINTER(ConvInfer), pi32, pi32]
     L.mi_diag_stream_read.argtypes = [vp, i64, vp]
     L.mi_diag_copy.argtypes = [vp, vp, i64, vp]
     L.mi_diag_mfma_rate.argtypes = [vp, i32, i32, vp, vp]

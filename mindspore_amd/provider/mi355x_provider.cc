@@ -3,7 +3,9 @@
 // This translation unit is the reference-side half of the drop-in boundary: it subclasses mindspore::kernel::Kernel
 // (include/api/kernel.h:29-55) and registers creators through registry::RegisterKernel
 // (mindspore/lite/include/registry/register_kernel.h:57-74) for MatMulFusion, FullConnection, Conv2DFusion (int8) and
-// DynamicQuant (float32).  Everything below the Kernel objects is the C ABI of include/mi355x_int8.h.
+// DynamicQuant (float32), plus a kernel::KernelInterface (include/kernel_interface.h:29-59) for their shape inference
+// through registry::RegisterKernelInterface (include/registry/register_kernel_interface.h:36-75).  Everything below
+// the Kernel objects is the C ABI of include/mi355x_int8.h.
 //
 // It needs a MindSpore Lite SDK to compile (register_kernel.h includes the flatc-generated schema/model_generated.h)
 // and is therefore not part of the library build:
@@ -23,7 +25,9 @@
 #include "include/api/kernel.h"
 #include "include/api/status.h"
 #include "include/api/types.h"
+#include "include/kernel_interface.h"
 #include "include/registry/register_kernel.h"
+#include "include/registry/register_kernel_interface.h"
 #include "mi355x_int8.h"
 #include "schema/model_generated.h"
 
@@ -156,33 +160,62 @@ class ConvKernel : public kernel::Kernel {
   using Kernel::Kernel;
   ~ConvKernel() override { mi_conv_destroy(conv_); }
 
-  int Prepare() override {
-    const auto *cv = primitive_->value_as_Conv2DFusion();
-    const MSTensor &w = inputs_[kWeightIndex];
-    const auto in_shape = inputs_[0].Shape();  // NHWC
+  int Prepare() override { return Build(); }
+
+  // Weights and quant parameters do not depend on the image size; SAME-mode padding does (the builtin kernel gets
+  // it from shape inference at every resize, conv2d_infer.c:34-50), so the handle is rebuilt only when it moved.
+  int ReSize() override {
+    if (conv_ == nullptr) return kSuccess;  // Prepare has not run yet
     mi_conv_desc d{};
-    d.in_channel = static_cast<int32_t>(cv->in_channel());
-    d.out_channel = static_cast<int32_t>(cv->out_channel());
-    d.kernel_h = static_cast<int32_t>(cv->kernel_size()->Get(0));
-    d.kernel_w = static_cast<int32_t>(cv->kernel_size()->Get(1));
-    d.stride_h = static_cast<int32_t>(cv->stride()->Get(0));
-    d.stride_w = static_cast<int32_t>(cv->stride()->Get(1));
-    d.dilation_h = static_cast<int32_t>(cv->dilation()->Get(0));
-    d.dilation_w = static_cast<int32_t>(cv->dilation()->Get(1));
-    d.group = static_cast<int32_t>(cv->group());
-    d.act_type = cv->activation_type();
-    if (cv->pad_mode() == schema::PadMode_SAME) {  // the builtin kernel gets these from shape inference
+    FillGeometry(&d);
+    if (d.pad_u == pads_[0] && d.pad_d == pads_[1] && d.pad_l == pads_[2] && d.pad_r == pads_[3]) return kSuccess;
+    mi_conv_destroy(conv_);
+    conv_ = nullptr;
+    return Build();
+  }
+
+  int Execute() override {
+    const auto s = inputs_[0].Shape();
+    const auto *x = static_cast<const int8_t *>(inputs_[0].Data().get());
+    auto *y = static_cast<int8_t *>(outputs_[0].MutableData());
+    if (x == nullptr || y == nullptr || s.size() != 4) return kLiteNullptr;
+    return ToStatus(mi_conv_run_host(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]),
+                                     static_cast<int32_t>(s[2]), y));
+  }
+
+ private:
+  void FillGeometry(mi_conv_desc *d) const {
+    const auto *cv = primitive_->value_as_Conv2DFusion();
+    const auto in_shape = inputs_[0].Shape();  // NHWC
+    d->in_channel = static_cast<int32_t>(cv->in_channel());
+    d->out_channel = static_cast<int32_t>(cv->out_channel());
+    d->kernel_h = static_cast<int32_t>(cv->kernel_size()->Get(0));
+    d->kernel_w = static_cast<int32_t>(cv->kernel_size()->Get(1));
+    d->stride_h = static_cast<int32_t>(cv->stride()->Get(0));
+    d->stride_w = static_cast<int32_t>(cv->stride()->Get(1));
+    d->dilation_h = static_cast<int32_t>(cv->dilation()->Get(0));
+    d->dilation_w = static_cast<int32_t>(cv->dilation()->Get(1));
+    d->group = static_cast<int32_t>(cv->group());
+    d->act_type = cv->activation_type();
+    if (cv->pad_mode() == schema::PadMode_SAME && in_shape.size() == 4) {
       int32_t oh = 0, ow = 0;
-      mi_conv_same_pad(static_cast<int32_t>(in_shape[1]), d.kernel_h, d.stride_h, d.dilation_h, &d.pad_u, &d.pad_d,
-                       &oh);
-      mi_conv_same_pad(static_cast<int32_t>(in_shape[2]), d.kernel_w, d.stride_w, d.dilation_w, &d.pad_l, &d.pad_r,
-                       &ow);
+      mi_conv_same_pad(static_cast<int32_t>(in_shape[1]), d->kernel_h, d->stride_h, d->dilation_h, &d->pad_u,
+                       &d->pad_d, &oh);
+      mi_conv_same_pad(static_cast<int32_t>(in_shape[2]), d->kernel_w, d->stride_w, d->dilation_w, &d->pad_l,
+                       &d->pad_r, &ow);
     } else if (cv->pad_mode() == schema::PadMode_PAD && cv->pad_list() != nullptr && cv->pad_list()->size() == 4) {
-      d.pad_u = static_cast<int32_t>(cv->pad_list()->Get(0));
-      d.pad_d = static_cast<int32_t>(cv->pad_list()->Get(1));
-      d.pad_l = static_cast<int32_t>(cv->pad_list()->Get(2));
-      d.pad_r = static_cast<int32_t>(cv->pad_list()->Get(3));
+      d->pad_u = static_cast<int32_t>(cv->pad_list()->Get(0));
+      d->pad_d = static_cast<int32_t>(cv->pad_list()->Get(1));
+      d->pad_l = static_cast<int32_t>(cv->pad_list()->Get(2));
+      d->pad_r = static_cast<int32_t>(cv->pad_list()->Get(3));
     }
+  }
+
+  int Build() {
+    const MSTensor &w = inputs_[kWeightIndex];
+    mi_conv_desc d{};
+    FillGeometry(&d);
+    pads_[0] = d.pad_u, pads_[1] = d.pad_d, pads_[2] = d.pad_l, pads_[3] = d.pad_r;
     const auto iq = inputs_[0].QuantParams().front();
     const auto oq = outputs_[0].QuantParams().front();
     d.in_scale = iq.scale;
@@ -202,18 +235,7 @@ class ConvKernel : public kernel::Kernel {
       mi_conv_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const int32_t *>(bias), &conv_));
   }
 
-  int ReSize() override { return kSuccess; }
-
-  int Execute() override {
-    const auto s = inputs_[0].Shape();
-    const auto *x = static_cast<const int8_t *>(inputs_[0].Data().get());
-    auto *y = static_cast<int8_t *>(outputs_[0].MutableData());
-    if (x == nullptr || y == nullptr || s.size() != 4) return kLiteNullptr;
-    return ToStatus(mi_conv_run_host(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]),
-                                     static_cast<int32_t>(s[2]), y));
-  }
-
- private:
+  int32_t pads_[4] = {0, 0, 0, 0};
   mi_conv *conv_ = nullptr;
 };
 
@@ -319,6 +341,96 @@ std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> 
   return std::make_shared<DynamicQuantKernel>(in, out, prim, ctx);
 }
 
+// ---- shape inference -----------------------------------------------------------------------------------------------
+// Lite asks a provider's KernelInterface before its builtin inference (infer_manager.cc:90-145).  Output shapes come
+// from the library's mi_infer_* functions, which reproduce nnacl's results; data types stay as the model file has
+// them (a provider cannot see CNode.quantType, which is what makes the builtin MatMul inference switch a
+// dynamic-quant output to float32, matmul_infer.c:137-139).
+class ShapeInference : public kernel::KernelInterface {
+ public:
+  Status Infer(std::vector<MSTensor> *inputs, std::vector<MSTensor> *outputs,
+               const schema::Primitive *primitive) override {
+    if (inputs == nullptr || outputs == nullptr || primitive == nullptr || inputs->empty() || outputs->size() != 1) {
+      return kLiteInferError;
+    }
+    const auto dims = [](const MSTensor &t) {
+      std::vector<int32_t> v;
+      for (int64_t d : t.Shape()) v.push_back(static_cast<int32_t>(d));
+      return v;
+    };
+    int32_t out[MI_MAX_DIMS] = {0};
+    int32_t out_dims = 0;
+    int ret = MI_INFER_ERR;
+    const size_t n = inputs->size();
+    const std::vector<int32_t> a = dims((*inputs)[0]);
+    const std::vector<int32_t> b = n > 1 ? dims((*inputs)[1]) : std::vector<int32_t>();
+    const std::vector<int32_t> bias = n > 2 ? dims((*inputs)[2]) : std::vector<int32_t>();
+    if (a.size() > MI_MAX_DIMS || b.size() > MI_MAX_DIMS || bias.size() > MI_MAX_DIMS) return kLiteInferError;
+    switch (primitive->value_type()) {
+      case schema::PrimitiveType_MatMulFusion: {
+        const auto *mm = primitive->value_as_MatMulFusion();
+        if (mm == nullptr || (n != 2 && n != 3)) return kLiteInferError;
+        ret = mi_infer_matmul(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()),
+                              bias.data(), static_cast<int32_t>(bias.size()), mm->transpose_a(), mm->transpose_b(), out,
+                              &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_FullConnection: {
+        const auto *fc = primitive->value_as_FullConnection();
+        if (fc == nullptr || n < 2) return kLiteInferError;
+        ret = mi_infer_fullconnection(a.data(), static_cast<int32_t>(a.size()), b.data(),
+                                      static_cast<int32_t>(b.size()), bias.data(), static_cast<int32_t>(bias.size()),
+                                      fc->has_bias(), fc->use_axis(), static_cast<int32_t>(fc->axis()), out, &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_Conv2DFusion: {
+        const auto *cv = primitive->value_as_Conv2DFusion();
+        if (cv == nullptr || (n != 2 && n != 3)) return kLiteInferError;
+        // attribute defaults as the builtin populate step fills them (ops/populate/conv2d_populate.cc)
+        mi_conv_infer p{};
+        const auto at = [](const flatbuffers::Vector<int64_t> *v, uint32_t i, int32_t dflt) {
+          return v != nullptr && v->size() > i ? static_cast<int32_t>(v->Get(i)) : dflt;
+        };
+        p.kernel_h = at(cv->kernel_size(), 0, -1);
+        p.kernel_w = at(cv->kernel_size(), 1, -1);
+        p.stride_h = at(cv->stride(), 0, 1);
+        p.stride_w = at(cv->stride(), 1, 1);
+        p.dilation_h = at(cv->dilation(), 0, 1);
+        p.dilation_w = at(cv->dilation(), 1, 1);
+        p.pad_mode = cv->pad_mode() == schema::PadMode_SAME    ? MI_PAD_SAME
+                     : cv->pad_mode() == schema::PadMode_VALID ? MI_PAD_VALID
+                                                               : MI_PAD_EXPLICIT;
+        const bool has_pads = cv->pad_list() != nullptr && cv->pad_list()->size() >= 4;
+        p.pad_u = has_pads ? at(cv->pad_list(), 0, 0) : 0;
+        p.pad_d = has_pads ? at(cv->pad_list(), 1, 0) : 0;
+        p.pad_l = has_pads ? at(cv->pad_list(), 2, 0) : 0;
+        p.pad_r = has_pads ? at(cv->pad_list(), 3, 0) : 0;
+        p.group = static_cast<int32_t>(cv->group());
+        ret = mi_infer_conv2d(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()), &p,
+                              out, &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_DynamicQuant: {  // same shape as the input (dynamic_quant_infer.c:21-40)
+        for (int32_t d : a) {
+          if (d < 0) return kLiteInferInvalid;
+        }
+        (*outputs)[0].SetFormat((*inputs)[0].format());
+        (*outputs)[0].SetShape((*inputs)[0].Shape());
+        return kSuccess;
+      }
+      default:
+        return kLiteInferError;
+    }
+    (*outputs)[0].SetFormat((*inputs)[0].format());
+    if (ret == MI_INFER_INVALID) return kLiteInferInvalid;
+    if (ret != MI_OK) return kLiteInferError;
+    (*outputs)[0].SetShape(std::vector<int64_t>(out, out + out_dims));
+    return kSuccess;
+  }
+};
+
+std::shared_ptr<kernel::KernelInterface> ShapeInferenceCreator() { return std::make_shared<ShapeInference>(); }
+
 // ---- registration: arch "CPU" for applications, arch "" for the stock benchmark tool --------------------------------
 namespace {
 struct Registrar {
@@ -332,6 +444,10 @@ struct Registrar {
                                           ConvCreator);
       registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeFloat32,
                                           schema::PrimitiveType_DynamicQuant, DynamicQuantCreator);
+    }
+    for (int op : {schema::PrimitiveType_MatMulFusion, schema::PrimitiveType_FullConnection,
+                   schema::PrimitiveType_Conv2DFusion, schema::PrimitiveType_DynamicQuant}) {
+      registry::RegisterKernelInterface::Reg("mi355x", op, ShapeInferenceCreator);
     }
   }
 } g_registrar;

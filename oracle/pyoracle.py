@@ -289,6 +289,43 @@ class Reference(_Base):
                                                    C.byref(mn), C.byref(mx))
         return mn.value, mx.value
 
+    # ---- shape inference: the real nnacl functions; status is "ok", "invalid" (unknown dimension) or "error" ----
+    def _infer_status(self, ret):
+        return "ok" if ret == 0 else "invalid" if ret == self.lib.ref_nnacl_infer_invalid() else "error"
+
+    @staticmethod
+    def _ishape(shape):
+        shape = [] if shape is None else [int(d) for d in shape]
+        return (C.c_int * max(len(shape), 1))(*shape), len(shape)
+
+    def infer_matmul(self, a_shape, b_shape, bias_shape=None, transpose_a=False, transpose_b=False):
+        a, an = self._ishape(a_shape)
+        b, bn = self._ishape(b_shape)
+        bias, biasn = self._ishape(bias_shape)
+        out, on = (C.c_int * 8)(), C.c_int(0)
+        ret = self.lib.ref_infer_matmul(a, an, b, bn, bias, biasn, int(transpose_a), int(transpose_b), out,
+                                        C.byref(on))
+        return self._infer_status(ret), [out[i] for i in range(min(on.value, 8))]
+
+    def infer_fullconnection(self, a_shape, w_shape, bias_shape=None, has_bias=False, use_axis=False, axis=0):
+        a, an = self._ishape(a_shape)
+        w, wn = self._ishape(w_shape)
+        bias, biasn = self._ishape(bias_shape)
+        out, on = (C.c_int * 8)(), C.c_int(0)
+        ret = self.lib.ref_infer_fullconnection(a, an, w, wn, bias, biasn, int(has_bias), int(use_axis), int(axis),
+                                                out, C.byref(on))
+        return self._infer_status(ret), [out[i] for i in range(min(on.value, 8))]
+
+    def infer_conv2d(self, in_shape, w_shape, kernel, stride, dilation, pad_mode, pads, group):
+        x, xn = self._ishape(in_shape)
+        w, wn = self._ishape(w_shape)
+        cp = (C.c_int * 12)(kernel[0], kernel[1], stride[0], stride[1], dilation[0], dilation[1], pad_mode,
+                            pads[0], pads[1], pads[2], pads[3], group)
+        out, on = (C.c_int * 8)(), C.c_int(0)
+        ret = self.lib.ref_infer_conv2d(x, xn, w, wn, cp, out, C.byref(on))
+        return (self._infer_status(ret), [out[i] for i in range(min(on.value, 8))], tuple(cp[7:11]),
+                (cp[0], cp[1]), cp[11])
+
     def minmax(self, x):
         x = _f32(x)
         mn, mx = C.c_float(np.finfo(np.float32).max), C.c_float(-np.finfo(np.float32).max)

@@ -693,3 +693,82 @@ static int ref_dyn_mm(const int8_t *a, const int8_t *w, const float *bias, float
   free(swf);
   return 0;
 }
+
+/* ---- shape inference: the real nnacl functions behind Lite's builtin inference ---------------------------------- */
+#include "nnacl/infer/conv2d_infer.h"
+#include "nnacl/infer/full_connection_infer.h"
+#include "nnacl/infer/matmul_infer.h"
+
+static void ref_tensor(TensorC *t, const int *shape, int dims, int dtype) {
+  memset(t, 0, sizeof(*t));
+  t->data_type_ = dtype;
+  t->format_ = Format_NHWC;
+  t->shape_size_ = (size_t)dims;
+  for (int i = 0; i < dims && i < MAX_SHAPE_SIZE; ++i) t->shape_[i] = shape[i];
+}
+
+static int ref_emit_shape(int ret, const TensorC *out, int *out_shape, int *out_dims) {
+  *out_dims = (int)out->shape_size_;
+  for (size_t i = 0; i < out->shape_size_ && i < MAX_SHAPE_SIZE; ++i) out_shape[i] = out->shape_[i];
+  return ret;
+}
+
+/* Returns nnacl's own status (NNACL_OK 0, NNACL_INFER_INVALID, or an error). bias_dims 0 = two inputs. */
+int ref_infer_matmul(const int *a_shape, int a_dims, const int *b_shape, int b_dims, const int *bias_shape,
+                     int bias_dims, int transpose_a, int transpose_b, int *out_shape, int *out_dims) {
+  TensorC a, b, bias, out;
+  ref_tensor(&a, a_shape, a_dims, kNumberTypeInt8);
+  ref_tensor(&b, b_shape, b_dims, kNumberTypeInt8);
+  ref_tensor(&bias, bias_shape, bias_dims, kNumberTypeInt32);
+  ref_tensor(&out, NULL, 0, kNumberTypeInt8);
+  MatMulParameter p;
+  memset(&p, 0, sizeof(p));
+  p.a_transpose_ = transpose_a != 0;
+  p.b_transpose_ = transpose_b != 0;
+  const TensorC *in[3] = {&a, &b, &bias};
+  TensorC *outs[1] = {&out};
+  int ret = MatmulInferShape(in, bias_dims > 0 ? 3 : 2, outs, 1, (OpParameter *)&p);
+  return ref_emit_shape(ret, &out, out_shape, out_dims);
+}
+
+int ref_infer_fullconnection(const int *a_shape, int a_dims, const int *w_shape, int w_dims, const int *bias_shape,
+                             int bias_dims, int has_bias, int use_axis, int axis, int *out_shape, int *out_dims) {
+  TensorC a, w, bias, out;
+  ref_tensor(&a, a_shape, a_dims, kNumberTypeInt8);
+  ref_tensor(&w, w_shape, w_dims, kNumberTypeInt8);
+  ref_tensor(&bias, bias_shape, bias_dims, kNumberTypeInt32);
+  ref_tensor(&out, NULL, 0, kNumberTypeInt8);
+  MatMulParameter p;
+  memset(&p, 0, sizeof(p));
+  p.has_bias_ = has_bias != 0;
+  p.use_axis_ = use_axis != 0;
+  p.axis_ = axis;
+  const TensorC *in[3] = {&a, &w, &bias};
+  TensorC *outs[1] = {&out};
+  int ret = FullConnectionInferShape(in, bias_dims > 0 ? 3 : 2, outs, 1, (OpParameter *)&p);
+  return ref_emit_shape(ret, &out, out_shape, out_dims);
+}
+
+/* cp: kernel_h, kernel_w, stride_h, stride_w, dilation_h, dilation_w, pad_mode, pad_u, pad_d, pad_l, pad_r, group
+ * (read, and written back as the reference leaves its ConvParameter). */
+int ref_infer_conv2d(const int *in_shape, int in_dims, const int *w_shape, int w_dims, int *cp, int *out_shape,
+                     int *out_dims) {
+  TensorC in, w, out;
+  ref_tensor(&in, in_shape, in_dims, kNumberTypeInt8);
+  ref_tensor(&w, w_shape, w_dims, kNumberTypeInt8);
+  w.format_ = Format_KHWC;
+  ref_tensor(&out, NULL, 0, kNumberTypeInt8);
+  ConvParameter p;
+  memset(&p, 0, sizeof(p));
+  p.kernel_h_ = cp[0], p.kernel_w_ = cp[1], p.stride_h_ = cp[2], p.stride_w_ = cp[3];
+  p.dilation_h_ = cp[4], p.dilation_w_ = cp[5], p.pad_mode_ = (PadType)cp[6];
+  p.pad_u_ = cp[7], p.pad_d_ = cp[8], p.pad_l_ = cp[9], p.pad_r_ = cp[10], p.group_ = cp[11];
+  const TensorC *ins[2] = {&in, &w};
+  TensorC *outs[1] = {&out};
+  int ret = Conv2dInferShape(ins, 2, outs, 1, (OpParameter *)&p);
+  cp[0] = p.kernel_h_, cp[1] = p.kernel_w_, cp[7] = p.pad_u_, cp[8] = p.pad_d_, cp[9] = p.pad_l_, cp[10] = p.pad_r_;
+  cp[11] = p.group_;
+  return ref_emit_shape(ret, &out, out_shape, out_dims);
+}
+
+int ref_nnacl_infer_invalid(void) { return NNACL_INFER_INVALID; }
