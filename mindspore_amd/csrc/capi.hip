@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <memory>
 #include <new>
 #include <vector>
 
@@ -100,6 +101,10 @@ static void activation_range(int act, int32_t zp, float scale, int32_t *mn, int3
 struct DevBuf {
   void *p = nullptr;
   size_t bytes = 0;
+  DevBuf() = default;
+  DevBuf(const DevBuf &) = delete;
+  DevBuf &operator=(const DevBuf &) = delete;
+  ~DevBuf() { release(); }
   int ensure(size_t want) {
     if (want <= bytes) return MI_OK;
     if (p != nullptr) {
@@ -242,8 +247,11 @@ static std::vector<int8_t> to_nk(const int8_t *w, int n, int k, int b_transpose)
   if (b_transpose) {
     memcpy(out.data(), w, out.size());
   } else {
-    for (int kk = 0; kk < k; ++kk)
-      for (int c = 0; c < n; ++c) out[(size_t)c * k + kk] = w[(size_t)kk * n + c];
+    constexpr int kTile = 64;  // both the reads and the writes of a tile stay within a few cache lines
+    for (int k0 = 0; k0 < k; k0 += kTile)
+      for (int c0 = 0; c0 < n; c0 += kTile)
+        for (int kk = k0; kk < std::min(k, k0 + kTile); ++kk)
+          for (int c = c0; c < std::min(n, c0 + kTile); ++c) out[(size_t)c * k + kk] = w[(size_t)kk * n + c];
   }
   return out;
 }
@@ -460,16 +468,16 @@ static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_h
   int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
   if (rc != MI_OK) return rc;
   if ((rc = ensure_device()) != MI_OK) return rc;
-  mi_matmul *h = new (std::nothrow) mi_matmul();
+  std::unique_ptr<mi_matmul> owner(new (std::nothrow) mi_matmul());  // the buffers free themselves if anything below throws
+  mi_matmul *h = owner.get();
   if (h == nullptr) return MI_MEMORY_FAILED;
   const std::vector<int8_t> w_nk = to_nk(weight_host, d->col, d->deep, d->b_transpose);
   rc = h->st.build(w_nk.data(), d->col, d->deep, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
                    d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
   if (rc != MI_OK) {
-    mi_matmul_destroy(h);
     return rc;
   }
-  *out = h;
+  *out = owner.release();
   return MI_OK;
 }
 
@@ -528,15 +536,7 @@ int mi_matmul_get_params(const mi_matmul *h, int32_t *multiplier, int32_t *left_
   return MI_OK;
 }
 
-void mi_matmul_destroy(mi_matmul *h) {
-  if (h == nullptr) return;
-  h->st.release();
-  h->a_ws.release();
-  h->c_ws.release();
-  h->h_in.release();
-  h->h_out.release();
-  delete h;
-}
+void mi_matmul_destroy(mi_matmul *h) { delete h; }  // every DevBuf member frees its device memory
 
 // ------------------------------------------------------------------------------------------------------------ conv
 int mi_conv_same_pad(int32_t in, int32_t kernel, int32_t stride, int32_t dilation, int32_t *pad_before,
@@ -581,7 +581,8 @@ static int mi_conv_create_impl(const mi_conv_desc *d, const int8_t *weight_host,
   int rc = check_filter_quant(d->filter_quant_num, d->out_channel, d->filter_scales, d->filter_zps);
   if (rc != MI_OK) return rc;
   if ((rc = ensure_device()) != MI_OK) return rc;
-  mi_conv *h = new (std::nothrow) mi_conv();
+  std::unique_ptr<mi_conv> owner(new (std::nothrow) mi_conv());  // the buffers free themselves if anything below throws
+  mi_conv *h = owner.get();
   if (h == nullptr) return MI_MEMORY_FAILED;
   h->d = *d;
   h->d.filter_scales = nullptr;
@@ -633,10 +634,9 @@ static int mi_conv_create_impl(const mi_conv_desc *d, const int8_t *weight_host,
                      d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
   }
   if (rc != MI_OK) {
-    mi_conv_destroy(h);
     return rc;
   }
-  *out = h;
+  *out = owner.release();
   return MI_OK;
 }
 
@@ -722,18 +722,7 @@ int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t i
   return MI_OK;
 }
 
-void mi_conv_destroy(mi_conv *h) {
-  if (h == nullptr) return;
-  h->st.release();
-  h->w16.release();
-  h->dw_bias.release();
-  h->dw_bias_folded.release();
-  h->col_ws.release();
-  h->c_ws.release();
-  h->h_in.release();
-  h->h_out.release();
-  delete h;
-}
+void mi_conv_destroy(mi_conv *h) { delete h; }  // every DevBuf member frees its device memory
 
 // ------------------------------------------------------------------------------------------------------- dynquant
 int mi_dynquant_create(int32_t symmetric, mi_dynquant **out) {
@@ -741,15 +730,15 @@ int mi_dynquant_create(int32_t symmetric, mi_dynquant **out) {
   *out = nullptr;
   int rc = ensure_device();
   if (rc != MI_OK) return rc;
-  mi_dynquant *h = new (std::nothrow) mi_dynquant();
+  std::unique_ptr<mi_dynquant> owner(new (std::nothrow) mi_dynquant());  // the buffers free themselves if anything below throws
+  mi_dynquant *h = owner.get();
   if (h == nullptr) return MI_MEMORY_FAILED;
   h->symmetric = symmetric ? 1 : 0;
   if ((rc = h->partials.ensure(sizeof(float2) * kDqMaxBlocks)) != MI_OK ||
       (rc = h->params.ensure(sizeof(mi_dq_params))) != MI_OK) {
-    mi_dynquant_destroy(h);
     return rc;
   }
-  *out = h;
+  *out = owner.release();
   return MI_OK;
 }
 
@@ -834,15 +823,7 @@ int mi_dynquant_run_host(mi_dynquant *h, const float *x_host, int64_t n, int8_t 
   return MI_OK;
 }
 
-void mi_dynquant_destroy(mi_dynquant *h) {
-  if (h == nullptr) return;
-  h->partials.release();
-  h->params.release();
-  h->h_in.release();
-  h->h_out.release();
-  h->h_params.release();
-  delete h;
-}
+void mi_dynquant_destroy(mi_dynquant *h) { delete h; }  // every DevBuf member frees its device memory
 
 // ---------------------------------------------------------------------------------------------------------- dynmm
 static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {
@@ -859,7 +840,8 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
   int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
   if (rc != MI_OK) return rc;
   if ((rc = ensure_device()) != MI_OK) return rc;
-  mi_dynmm *h = new (std::nothrow) mi_dynmm();
+  std::unique_ptr<mi_dynmm> owner(new (std::nothrow) mi_dynmm());  // the buffers free themselves if anything below throws
+  mi_dynmm *h = owner.get();
   if (h == nullptr) return MI_MEMORY_FAILED;
   h->n = d->col;
   h->k = d->deep;
@@ -886,10 +868,9 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
   if (rc == MI_OK) rc = upload(&h->wsum, wsum);
   if (rc == MI_OK && h->has_bias) rc = upload(&h->bias, bs);
   if (rc != MI_OK) {
-    mi_dynmm_destroy(h);
     return rc;
   }
-  *out = h;
+  *out = owner.release();
   return MI_OK;
 }
 
@@ -1009,18 +990,6 @@ int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in
   return MI_OK;
 }
 
-void mi_dynmm_destroy(mi_dynmm *h) {
-  if (h == nullptr) return;
-  h->w.release();
-  h->wscale.release();
-  h->wsum.release();
-  h->bias.release();
-  h->a_ws.release();
-  h->c_ws.release();
-  h->h_in.release();
-  h->h_out.release();
-  h->h_params.release();
-  delete h;
-}
+void mi_dynmm_destroy(mi_dynmm *h) { delete h; }  // every DevBuf member frees its device memory
 
 }  // extern "C"

@@ -2,6 +2,8 @@
 // MindSpore Lite provider kernel is.  (A Python caller spends about as long per call as a decode GEMV runs, so it
 // measures the interpreter, not the kernel.)  Prints one JSON object.
 //   native_bench decode <rows> <layers> <steps> <warmup>   the five 7B-class layer matrices x layers, cycled
+//   native_bench warm <rows> <steps> <warmup>              each of the five matrices alone, back to back (its weights
+//                                                          stay in the 256 MB Infinity Cache between launches)
 //   native_bench read <mib> <steps> <warmup>               the library's plain read stream over slices of 3 GiB
 #include <hip/hip_runtime.h>
 
@@ -62,48 +64,90 @@ const Shape kDecode[5] = {{"qkv", 12288, 4096}, {"o", 4096, 4096}, {"gate", 1100
                           {"down", 4096, 11008}};
 }  // namespace
 
+struct Matrix {
+  mi_matmul *h = nullptr;
+  int8_t *act = nullptr, *out = nullptr;
+  int n = 0, k = 0;
+  double bytes = 0;
+};
+
+static int make_matrix(const Shape &shape, int rows, Rng *rng, Matrix *m) {
+  const int n = shape.n, k = shape.k;
+  std::vector<int8_t> w((size_t)n * k);
+  for (auto &x : w) x = normal_weight(rng);
+  std::vector<double> scales(n);
+  std::vector<int32_t> zps(n, 0), bias(n);
+  for (int c = 0; c < n; ++c) {
+    scales[c] = 0.001 + 0.009 * rng->uniform();
+    bias[c] = (int32_t)(rng->next() % 10001) - 5000;
+  }
+  mi_matmul_desc d{};
+  d.deep = k;
+  d.col = n;
+  d.b_transpose = 1;
+  d.act_type = MI_ACT_NONE;
+  d.in_scale = 0.02;
+  d.in_zp = (int32_t)(rng->next() % 17) - 8;
+  d.out_scale = 0.02 * 0.0055 * std::sqrt((double)k) * 40.0;
+  d.out_zp = 0;
+  d.filter_quant_num = n;
+  d.filter_scales = scales.data();
+  d.filter_zps = zps.data();
+  CHECK_MI(mi_matmul_create(&d, w.data(), bias.data(), &m->h));
+  std::vector<int8_t> a((size_t)rows * k);
+  for (auto &x : a) x = (int8_t)(rng->next() & 0xff);
+  CHECK_HIP(hipMalloc(&m->act, a.size()));
+  CHECK_HIP(hipMalloc(&m->out, (size_t)rows * n));
+  CHECK_HIP(hipMemcpy(m->act, a.data(), a.size(), hipMemcpyHostToDevice));
+  m->n = n;
+  m->k = k;
+  m->bytes = (double)n * k + (double)rows * k + (double)rows * n + 16.0 * n;
+  return 0;
+}
+
+static int run_warm(int rows, int steps, int warmup) {
+  Rng rng{777};
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  printf("{\"mode\": \"warm\", \"m\": %d", rows);
+  for (int s = 0; s < 5; ++s) {
+    if (s == 3) continue;  // "up" has the shape of "gate"
+    Matrix m;
+    if (make_matrix(kDecode[s], rows, &rng, &m)) return 1;
+    for (int i = 0; i < warmup; ++i) CHECK_MI(mi_matmul_run(m.h, m.act, rows, m.out, st));
+    CHECK_HIP(hipStreamSynchronize(st));
+    CHECK_HIP(hipEventRecord(e0, st));
+    for (int i = 0; i < steps; ++i) CHECK_MI(mi_matmul_run(m.h, m.act, rows, m.out, st));
+    CHECK_HIP(hipEventRecord(e1, st));
+    CHECK_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+    printf(", \"%s\": {\"n\": %d, \"k\": %d, \"us\": %.3f, \"gbps\": %.1f}", kDecode[s].name, m.n, m.k,
+           ms / steps * 1e3, m.bytes / (ms / steps * 1e-3) / 1e9);
+    mi_matmul_destroy(m.h);
+    CHECK_HIP(hipFree(m.act));
+    CHECK_HIP(hipFree(m.out));
+  }
+  printf("}\n");
+  return 0;
+}
+
 static int run_decode(int rows, int layers, int steps, int warmup) {
   std::vector<mi_matmul *> handles;
   std::vector<int8_t *> acts, outs;
-  std::vector<int> which;
   double bytes = 0;
   Rng rng{12345};
   for (int l = 0; l < layers; ++l) {
     for (int s = 0; s < 5; ++s) {
-      const int n = kDecode[s].n, k = kDecode[s].k;
-      std::vector<int8_t> w((size_t)n * k);
-      for (auto &x : w) x = normal_weight(&rng);
-      std::vector<double> scales(n);
-      std::vector<int32_t> zps(n, 0), bias(n);
-      for (int c = 0; c < n; ++c) {
-        scales[c] = 0.001 + 0.009 * rng.uniform();
-        bias[c] = (int32_t)(rng.next() % 10001) - 5000;
-      }
-      mi_matmul_desc d{};
-      d.deep = k;
-      d.col = n;
-      d.b_transpose = 1;
-      d.act_type = MI_ACT_NONE;
-      d.in_scale = 0.02;
-      d.in_zp = (int32_t)(rng.next() % 17) - 8;
-      d.out_scale = 0.02 * 0.0055 * std::sqrt((double)k) * 40.0;
-      d.out_zp = 0;
-      d.filter_quant_num = n;
-      d.filter_scales = scales.data();
-      d.filter_zps = zps.data();
-      mi_matmul *h = nullptr;
-      CHECK_MI(mi_matmul_create(&d, w.data(), bias.data(), &h));
-      handles.push_back(h);
-      which.push_back(s);
-      std::vector<int8_t> a((size_t)rows * k);
-      for (auto &x : a) x = (int8_t)(rng.next() & 0xff);
-      int8_t *ad = nullptr, *od = nullptr;
-      CHECK_HIP(hipMalloc(&ad, a.size()));
-      CHECK_HIP(hipMalloc(&od, (size_t)rows * n));
-      CHECK_HIP(hipMemcpy(ad, a.data(), a.size(), hipMemcpyHostToDevice));
-      acts.push_back(ad);
-      outs.push_back(od);
-      bytes += (double)n * k + (double)rows * k + (double)rows * n + 16.0 * n;
+      Matrix m;
+      if (make_matrix(kDecode[s], rows, &rng, &m)) return 1;
+      handles.push_back(m.h);
+      acts.push_back(m.act);
+      outs.push_back(m.out);
+      bytes += m.bytes;
     }
   }
   hipStream_t st;
@@ -160,11 +204,12 @@ static int run_read(int mib, int steps, int warmup) {
 
 int main(int argc, char **argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | read <mib> <steps> <warmup>\n");
+    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup>\n");
     return 2;
   }
   CHECK_MI(mi_init(0));
   if (strcmp(argv[1], "decode") == 0 && argc >= 6) return run_decode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
+  if (strcmp(argv[1], "warm") == 0 && argc >= 5) return run_warm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
   if (strcmp(argv[1], "read") == 0 && argc >= 5) return run_read(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
   fprintf(stderr, "bad arguments\n");
   return 2;
