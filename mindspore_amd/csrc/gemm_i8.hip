@@ -344,9 +344,11 @@ __device__ __forceinline__ void hint_interleave_reads() {
 // direct main loop: NST LDS stages x 64 bytes of K, asynchronous global -> LDS loads NST - 1 tiles ahead.
 // NST = 4 for the compute-bound shapes; NST = 16 with 64 x 64 tiles for a few (<= 64) activation rows, where the
 // kernel is a weight stream and what counts is the number of bytes in flight per CU.
+// OCC = workgroups the register allocation leaves room for on one CU (waves per SIMD): 1 for the 256 x 256 tile, which
+// needs the whole register file, 2 for the 128 x 128 tile.
 // =====================================================================================================================
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
   constexpr int BKD = 64, PD = NST - 1;  // PD: prefetch distance in K steps
   static_assert((NST & (NST - 1)) == 0 && NST >= 4, "stage count must be a power of two");
   constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
@@ -476,12 +478,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4>
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4, int OCC = 1>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
   g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
   g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
   const int blocks = g.tiles_m * g.tiles_n;
-  auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST>;
+  auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST, OCC>;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, g, rq, dq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
@@ -495,8 +497,16 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // a few activation rows against a big weight matrix: one row of 64 x 64 tiles, deep prefetch (HBM-bound)
   if (g.m <= 64 && g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 16>(g, rq, dq, stream);
   if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
-  if (tiles_l >= 192) return launch_cfg<256, 256, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
-  if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  // the fp32 epilogue writes four times the bytes: below one 256 x 256 tile per CU it is worth more to overlap it
+  // with another workgroup's main loop (two 128 x 128 tiles per CU) than to save operand traffic
+  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192)) return launch_cfg<256, 256, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  // a few hundred activation rows against many channels: 256-channel x 128-row tiles keep the weight re-reads of
+  // the square 128 tile away while still giving every CU a tile
+  if (g.m <= 512 && (int64_t)((g.m + 127) / 128) * ((g.n + 255) / 256) >= 128)
+    return launch_cfg<256, 128, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  // the 128 x 128 tile needs a quarter of the registers and 64 KiB of LDS: two workgroups share a CU, so one tile's
+  // prologue and epilogue overlap the other's main loop (what short-K shapes are made of)
+  if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 4, 2>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
 

@@ -49,7 +49,10 @@ MM_SHAPES = [(1, 1, 1), (1, 64, 16), (2, 5, 7), (3, 100, 15), (4, 256, 128), (5,
              (300, 100, 17), (500, 1030, 96), (1000, 3, 256), (2049, 1100, 64),
              # few rows against long weight rows: the deep-prefetch tile configuration (16 LDS stages)
              (17, 100, 1024), (33, 260, 2048), (64, 512, 4096), (40, 64, 1280), (20, 36, 5120),
-             (65, 100, 1024), (128, 260, 2048), (100, 64, 1280)]
+             (65, 100, 1024), (128, 260, 2048), (100, 64, 1280),
+             # a few hundred rows against many channels: the 256-channel x 128-row tile; two workgroups per CU on the
+             # 128 x 128 tile (4224 x 2100 gives 33 x 17 of them)
+             (300, 11008, 80), (512, 8196, 272), (129, 32772, 48), (4224, 2100, 144)]
 
 
 @pytest.mark.parametrize("m,n,k", MM_SHAPES)
