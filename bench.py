@@ -24,7 +24,7 @@ PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E peak, GB/s
 
 # HBM-side bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
 # this script, each scaled by what the same counter reads for the 256 MiB copy of --calibrate (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000; summary in profiles/gemm_direct_kernel_gemm4096.txt): (99515 + 16640) KiB.  None = not measured.
+# WRITE_SIZE x 1.000; summary in profiles/gemm_direct_kernel_gemm4096.txt): (99337 + 16640) KiB.  None = not measured.
 MEASURED_TRAFFIC_BYTES = {"gemm4096": (99337 + 16640) * 1024, "gemm8192": None}
 
 
