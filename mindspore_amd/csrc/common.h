@@ -62,8 +62,9 @@ struct WeightView {
   int k_pad;
   int ldw;
   // Second copy for the matrix-core decode kernel (3..16 activation rows), or nullptr: the same bytes regrouped into
-  // 1 KiB blocks [row / 16][k / 64][row % 16][k % 64], so that the 16 rows x 64 bytes a wave instruction fetches are
-  // contiguous.  Built on the device on first use (launch_block_weights).
+  // 1 KiB blocks [row / 16][k / 64], the 64 16-byte chunks of a block in the order the lanes of the MFMA operand take
+  // them ([(k % 64) / 16][row % 16]), so that a wave instruction fetches 1 KiB front to back.  Built on the device on
+  // first use (launch_block_weights).
   const int8_t *blocked;
 };
 inline int weight_row_stride(int k_pad) { return (k_pad / 256) % 2 == 0 ? k_pad + 256 : k_pad; }
