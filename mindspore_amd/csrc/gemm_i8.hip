@@ -342,7 +342,7 @@ __device__ __forceinline__ void hint_interleave_reads() {
 
 // =====================================================================================================================
 // direct main loop: NST LDS stages x 64 bytes of K, asynchronous global -> LDS loads NST - 1 tiles ahead.
-// NST = 4 for the compute-bound shapes; NST = 16 with 64 x 64 tiles for a few (<= 64) activation rows, where the
+// NST = 4 for the compute-bound shapes (3 for short K, where a third workgroup per CU is worth more than depth); NST = 16 with 64 x 64 tiles for a few (<= 64) activation rows, where the
 // kernel is a weight stream and what counts is the number of bytes in flight per CU.
 // OCC = workgroups the register allocation leaves room for on one CU (waves per SIMD): 1 for the 256 x 256 tile, which
 // needs the whole register file, 2 for the 128 x 128 tile.
@@ -350,11 +350,15 @@ __device__ __forceinline__ void hint_interleave_reads() {
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
   constexpr int BKD = 64, PD = NST - 1;  // PD: prefetch distance in K steps
-  static_assert((NST & (NST - 1)) == 0 && NST >= 4, "stage count must be a power of two");
+  static_assert(NST >= 3, "the loop keeps NST - 1 >= 2 tiles in flight");
+  auto wrap = [](int x) { return x >= NST ? x - NST : x; };  // stage index after an increment of at most NST
   constexpr int WN = TILE_N / 2, WM = TILE_M / 2, TN = WN / 32, TM = WM / 32;
   constexpr int STAGE = (TILE_N + TILE_M) * BKD;
   constexpr int WPW = TILE_N / 16 / 4, APW = TILE_M / 16 / 4, LPW = WPW + APW;  // 1 KiB blocks per wave and tile
   static_assert(WPW >= 1 && APW >= 1, "tile too small");
+  static_assert(EPI == EPI_REQUANT ? (TN != 4 || TM != 4 || NST * STAGE >= kEpiArrays * TILE_N * 4 + 4 * 16384)
+                                   : NST * STAGE >= kEpiArrays * TILE_N * 4 + 4 * epi_stage_bytes<EPI, TM>(),
+                "the epilogue staging must fit the main loop's LDS");
   __shared__ __attribute__((aligned(1024))) char lds[NST * STAGE];
 
   int tile_m, tile_n;
@@ -434,8 +438,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
     asm volatile("s_barrier" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     const int nxt = kt + PD < ktiles ? kt + PD : ktiles - 1;
-    read_frag(f0, (st + 1) & (NST - 1), 0);
-    dma_tile((st + PD) & (NST - 1), nxt);
+    read_frag(f0, wrap(st + 1), 0);
+    dma_tile(wrap(st + PD), nxt);
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1, (kt * 4 + 2 + h < kchunks) ? 0x01010101 : 0);
     {
       // operand reads first (the next sub-step waits for them), the loads of tile kt+3 behind them (they have
@@ -467,7 +471,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
   for (int t = 0; t < PD; ++t) dma_tile(t, t < ktiles ? t : ktiles - 1);
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PD - 1) * LPW) : "memory");
   read_frag(f0, 0, 0);
-  for (int kt = 0; kt < ktiles; ++kt) step(kt, kt & (NST - 1));
+  for (int kt = 0, st = 0; kt < ktiles; ++kt, st = wrap(st + 1)) step(kt, st);
   // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
@@ -506,6 +510,9 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
     return launch_cfg<256, 128, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // the 128 x 128 tile needs a quarter of the registers and 64 KiB of LDS: two workgroups share a CU, so one tile's
   // prologue and epilogue overlap the other's main loop (what short-K shapes are made of)
+  // short K and more tiles than two per CU: three stages (48 KiB) let a third workgroup in, which saves a round of
+  // tiles; the shallower prefetch only costs when K is long
+  if (tiles_m > 512 && g.k <= 1024) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 3, 3>(g, rq, dq, stream);
   if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 4, 2>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
