@@ -286,7 +286,14 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         const int row = t * 8 + lr;
         const v4f v = *reinterpret_cast<const v4f *>(cstage + row * kRowB + lc * 16);
         const int m = m_w + row;
-        if (m < g.m && n < g.n) *reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + n) = v;
+        if (m < g.m && n < g.n) {
+          v4f *dst = reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + n);
+          if (FAST) {  // in this epilogue the parameter selects non-temporal stores (see stream_out_hint)
+            __builtin_nontemporal_store(v, dst);
+          } else {
+            *dst = v;
+          }
+        }
       }
     }
   }
@@ -517,6 +524,12 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
 
+// Large fp32 outputs are written with non-temporal stores: they are not re-read out of L2 by whatever runs next, and
+// they do not queue behind dirty lines.  Measured over twelve shapes with 12-75 MB of output: 3-13 % faster (BERT QKV
+// 22.0 -> 19.5 us) except where every tile of the grid finishes in the same moment (exactly three tiles per CU: 2-6 %
+// slower).  A compile-time choice: the two kinds of store under a run-time condition are merged into plain stores.
+static bool stream_out_hint(int64_t out_bytes) { return out_bytes >= ((int64_t)8 << 20); }
+
 static int check_args(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n, const void *c,
                       int64_t ldc, int c_align) {
   const int8_t *w = wv.w;
@@ -555,8 +568,14 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
   if (rc != MI_OK) return rc;
   GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
   RequantParams rq{};
-  return dq.zw0 != 0 ? launch_pick_tile<EPI_DEQUANT, true, false>(g, rq, dq, stream)
-                     : launch_pick_tile<EPI_DEQUANT, false, false>(g, rq, dq, stream);
+  // the third parameter (the fast-rounding switch of the int8 epilogue) selects non-temporal stores here
+  const bool nt = stream_out_hint((int64_t)m * n * 4);
+  if (dq.zw0 != 0) {
+    return nt ? launch_pick_tile<EPI_DEQUANT, true, true>(g, rq, dq, stream)
+              : launch_pick_tile<EPI_DEQUANT, true, false>(g, rq, dq, stream);
+  }
+  return nt ? launch_pick_tile<EPI_DEQUANT, false, true>(g, rq, dq, stream)
+            : launch_pick_tile<EPI_DEQUANT, false, false>(g, rq, dq, stream);
 }
 
 // Measurement aid: nothing but back-to-back MFMAs on register operands taken from `operands` (256 threads x 8 x 16
