@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4i *__restrict_
   for (int i = 0; i < 8; ++i) {
     int64_t c = wave * 512 + i * 64 + lane;
     c = c < chunks ? c : chunks - 1;
-    buf[i] = src[c];
+    buf[i] = __builtin_nontemporal_load(src + c);  // as the decode kernels read their weights
   }
   int s = 0;
 #pragma unroll

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
     const int seg = c / R, rr = c % R;
     int off = seg * 1024 + lane * 16;
     off = off < last_off ? off : last_off;
-    return *reinterpret_cast<const v4i *>(wrow + (int64_t)rr * g.ldw + off);
+    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wrow + (int64_t)rr * g.ldw + off));
   };
   v4i buf[D];
 #pragma unroll
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, 
   auto load_w = [&](int j, int rg) -> v4i {
     int s = s0 + j;
     s = s < total ? s : total - 1;
-    return *reinterpret_cast<const v4i *>(wbase + ((int64_t)rg * total + s) * 1024);
+    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wbase + ((int64_t)rg * total + s) * 1024));
   };
   auto load_x = [&](int j) -> v4i {
     int off = (s0 + j) * 64 + grp * 16;
