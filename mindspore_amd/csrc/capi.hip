@@ -140,7 +140,7 @@ static int upload(DevBuf *b, const std::vector<T> &v) {
 struct RequantState {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
-  DevBuf w_blocked;  // built by the first run with 3..16 activation rows
+  DevBuf w_blocked;  // built by the first run with 3..32 activation rows
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
   bool has_zw = false, fast = false;

@@ -1,5 +1,6 @@
-// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 16 activation rows
-// against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw) (v_dot4 kernel for M <= 2, matrix-core kernel for 3 <= M <= 16).  The kernel is HBM-bound on the weight stream, so the design goal
+// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 32 activation rows
+// against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw): a v_dot4 kernel for M <= 2, a
+// matrix-core kernel for 3 <= M <= 32.  The kernels are HBM-bound on the weight stream, so the design goal
 // is "every weight byte crosses HBM once, in 1 KiB coalesced wave loads, with enough loads in flight":
 //   - a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes);
 //   - it keeps D 16-byte loads per lane (D KiB per wave) in flight at all times, refilling a register slot as soon
@@ -229,7 +230,8 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 }
 
 // =====================================================================================================================
-// 3 <= M <= 16 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
+// 3 <= M <= 32 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M
+// (MG = 1 up to 16 rows, MG = 2 row groups of 16 above).
 // v_mfma_i32_16x16x64_i8 with the WEIGHTS as the 16-row operand: lane (g = lane / 16, i = lane % 16) supplies 16
 // contiguous K bytes of weight row i (K offset 16 g inside the 64-byte step) and the same 16 K bytes of activation row
 // i (zero for i >= M); the result register r of that lane is output (channel 4 g + r, activation row i).
@@ -240,10 +242,10 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 // A workgroup of 8 waves owns RG x 16 channels; the waves split K into contiguous slices, each wave keeps D steps
 // (D x RG KiB of weights) in flight, and the partial sums meet in LDS.
 // =====================================================================================================================
-template <int RG, int D>
+template <int RG, int D, int MG>
 __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, RequantParams rq) {
   constexpr int WAVES = 8;
-  __shared__ v4i red[WAVES][RG + 1][64];
+  __shared__ v4i red[WAVES][(RG + 1) * MG][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane >> 4, idx = lane & 15;
   const int n0 = blockIdx.x * (RG * 16);
@@ -254,8 +256,13 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, 
   // blocked weights: 1 KiB block (row group, step) = 16 rows x 64 bytes, chunk of lane (grp, idx) = row idx, K chunk
   // grp at position lane
   const int8_t *wbase = g.w + (int64_t)(n0 >> 4) * total * 1024 + lane * 16;
-  const int arow = idx < m_rows ? idx : m_rows - 1;
-  const int8_t *abase = g.a + (int64_t)arow * g.lda;
+  // activation rows of this lane: idx + 16 * mg (a row past the last one re-reads the last and is zeroed)
+  const int8_t *abase[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) {
+    const int row = idx + 16 * mg;
+    abase[mg] = g.a + (int64_t)(row < m_rows ? row : m_rows - 1) * g.lda;
+  }
 
   // the finishing lanes (first RG waves) fetch their channels' parameters while the weights stream
   int32_t p_mult[4], p_e[4], p_ls[4], p_bias2[4], p_zw[4];
@@ -276,45 +283,60 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, 
     s = s < total ? s : total - 1;
     return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wbase + ((int64_t)rg * total + s) * 1024));
   };
-  auto load_x = [&](int j) -> v4i {
+  auto load_x = [&](int j, int mg) -> v4i {
     int off = (s0 + j) * 64 + grp * 16;
     off = off < k_bytes ? off : k_bytes - 16;
-    return *reinterpret_cast<const v4i *>(abase + off);
+    return *reinterpret_cast<const v4i *>(abase[mg] + off);
   };
-  v4i wbuf[D][RG], xbuf[D];
+  v4i wbuf[D][RG], xbuf[D][MG];
 #pragma unroll
   for (int j = 0; j < D; ++j) {
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(j, rg);
-    xbuf[j] = load_x(j);
+#pragma unroll
+    for (int mg = 0; mg < MG; ++mg) xbuf[j][mg] = load_x(j, mg);
   }
 
-  v4i acc[RG], asum = {0, 0, 0, 0};
+  v4i acc[RG][MG], asum[MG];
 #pragma unroll
-  for (int rg = 0; rg < RG; ++rg) acc[rg] = v4i{0, 0, 0, 0};
+  for (int mg = 0; mg < MG; ++mg) {
+    asum[mg] = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) acc[rg][mg] = v4i{0, 0, 0, 0};
+  }
   const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
 
   auto pass = [&](int base, auto refill) {
 #pragma unroll
     for (int j = 0; j < D; ++j) {
       const int jj = base + j;
-      const bool live = idx < m_rows && jj < spw && s0 + jj < total && (s0 + jj) * 64 + grp * 16 < k_bytes;
-      v4i x = xbuf[j];
-      x.x = live ? x.x : 0;
-      x.y = live ? x.y : 0;
-      x.z = live ? x.z : 0;
-      x.w = live ? x.w : 0;
+      const bool in_k = jj < spw && s0 + jj < total && (s0 + jj) * 64 + grp * 16 < k_bytes;
+      v4i x[MG];
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) {
+        const bool live = in_k && idx + 16 * mg < m_rows;
+        x[mg] = xbuf[j][mg];
+        x[mg].x = live ? x[mg].x : 0;
+        x[mg].y = live ? x[mg].y : 0;
+        x[mg].z = live ? x[mg].z : 0;
+        x[mg].w = live ? x[mg].w : 0;
+      }
       v4i w[RG];
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];
       if (decltype(refill)::value) {
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(jj + D, rg);
-        xbuf[j] = load_x(jj + D);
+#pragma unroll
+        for (int mg = 0; mg < MG; ++mg) xbuf[j][mg] = load_x(jj + D, mg);
       }
 #pragma unroll
-      for (int rg = 0; rg < RG; ++rg) acc[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x, acc[rg], 0, 0, 0);
-      if (rq.has_zw) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x, asum, 0, 0, 0);
+      for (int mg = 0; mg < MG; ++mg) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg)
+          acc[rg][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x[mg], acc[rg][mg], 0, 0, 0);
+        if (rq.has_zw) asum[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x[mg], asum[mg], 0, 0, 0);
+      }
     }
   };
   int base = 0;
@@ -322,47 +344,54 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, 
   pass(base, std::false_type());
 
 #pragma unroll
-  for (int rg = 0; rg < RG; ++rg) red[wave][rg][lane] = acc[rg];
-  red[wave][RG][lane] = asum;
+  for (int mg = 0; mg < MG; ++mg) {
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) red[wave][mg * (RG + 1) + rg][lane] = acc[rg][mg];
+    red[wave][mg * (RG + 1) + RG][lane] = asum[mg];
+  }
   __syncthreads();
   if (wave < RG) {
-    v4i tot = {0, 0, 0, 0}, xs = {0, 0, 0, 0};
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
-      tot += red[w][wave][lane];
-      xs += red[w][RG][lane];
-    }
-    if (idx < m_rows) {
-      const int nb = n0 + wave * 16 + 4 * grp;
-      int8_t outv[4];
+    for (int mg = 0; mg < MG; ++mg) {
+      v4i tot = {0, 0, 0, 0}, xs = {0, 0, 0, 0};
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        uint32_t v = (uint32_t)tot[r];
-        if (rq.has_zw) v -= (uint32_t)xs[0] * (uint32_t)p_zw[r];
-        v += (uint32_t)p_bias2[r];
-        int32_t y;
-        if (rq.fast) {
-          y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[r]), p_e[r], (1 << p_e[r]) >> 1);
-        } else {
-          y = rdiv_pot(srdhm((int32_t)(v << p_ls[r]), p_mult[r]), p_e[r]);
-        }
-        y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
-        y = y < rq.amax ? y : rq.amax;
-        y = y > rq.amin ? y : rq.amin;
-        outv[r] = (int8_t)y;
+      for (int w = 0; w < WAVES; ++w) {
+        tot += red[w][mg * (RG + 1) + wave][lane];
+        xs += red[w][mg * (RG + 1) + RG][lane];
       }
-      int8_t *dst = g.c + (int64_t)idx * g.ldc + nb;
+      const int row = idx + 16 * mg;
+      if (row < m_rows) {
+        const int nb = n0 + wave * 16 + 4 * grp;
+        int8_t outv[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (nb + r < g.n) dst[r] = outv[r];
+        for (int r = 0; r < 4; ++r) {
+          uint32_t v = (uint32_t)tot[r];
+          if (rq.has_zw) v -= (uint32_t)xs[0] * (uint32_t)p_zw[r];
+          v += (uint32_t)p_bias2[r];
+          int32_t y;
+          if (rq.fast) {
+            y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[r]), p_e[r], (1 << p_e[r]) >> 1);
+          } else {
+            y = rdiv_pot(srdhm((int32_t)(v << p_ls[r]), p_mult[r]), p_e[r]);
+          }
+          y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+          y = y < rq.amax ? y : rq.amax;
+          y = y > rq.amin ? y : rq.amin;
+          outv[r] = (int8_t)y;
+        }
+        int8_t *dst = g.c + (int64_t)row * g.ldc + nb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (nb + r < g.n) dst[r] = outv[r];
+      }
     }
   }
 }
 
-template <int RG, int D>
+template <int RG, int D, int MG = 1>
 static int launch_mfma(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
   const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
-  hipLaunchKernelGGL((gemv_mfma_kernel<RG, D>), dim3(blocks), dim3(512), 0, stream, g, m, rq);
+  hipLaunchKernelGGL((gemv_mfma_kernel<RG, D, MG>), dim3(blocks), dim3(512), 0, stream, g, m, rq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -412,6 +441,10 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
     g.w = wv.blocked;
     // two 16-channel groups per workgroup (half the activation traffic) once there are enough channels to fill the
     // device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (m > 16) {  // two groups of 16 activation rows against every weight fragment
+      if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4, 2>(g, m, rq, stream);
+      return launch_mfma<1, 8, 2>(g, m, rq, stream);
+    }
     if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4>(g, m, rq, stream);
     return launch_mfma<1, 8>(g, m, rq, stream);
   }

@@ -68,12 +68,13 @@ def test_matmul_shapes(orc, m, n, k):
 
 @pytest.mark.parametrize("n,k", [(40, 2048), (24, 4000), (16, 5008), (9, 13008), (8200, 1040), (8196, 208)])
 def test_decode_rows_every_stream_shape(orc, n, k):
-    """1..16 activation rows (v_dot4 kernel up to 2, matrix-core kernel above) against every weight-stream shape the
+    """1..32 activation rows (v_dot4 kernel up to 2, matrix-core kernel above: one group of 16 rows up to 16, two
+    groups up to 32) and the first row counts of the GEMM path, against every weight-stream shape the
     skinny path distinguishes: rows of one, two, up to four and more 1 KiB segments, a stream longer than the
     in-flight queue, few and many output channels."""
     rng = np.random.default_rng(n * 131 + k)
     orc.set_threads(16)
-    for m in range(1, 17):
+    for m in list(range(1, 19)) + [23, 31, 32, 33, 40]:
         case = _mm_case(rng, m, n, k, bool(m & 1), bool(m & 2), m != 4, [0, 1, 3][m % 3])
         got, _ = _gpu_matmul(case, device_tensors=bool(m & 4))
         want = orc.matmul_int8(**case)
