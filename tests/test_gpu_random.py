@@ -105,3 +105,29 @@ def test_random_depthwise(orc, seed):
         ran += 1
         assert np.array_equal(got, orc.conv_dw_int8(**case)), (seed, it, b, ih, iw, c, kh, kw, stride, dil, pad)
     assert ran > 200
+
+
+@pytest.mark.parametrize("seed", [6])
+def test_random_matmul_large_tiles(orc, seed):
+    """Shapes large enough for every tile configuration of the GEMM (64, 128 with two and three workgroups per CU,
+    256 x 128, 256 x 256), int8 and fp32 epilogues, random flags."""
+    rng = np.random.default_rng(seed)
+    orc.set_threads(16)
+    shapes = [(2100, 1300, 48), (2048 + 37, 2048 + 4, 272), (4224, 2100, 144), (4100, 2700, 1040), (4096, 3100, 80),
+              (4500, 3600, 16), (300, 11008, 80), (512, 8200, 272), (700, 640, 3000), (1500, 1500, 1024)]
+    for it, (m, n, k) in enumerate(shapes):
+        case = T._mm_case(rng, m, n, k, _flag(rng), _flag(rng), _flag(rng), _pick(rng, [0, 1, 3]), _flag(rng))
+        got, _ = T._gpu_matmul(case, device_tensors=True)
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (seed, it, m, n, k, int((got != want).sum()))
+        # the same operands through the fp32 (dynamic MatMul) epilogue
+        w_nk = case["w"] if case["b_transpose"] else np.ascontiguousarray(case["w"].T)
+        sw, zw = case["sw"], case["zw"]
+        if len(zw) > 1:
+            zw = np.zeros_like(zw)  # per-channel dynamic weights are symmetric in the reference
+        bias = rng.standard_normal(n).astype(np.float32) if _flag(rng) else None
+        act = _pick(rng, [0, 1, 3])
+        kern = K.MatmulDynamicInt8Kernel(w_nk, bias, T._qps(sw, zw), True, act)
+        wantf = orc.dynamic_matmul(case["a"], w_nk, bias, 0.037, case["zx"], sw, zw, act, True)
+        gotf = kern.run(case["a"], K.QuantParam(0.037, case["zx"]))
+        assert np.array_equal(gotf.view(np.uint32), wantf.view(np.uint32)), (seed, it, m, n, k, "fp32")
