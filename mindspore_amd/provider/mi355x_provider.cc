@@ -9,8 +9,10 @@
 //
 // It needs a MindSpore Lite SDK to compile (register_kernel.h includes the flatc-generated schema/model_generated.h)
 // and is therefore not part of the library build:
-//   g++ -std=c++17 -fPIC -shared mi355x_provider.cc -I<lite-sdk>/runtime -I<repo>/include \
+//   g++ -std=c++17 -fPIC -shared mi355x_provider.cc -I<lite-sdk>/runtime -I<repo>/include
 //       -L<lite-sdk>/runtime/lib -lmindspore-lite -L<repo>/mindspore_amd -lmi355x_int8 -o libmi355x_provider.so
+// Without an SDK the tests compile it against hand-written stand-ins of those headers (tests/lite_stub) and drive it
+// through a harness that plays the scheduler.
 // An application selects it with CPUDeviceInfo::SetProvider("mi355x") (+ SetProviderDevice("CPU")); the stock
 // benchmark tool with --provider=mi355x (it leaves the provider device empty, hence the second registration under "").
 //

@@ -1,0 +1,191 @@
+// TEST INFRASTRUCTURE.  Plays the part of the Lite scheduler for mindspore_amd/provider/mi355x_provider.cc, compiled
+// against the stand-in API of this directory: looks the creator up by (arch, provider, data type, op type) as
+// scheduler.cc:1131-1177 does, runs the provider's shape inference, Prepare / ReSize / Execute, and hands tensors in
+// and out through a C interface for the Python tests.  The provider source is included, so its static registrar
+// runs when this library is loaded.
+#include <string.h>
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../../mindspore_amd/provider/mi355x_provider.cc"
+
+using mindspore::MSTensor;
+namespace schema = mindspore::schema;
+
+extern "C" {
+typedef struct ph_tensor {
+  int32_t dtype;  // mindspore::DataType id
+  int32_t dims;
+  int64_t shape[8];
+  const void *data;  // NULL: not materialised (an activation before the first run)
+  int64_t bytes;
+  int32_t is_const;
+  int32_t nquant;
+  const double *scales;
+  const int32_t *zps;
+} ph_tensor;
+
+typedef struct ph_op {
+  int32_t type;  // schema::PrimitiveType id
+  int32_t transpose_a, transpose_b, act;
+  int32_t has_bias, use_axis, axis;
+  int64_t kernel[2], stride[2], dilation[2], pad_list[4];
+  int32_t has_pad_list, pad_mode;
+  int64_t group, in_channel, out_channel;
+  int32_t symmetric;
+  int64_t dst_type;
+  int32_t n_prefer_axes;
+  int32_t prefer_axes[8];
+} ph_op;
+}
+
+namespace {
+enum Stage { kOk = 0, kNoCreator = 1, kDeclined = 2, kInferFailed = 3, kPrepareFailed = 4, kResizeFailed = 5, kExecuteFailed = 6 };
+
+struct Session {
+  schema::Primitive prim;
+  std::vector<MSTensor> inputs, outputs;
+  std::shared_ptr<mindspore::kernel::Kernel> kernel;
+  std::shared_ptr<mindspore::kernel::KernelInterface> infer;
+  mindspore::Context ctx;
+};
+
+std::vector<mindspore::QuantParam> Quant(int n, const double *scales, const int32_t *zps) {
+  std::vector<mindspore::QuantParam> q;
+  for (int i = 0; i < n; ++i) q.push_back({8, scales[i], zps[i], 0.0, 0.0});
+  return q;
+}
+
+MSTensor Tensor(const ph_tensor &t, const std::string &name) {
+  MSTensor ms(name, static_cast<mindspore::DataType>(t.dtype), std::vector<int64_t>(t.shape, t.shape + t.dims), t.data,
+              static_cast<size_t>(t.bytes), t.is_const != 0);
+  ms.SetQuantParams(Quant(t.nquant, t.scales, t.zps));
+  return ms;
+}
+
+void Fill(const ph_op &op, schema::Primitive *p) {
+  p->type_ = static_cast<schema::PrimitiveType>(op.type);
+  const auto act = static_cast<schema::ActivationType>(op.act);
+  p->matmul_.transpose_a_ = op.transpose_a != 0;
+  p->matmul_.transpose_b_ = op.transpose_b != 0;
+  p->matmul_.activation_type_ = act;
+  p->fc_.has_bias_ = op.has_bias != 0;
+  p->fc_.use_axis_ = op.use_axis != 0;
+  p->fc_.axis_ = op.axis;
+  p->fc_.activation_type_ = act;
+  p->conv_.kernel_size_ = flatbuffers::Vector<int64_t>({op.kernel[0], op.kernel[1]});
+  p->conv_.stride_ = flatbuffers::Vector<int64_t>({op.stride[0], op.stride[1]});
+  p->conv_.dilation_ = flatbuffers::Vector<int64_t>({op.dilation[0], op.dilation[1]});
+  p->conv_.pad_list_ = flatbuffers::Vector<int64_t>({op.pad_list[0], op.pad_list[1], op.pad_list[2], op.pad_list[3]});
+  p->conv_.has_pad_list_ = op.has_pad_list != 0;
+  p->conv_.pad_mode_ = static_cast<schema::PadMode>(op.pad_mode);
+  p->conv_.group_ = op.group;
+  p->conv_.in_channel_ = op.in_channel;
+  p->conv_.out_channel_ = op.out_channel;
+  p->conv_.activation_type_ = act;
+  p->dynquant_.symmetric_ = op.symmetric != 0;
+  p->dynquant_.dst_type_ = op.dst_type;
+  p->dynquant_.has_prefer_axes_ = op.n_prefer_axes > 0;
+  p->dynquant_.prefer_axes_ = flatbuffers::Vector<int32_t>(std::vector<int32_t>(op.prefer_axes, op.prefer_axes + op.n_prefer_axes));
+}
+
+int Infer(Session *s) {
+  if (s->infer == nullptr) return kOk;  // the builtin inference would run; the tests always register one
+  const mindspore::Status st = s->infer->Infer(&s->inputs, &s->outputs, &s->prim);
+  return st.IsOk() ? kOk : kInferFailed;
+}
+}  // namespace
+
+extern "C" {
+// Builds the node: tensors, shape inference, creator lookup and call, Prepare().  *stage tells how far it got;
+// *code is the status of the failing call (0 otherwise).  Returns NULL unless the kernel is ready to execute.
+void *ph_create(const ph_op *op, const char *arch, const char *provider, const ph_tensor *inputs, int32_t n_in,
+                int32_t out_dtype, int32_t out_nquant, const double *out_scales, const int32_t *out_zps,
+                int32_t *stage, int32_t *code) {
+  auto s = std::make_unique<Session>();
+  *stage = kOk;
+  *code = 0;
+  Fill(*op, &s->prim);
+  for (int i = 0; i < n_in; ++i) s->inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
+  MSTensor out("out", static_cast<mindspore::DataType>(out_dtype), {}, nullptr, 0, false);
+  out.SetQuantParams(Quant(out_nquant, out_scales, out_zps));
+  s->outputs.push_back(out);
+  s->infer = mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &s->prim);
+  if ((*stage = Infer(s.get())) != kOk) return nullptr;
+  mindspore::registry::KernelDesc desc{s->inputs[0].DataType(), op->type, arch, provider};
+  auto creator = mindspore::registry::RegisterKernel::GetCreator(&s->prim, &desc);
+  if (creator == nullptr) {
+    *stage = kNoCreator;
+    return nullptr;
+  }
+  s->kernel = creator(s->inputs, s->outputs, &s->prim, &s->ctx);
+  if (s->kernel == nullptr) {
+    *stage = kDeclined;  // the scheduler would now take the builtin CPU kernel
+    return nullptr;
+  }
+  if ((*code = s->kernel->Prepare()) != 0) {
+    *stage = kPrepareFailed;
+    return nullptr;
+  }
+  return s.release();
+}
+
+// Sets input 0 (new shape allowed: the output shape is inferred again and ReSize() is called, as the runtime does on
+// Model::Resize), optionally its quant params (the dynamic MatMul reads them at every Execute), and executes.
+int32_t ph_execute(void *h, const void *in0, const int64_t *shape, int32_t dims, int32_t nquant, const double *scales,
+                   const int32_t *zps, int32_t *code) {
+  auto *s = static_cast<Session *>(h);
+  *code = 0;
+  MSTensor &x = s->inputs[0];
+  const std::vector<int64_t> new_shape(shape, shape + dims);
+  const bool resized = new_shape != x.Shape();
+  x.SetShape(new_shape);
+  memcpy(x.MutableData(), in0, x.DataSize());
+  if (nquant > 0) x.SetQuantParams(Quant(nquant, scales, zps));
+  if (resized) {
+    if (Infer(s) != kOk) return kInferFailed;
+    if ((*code = s->kernel->ReSize()) != 0) return kResizeFailed;
+  }
+  if ((*code = s->kernel->Execute()) != 0) return kExecuteFailed;
+  return kOk;
+}
+
+// Output tensor as the kernel left it.  Returns the number of data bytes (copied when they fit `cap`).
+int64_t ph_output(void *h, int64_t *shape, int32_t *dims, void *buf, int64_t cap, double *scales, int32_t *zps,
+                  int32_t max_quant, int32_t *nquant) {
+  auto *s = static_cast<Session *>(h);
+  MSTensor &y = s->outputs[0];
+  *dims = static_cast<int32_t>(y.Shape().size());
+  for (int i = 0; i < *dims && i < 8; ++i) shape[i] = y.Shape()[i];
+  const auto q = y.QuantParams();
+  *nquant = static_cast<int32_t>(q.size());
+  for (int i = 0; i < *nquant && i < max_quant; ++i) {
+    scales[i] = q[i].scale;
+    zps[i] = q[i].zero_point;
+  }
+  const int64_t bytes = static_cast<int64_t>(y.DataSize());
+  auto data = y.Data();
+  if (data != nullptr && bytes <= cap) memcpy(buf, data.get(), static_cast<size_t>(bytes));
+  return bytes;
+}
+
+// Shape inference alone (no GPU needed): output dims, or -1 on failure, -2 while a dimension is unknown.
+int32_t ph_infer(const ph_op *op, const char *provider, const ph_tensor *inputs, int32_t n_in, int64_t *shape) {
+  Session s;
+  Fill(*op, &s.prim);
+  for (int i = 0; i < n_in; ++i) s.inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
+  s.outputs.push_back(MSTensor("out", mindspore::DataType::kNumberTypeInt8, {}, nullptr, 0, false));
+  auto iface = mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &s.prim);
+  if (iface == nullptr) return -3;
+  const mindspore::Status st = iface->Infer(&s.inputs, &s.outputs, &s.prim);
+  if (st == mindspore::kLiteInferInvalid) return -2;
+  if (!st.IsOk()) return -1;
+  const auto &out = s.outputs[0].Shape();
+  for (size_t i = 0; i < out.size() && i < 8; ++i) shape[i] = out[i];
+  return static_cast<int32_t>(out.size());
+}
+
+void ph_destroy(void *h) { delete static_cast<Session *>(h); }
+}

@@ -1,0 +1,295 @@
+"""The MindSpore Lite provider (mindspore_amd/provider/mi355x_provider.cc) without a Lite SDK:
+  * compiled against the reference's own public headers, with only the flatc-generated schema header replaced by a
+    hand-written stand-in (CPU, needs the reference tree);
+  * compiled against the stand-in Lite API of tests/lite_stub and driven by a harness that plays the scheduler:
+    creator lookup by (arch, provider, data type, op type), shape inference, Prepare / ReSize / Execute.  On the CPU
+    every creator must decline (no gfx950: the scheduler would fall back to the builtin kernels); on the GPU the outputs
+    must equal the oracle's, as for the C ABI itself."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from tests.lite_stub import build as stub_build
+
+I8, I32, F32 = 32, 34, 43
+MATMUL, FC, CONV, DYNQUANT = 89, 67, 35, 203
+OK, NO_CREATOR, DECLINED, INFER_FAILED, PREPARE_FAILED, RESIZE_FAILED, EXECUTE_FAILED = range(7)
+
+
+class PhTensor(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("dims", C.c_int32), ("shape", C.c_int64 * 8), ("data", C.c_void_p),
+                ("bytes", C.c_int64), ("is_const", C.c_int32), ("nquant", C.c_int32),
+                ("scales", C.POINTER(C.c_double)), ("zps", C.POINTER(C.c_int32))]
+
+
+class PhOp(C.Structure):
+    _fields_ = [("type", C.c_int32), ("transpose_a", C.c_int32), ("transpose_b", C.c_int32), ("act", C.c_int32),
+                ("has_bias", C.c_int32), ("use_axis", C.c_int32), ("axis", C.c_int32),
+                ("kernel", C.c_int64 * 2), ("stride", C.c_int64 * 2), ("dilation", C.c_int64 * 2),
+                ("pad_list", C.c_int64 * 4), ("has_pad_list", C.c_int32), ("pad_mode", C.c_int32),
+                ("group", C.c_int64), ("in_channel", C.c_int64), ("out_channel", C.c_int64),
+                ("symmetric", C.c_int32), ("dst_type", C.c_int64), ("n_prefer_axes", C.c_int32),
+                ("prefer_axes", C.c_int32 * 8)]
+
+
+@pytest.fixture(scope="module")
+def H():
+    from mindspore_amd import lib
+    lib.load()  # maps the HIP runtime and libmi355x_int8.so first
+    if not os.path.exists(stub_build.OUT):
+        stub_build.build_harness()
+    h = C.CDLL(stub_build.OUT)
+    h.ph_create.restype = C.c_void_p
+    h.ph_create.argtypes = [C.POINTER(PhOp), C.c_char_p, C.c_char_p, C.POINTER(PhTensor), C.c_int32, C.c_int32,
+                            C.c_int32, C.POINTER(C.c_double), C.POINTER(C.c_int32), C.POINTER(C.c_int32),
+                            C.POINTER(C.c_int32)]
+    h.ph_execute.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int32, C.c_int32,
+                             C.POINTER(C.c_double), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]
+    h.ph_output.restype = C.c_int64
+    h.ph_output.argtypes = [C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_void_p, C.c_int64,
+                            C.POINTER(C.c_double), C.POINTER(C.c_int32), C.c_int32, C.POINTER(C.c_int32)]
+    h.ph_infer.argtypes = [C.POINTER(PhOp), C.c_char_p, C.POINTER(PhTensor), C.c_int32, C.POINTER(C.c_int64)]
+    h.ph_destroy.argtypes = [C.c_void_p]
+    h.ph_destroy.restype = None
+    return h
+
+
+_keep = []  # ctypes buffers referenced by PhTensor structs
+
+
+def tensor(dtype, shape, data=None, const=False, quant=()):
+    t = PhTensor()
+    t.dtype, t.dims, t.is_const = dtype, len(shape), int(const)
+    for i, d in enumerate(shape):
+        t.shape[i] = d
+    if data is not None:
+        data = np.ascontiguousarray(data)
+        _keep.append(data)
+        t.data, t.bytes = data.ctypes.data, data.nbytes
+    scales = (C.c_double * max(len(quant), 1))(*[float(q[0]) for q in quant])
+    zps = (C.c_int32 * max(len(quant), 1))(*[int(q[1]) for q in quant])
+    _keep.extend([scales, zps])
+    t.nquant, t.scales, t.zps = len(quant), scales, zps
+    return t
+
+
+def op(type_, **kw):
+    o = PhOp()
+    o.type = type_
+    o.dst_type = I8
+    o.group = 1
+    for k, v in kw.items():
+        if isinstance(v, (tuple, list)):
+            arr = getattr(o, k)
+            for i, x in enumerate(v):
+                arr[i] = x
+        else:
+            setattr(o, k, v)
+    return o
+
+
+class Node:
+    def __init__(self, H, o, inputs, out_dtype, out_quant=(), arch=b"CPU", provider=b"mi355x"):
+        self.H = H
+        arr = (PhTensor * len(inputs))(*inputs)
+        scales = (C.c_double * max(len(out_quant), 1))(*[float(q[0]) for q in out_quant])
+        zps = (C.c_int32 * max(len(out_quant), 1))(*[int(q[1]) for q in out_quant])
+        stage, code = C.c_int32(-1), C.c_int32(0)
+        self.h = H.ph_create(C.byref(o), arch, provider, arr, len(inputs), out_dtype, len(out_quant), scales, zps,
+                             C.byref(stage), C.byref(code))
+        self.stage, self.code, self.out_dtype = stage.value, code.value, out_dtype
+
+    def run(self, x, quant=()):
+        x = np.ascontiguousarray(x)
+        shape = (C.c_int64 * x.ndim)(*x.shape)
+        scales = (C.c_double * max(len(quant), 1))(*[float(q[0]) for q in quant])
+        zps = (C.c_int32 * max(len(quant), 1))(*[int(q[1]) for q in quant])
+        code = C.c_int32(0)
+        st = self.H.ph_execute(self.h, x.ctypes.data, shape, x.ndim, len(quant), scales, zps, C.byref(code))
+        assert st == OK, (st, code.value)
+        oshape, dims, nq = (C.c_int64 * 8)(), C.c_int32(0), C.c_int32(0)
+        qs, qz = (C.c_double * 65536)(), (C.c_int32 * 65536)()
+        nbytes = self.H.ph_output(self.h, oshape, C.byref(dims), None, 0, qs, qz, 65536, C.byref(nq))
+        out = np.empty(nbytes, np.uint8)
+        self.H.ph_output(self.h, oshape, C.byref(dims), out.ctypes.data, nbytes, qs, qz, 65536, C.byref(nq))
+        np_dtype = {I8: np.int8, F32: np.float32}[self.out_dtype]
+        y = out.view(np_dtype).reshape([oshape[i] for i in range(dims.value)])
+        return y, [(qs[i], qz[i]) for i in range(nq.value)]
+
+    def close(self):
+        if self.h:
+            self.H.ph_destroy(self.h)
+            self.h = None
+
+
+def _fc_inputs(rng, m, n, k, bias=True, w_const=True):
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
+    b = rng.integers(-5000, 5001, n).astype(np.int32) if bias else None
+    ins = [tensor(I8, (m, k), None, False, [(0.02, -3)]),
+           tensor(I8, (n, k), w, w_const, [(s, 0) for s in sw])]
+    if bias:
+        ins.append(tensor(I32, (n,), b, True))
+    return a, w, sw, b, ins
+
+
+# ---------------------------------------------------------------------------------------------------- CPU
+def test_provider_compiles_against_reference_headers():
+    out = stub_build.syntax_check_against_reference_headers()
+    if out is None:
+        pytest.skip("reference tree absent")
+    assert out == "", out
+
+
+def test_shape_inference_through_the_provider(H):
+    shp = (C.c_int64 * 8)()
+    ins = (PhTensor * 2)(tensor(I8, (2, 5, 128), None), tensor(I8, (96, 128), None, True))
+    assert H.ph_infer(C.byref(op(MATMUL, transpose_b=1)), b"mi355x", ins, 2, shp) == 3 and list(shp[:3]) == [2, 5, 96]
+    assert H.ph_infer(C.byref(op(FC)), b"mi355x", ins, 2, shp) == 2 and list(shp[:2]) == [10, 96]
+    ins = (PhTensor * 2)(tensor(I8, (1, 224, 224, 3), None), tensor(I8, (32, 3, 3, 3), None, True))
+    conv = op(CONV, kernel=(3, 3), stride=(2, 2), dilation=(1, 1), pad_mode=1, in_channel=3, out_channel=32)
+    assert H.ph_infer(C.byref(conv), b"mi355x", ins, 2, shp) == 4 and list(shp[:4]) == [1, 112, 112, 32]
+    ins = (PhTensor * 2)(tensor(I8, (1, -1, 224, 3), None), tensor(I8, (32, 3, 3, 3), None, True))
+    assert H.ph_infer(C.byref(conv), b"mi355x", ins, 2, shp) == -2          # unknown dimension: infer again later
+    ins = (PhTensor * 2)(tensor(I8, (4, 7), None), tensor(I8, (96, 128), None, True))
+    assert H.ph_infer(C.byref(op(MATMUL, transpose_b=1)), b"mi355x", ins, 2, shp) == -1
+    ins = (PhTensor * 1)(tensor(F32, (3, 4, 5), None))
+    assert H.ph_infer(C.byref(op(DYNQUANT)), b"mi355x", ins, 1, shp) == 3 and list(shp[:3]) == [3, 4, 5]
+    assert H.ph_infer(C.byref(op(DYNQUANT)), b"other", ins, 1, shp) == -3     # nothing registered for that provider
+
+
+def test_registration_keys_and_decline_without_a_gpu(H):
+    """Both arch keys are registered ("CPU" for applications, "" for the stock benchmark tool); an unknown key has no
+    creator; without a gfx950 device every creator declines, so the scheduler would use the builtin kernels."""
+    import torch
+    rng = np.random.default_rng(0)
+    a, w, sw, b, ins = _fc_inputs(rng, 4, 8, 16)
+    node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], arch=b"GPU")
+    assert node.stage == NO_CREATOR
+    node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], provider=b"someone")
+    assert node.stage == NO_CREATOR
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present: the creators accept")
+    for arch in (b"CPU", b""):
+        node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], arch=arch)
+        assert node.stage == DECLINED and node.h is None
+
+
+# ---------------------------------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+def test_fullconnection_and_matmul_through_the_provider(H, orc):
+    rng = np.random.default_rng(1)
+    for arch in (b"CPU", b""):
+        a, w, sw, b, ins = _fc_inputs(rng, 128, 768, 768)
+        node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], arch=arch)
+        assert node.stage == OK, (node.stage, node.code)
+        y, _ = node.run(a)
+        want = orc.matmul_int8(a, w, b, 0.02, -3, sw, np.zeros(768, np.int32), 0.05, 5, 0, True)
+        assert y.shape == (128, 768) and np.array_equal(y, want)
+        # another row count through the same kernel: ReSize + Execute
+        a2 = rng.integers(-128, 128, (5, 768), dtype=np.int8)
+        y2, _ = node.run(a2)
+        assert np.array_equal(y2, orc.matmul_int8(a2, w, b, 0.02, -3, sw, np.zeros(768, np.int32), 0.05, 5, 0, True))
+        node.close()
+    # MatMulFusion with a [K, N] weight, ReLU6, 3-D activation
+    k, n = 100, 36
+    a = rng.integers(-128, 128, (2, 7, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    ins = [tensor(I8, a.shape, None, False, [(0.03, 4)]), tensor(I8, (k, n), w, True, [(0.004, 2)])]
+    node = Node(H, op(MATMUL, transpose_b=0, act=3), ins, I8, [(0.04, -7)])
+    assert node.stage == OK
+    y, _ = node.run(a)
+    want = orc.matmul_int8(a.reshape(14, k), w, None, 0.03, 4, np.array([0.004]), np.array([2], np.int32), 0.04, -7, 3,
+                           False)
+    assert y.shape == (2, 7, n) and np.array_equal(y.reshape(14, n), want)
+    node.close()
+
+
+@pytest.mark.gpu
+def test_what_the_provider_declines(H):
+    rng = np.random.default_rng(2)
+    a, w, sw, b, ins = _fc_inputs(rng, 4, 8, 16, w_const=False)            # weight produced at run time
+    assert Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)]).stage == DECLINED
+    a, w, sw, b, ins = _fc_inputs(rng, 4, 8, 16)
+    assert Node(H, op(MATMUL, transpose_a=1, transpose_b=1), ins, I8, [(0.05, 5)]).stage in (DECLINED, INFER_FAILED)
+    assert Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5), (0.06, 5)]).stage == DECLINED   # per-channel output
+    x = tensor(I8, (1, 8, 8, 4), None, False, [(0.02, 1)])
+    wc = tensor(I8, (8, 3, 3, 4), rng.integers(-128, 128, (8, 3, 3, 4), dtype=np.int8), True, [(0.01, 0)])
+    conv = op(CONV, kernel=(3, 3), stride=(1, 1), dilation=(1, 1), pad_mode=1, in_channel=4, out_channel=8)
+    assert Node(H, conv, [x, wc], I8, [(0.05, 0)]).stage == DECLINED       # dense 3x3 stride 1: Winograd on the CPU
+    dq = op(DYNQUANT, n_prefer_axes=1, prefer_axes=(1,))
+    assert Node(H, dq, [tensor(F32, (4, 6, 8), None)], I8).stage == DECLINED  # would need the transposition
+
+
+@pytest.mark.gpu
+def test_conv_through_the_provider_with_resize(H, orc):
+    from oracle.pyoracle import conv_shape
+    rng = np.random.default_rng(3)
+    ic, oc = 3, 32
+    w = rng.integers(-128, 128, (oc, 3, 3, ic), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, oc).astype(np.float32).astype(np.float64)
+    bias = rng.integers(-3000, 3001, oc).astype(np.int32)
+    conv = op(CONV, kernel=(3, 3), stride=(2, 2), dilation=(1, 1), pad_mode=1, in_channel=ic, out_channel=oc, act=3)
+    ins = [tensor(I8, (1, 224, 224, ic), None, False, [(0.02, 3)]), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+           tensor(I32, (oc,), bias, True)]
+    node = Node(H, conv, ins, I8, [(0.03, -10)])
+    assert node.stage == OK, (node.stage, node.code)
+    for b, ih, iw, pad in [(1, 224, 224, (0, 1, 0, 1)), (2, 33, 17, (1, 1, 1, 1)), (1, 224, 224, (0, 1, 0, 1))]:
+        x = rng.integers(-128, 128, (b, ih, iw, ic), dtype=np.int8)
+        y, _ = node.run(x)          # SAME padding moves with the image size: ReSize rebuilds the handle
+        shape = conv_shape(b, ih, iw, ic, oc, (3, 3), (2, 2), (1, 1), pad)
+        want = orc.conv_int8(x, w, bias, shape, 0.02, 3, sw, np.zeros(oc, np.int32), 0.03, -10, 3)
+        assert y.shape == want.shape and np.array_equal(y, want), (b, ih, iw)
+    node.close()
+    # depthwise 3x3 and a 1x1 with explicit padding
+    c = 16
+    wd = rng.integers(-128, 128, (c, 3, 3, 1), dtype=np.int8)
+    swd = rng.uniform(1e-3, 1e-2, c).astype(np.float32).astype(np.float64)
+    dw = op(CONV, kernel=(3, 3), stride=(1, 1), dilation=(1, 1), pad_mode=0, pad_list=(1, 1, 1, 1), has_pad_list=1,
+            group=c, in_channel=c, out_channel=c)
+    node = Node(H, dw, [tensor(I8, (1, 12, 12, c), None, False, [(0.02, -4)]),
+                        tensor(I8, wd.shape, wd, True, [(s, 0) for s in swd])], I8, [(0.01, 2)])
+    assert node.stage == OK, (node.stage, node.code)
+    x = rng.integers(-128, 128, (1, 12, 12, c), dtype=np.int8)
+    y, _ = node.run(x)
+    shape = conv_shape(1, 12, 12, c, c, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1))
+    want = orc.conv_dw_int8(x, wd.reshape(c, 3, 3), None, shape, 0.02, -4, swd, np.zeros(c, np.int32), 0.01, 2, 0)
+    assert np.array_equal(y, want)
+    node.close()
+
+
+@pytest.mark.gpu
+def test_dynamic_quant_and_dynamic_matmul_through_the_provider(H, orc):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((37, 96)) * 2).astype(np.float32)
+    w = rng.integers(-127, 128, (80, 96), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, 80).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(80).astype(np.float32)
+    zw = np.zeros(80, np.int32)
+    mm_ins = lambda: [tensor(I8, (37, 96), None), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+                      tensor(F32, (80,), bias, True)]
+    # per tensor: DynamicQuant writes {scale, zero point} onto its output tensor; the MatMul reads them at Execute
+    dq = Node(H, op(DYNQUANT), [tensor(F32, x.shape, None)], I8)
+    assert dq.stage == OK, (dq.stage, dq.code)
+    q, qp = dq.run(x)
+    q_ref, s_ref, z_ref = orc.dynamic_quant(x, False)
+    assert np.array_equal(q, q_ref) and qp == [(s_ref, z_ref)]
+    mm = Node(H, op(MATMUL, transpose_b=1), mm_ins(), F32)
+    assert mm.stage == OK, (mm.stage, mm.code)
+    y, _ = mm.run(q, qp)
+    want = orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    # per row (prefer_axes = the leading axis), symmetric as the converter emits it
+    dqr = Node(H, op(DYNQUANT, symmetric=1, n_prefer_axes=1, prefer_axes=(0,)), [tensor(F32, x.shape, None)], I8)
+    assert dqr.stage == OK, (dqr.stage, dqr.code)
+    qr, qpr = dqr.run(x)
+    qr_ref, scales_ref, zps_ref = orc.dynamic_quant_segments(x, True)
+    assert np.array_equal(qr, qr_ref) and [p[0] for p in qpr] == list(scales_ref) and all(p[1] == 0 for p in qpr)
+    yr, _ = mm.run(qr, qpr)
+    wantr = orc.dynamic_matmul_rows(qr_ref, w, bias, scales_ref, 0, sw, zw)
+    assert np.array_equal(yr.view(np.uint32), wantr.view(np.uint32))
+    for n in (dq, mm, dqr):
+        n.close()
