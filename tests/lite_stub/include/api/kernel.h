@@ -1,4 +1,6 @@
-// TEST INFRASTRUCTURE.  Stand-in for include/api/kernel.h (:29-55): kernel::Kernel over schema::Primitive.
+// TEST INFRASTRUCTURE.  Stand-in for include/api/kernel.h: the base class a provider kernel derives from, bound to
+// the schema's Primitive.  Only construction is needed here; the reference class (:29-55) also carries the op and
+// quant type, which no provider kernel of this repository reads.
 #ifndef TESTS_LITE_STUB_INCLUDE_API_KERNEL_H_
 #define TESTS_LITE_STUB_INCLUDE_API_KERNEL_H_
 #include <vector>
@@ -11,19 +13,9 @@
 namespace mindspore::kernel {
 class Kernel : public IKernel<schema::Primitive> {
  public:
-  Kernel() = default;
-  Kernel(const std::vector<mindspore::MSTensor> &inputs, const std::vector<mindspore::MSTensor> &outputs,
-         const schema::Primitive *primitive, const mindspore::Context *ctx)
-      : IKernel<schema::Primitive>(inputs, outputs, primitive, ctx) {
-    if (primitive != nullptr) type_ = primitive->value_type();
-  }
-  virtual ~Kernel() = default;
-  virtual schema::PrimitiveType type() const { return type_; }
-  virtual schema::QuantType quant_type() const { return quant_type_; }
-
- protected:
-  schema::PrimitiveType type_ = schema::PrimitiveType_NONE;
-  schema::QuantType quant_type_ = schema::QuantType_QUANT_NONE;  // never populated by the runtime either
+  Kernel(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out, const schema::Primitive *prim,
+         const Context *ctx)
+      : IKernel<schema::Primitive>(in, out, prim, ctx) {}
 };
 }  // namespace mindspore::kernel
 #endif  // TESTS_LITE_STUB_INCLUDE_API_KERNEL_H_

@@ -1,28 +1,18 @@
-// TEST INFRASTRUCTURE.  Stand-in for mindspore/lite/include/kernel_interface.h (:29-59).
+// TEST INFRASTRUCTURE.  Stand-in for mindspore/lite/include/kernel_interface.h: the one virtual a provider overrides
+// to answer shape inference (reference :29-59, which also has an overload that receives the kernel).
 #ifndef TESTS_LITE_STUB_INCLUDE_KERNEL_INTERFACE_H_
 #define TESTS_LITE_STUB_INCLUDE_KERNEL_INTERFACE_H_
-#include <memory>
 #include <vector>
 
 #include "include/api/status.h"
 #include "include/api/types.h"
 #include "schema/model_generated.h"
 
-namespace mindspore {
-namespace kernel {
-class Kernel;
+namespace mindspore::kernel {
 class KernelInterface {
  public:
   virtual ~KernelInterface() = default;
-  virtual Status Infer(std::vector<mindspore::MSTensor> *inputs, std::vector<mindspore::MSTensor> *outputs,
-                       const schema::Primitive *primitive) {
-    return kSuccess;
-  }
-  virtual Status Infer(std::vector<mindspore::MSTensor> *inputs, std::vector<mindspore::MSTensor> *outputs,
-                       const schema::Primitive *primitive, const Kernel *kernel) {
-    return Infer(inputs, outputs, primitive);
-  }
+  virtual Status Infer(std::vector<MSTensor> *inputs, std::vector<MSTensor> *outputs, const schema::Primitive *prim) = 0;
 };
-}  // namespace kernel
-}  // namespace mindspore
+}  // namespace mindspore::kernel
 #endif  // TESTS_LITE_STUB_INCLUDE_KERNEL_INTERFACE_H_
