@@ -255,27 +255,37 @@ def bench_small_configs(steps, warmup):
 
 def cpu_baseline(case, size):
     """nnacl's CPU path (compiled from the reference tree, oracle/_ref) -- or the restatement if that library did
-    not travel -- on a bounded sample: the first `rows` activation rows of the same GEMM, all host cores."""
+    not travel -- on a bounded sample: the first `rows` activation rows of the same GEMM on all host cores (about 20
+    core-seconds), and the first 64 rows on one thread."""
     from oracle import pyoracle
     cores = min(16, os.cpu_count() or 1)
-    rows = 512 if size <= 4096 else 128
-    sub = dict(case)
-    sub["a"] = case["a"][:rows].copy()
     if pyoracle.Reference.available():
         eng, kind = pyoracle.reference(), "reference"
-        eng.threads = cores
-        eng.matmul_int8(**sub)
-        secs = eng.last_seconds
     else:
         eng, kind = pyoracle.oracle(), "port"
-        eng.set_threads(cores)
-        t0 = time.perf_counter()
-        eng.matmul_int8(**sub)
-        secs = time.perf_counter() - t0
-    ops = 2.0 * rows * size * size
-    return dict(value=ops / secs / 1e12, unit="TOP/s", cores=cores, kind=kind, seconds=secs,
+
+    def run(rows, threads):
+        sub = dict(case)
+        sub["a"] = case["a"][:rows].copy()
+        if kind == "reference":
+            eng.threads = threads
+            eng.matmul_int8(**sub)
+            secs = eng.last_seconds
+        else:
+            eng.set_threads(threads)
+            t0 = time.perf_counter()
+            eng.matmul_int8(**sub)
+            secs = time.perf_counter() - t0
+        return 2.0 * rows * size * size / secs / 1e12, secs
+
+    rows = 1024 if size <= 4096 else 256
+    tops, secs = run(rows, cores)
+    tops1, secs1 = run(64 if size <= 4096 else 16, 1)
+    return dict(value=tops, unit="TOP/s", cores=cores, kind=kind, seconds=secs,
                 sample="first %d of %d activation rows of the same %d^3 GEMM (A-pack + row sums + MatmulInt8Opt "
-                       "column stripes on %d threads)" % (rows, size, size, cores))
+                       "column stripes on %d threads)" % (rows, size, size, cores),
+                single_thread=dict(value=tops1, unit="TOP/s", cores=1, seconds=secs1,
+                                   sample="first %d rows" % (64 if size <= 4096 else 16)))
 
 
 def cpu_side_by_side():
