@@ -520,6 +520,9 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // short K and more tiles than two per CU: three stages (48 KiB) let a third workgroup in, which saves a round of
   // tiles; the shallower prefetch only costs when K is long
   if (tiles_m > 512 && g.k <= 1024) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 3, 3>(g, rq, dq, stream);
+  // short K, fp32 out and fewer 128 x 128 tiles than CUs: half-width tiles, three per CU, fill the device
+  if (EPI == EPI_DEQUANT && tiles_m >= 128 && tiles_m < 256 && g.k <= 1024)
+    return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 4, 3>(g, rq, dq, stream);
   if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 4, 2>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
