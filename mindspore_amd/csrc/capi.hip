@@ -283,7 +283,14 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
                             DevBuf *c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
-  if (rows <= kGemvMaxRows && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024)) {
+  bool skinny = rows <= kGemvMaxRows && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024);
+  if (skinny && rows > kGemvDotRows && st.w_blocked.p == nullptr) {
+    // the blocked copy needs an allocation and a wait, neither of which a stream under graph capture allows: such
+    // a call takes the GEMM path (same results), and the copy is built by the first call outside a capture
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) skinny = false;
+  }
+  if (skinny) {
     if (rows > kGemvDotRows) {
       if (st.w_blocked.p == nullptr) {
         int rc = st.w_blocked.ensure((size_t)st.n_pad * st.k_pad);

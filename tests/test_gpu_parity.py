@@ -345,3 +345,32 @@ def test_error_paths():
     assert e.value.code == K._lib.MI_PARAM_INVALID
     with pytest.raises(TypeError):
         K.MatmulInt8Kernel(np.zeros((4, 8), np.int8), np.zeros(4, np.float32), QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0))
+
+
+def test_first_decode_call_inside_a_graph_capture(orc):
+    """The matrix-core decode kernel wants a blocked copy of the weights that is built on first use (an allocation and
+    a wait).  A first call under stream capture must not do either: it takes the GEMM path, the capture stays valid,
+    every replay is right, and a later eager call builds the copy."""
+    import torch
+    rng = np.random.default_rng(77)
+    case = _mm_case(rng, 8, 200, 512, True, False, True, 0)
+    kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
+                              QP(case["so"], case["zo"]), True, 0)
+    a = torch.from_numpy(case["a"]).cuda()
+    out = torch.zeros((8, 200), dtype=torch.int8, device="cuda")
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            kern.run(a, out=out)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        a.copy_(torch.from_numpy(rng.integers(-128, 128, (8, 512), dtype=np.int8)))
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        case["a"] = a.cpu().numpy()
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(out.cpu().numpy(), want), rep
+        assert np.array_equal(kern.run(a).cpu().numpy(), want)   # eager: builds and uses the blocked copy
