@@ -338,14 +338,54 @@ def test_dynamic_quant_per_row_and_matmul(orc, rows, k):
 
 
 def test_error_paths():
-    L = K._lib.init()
-    assert L.mi_matmul_run(None, None, 1, None, None) == K._lib.MI_NULL_PTR
-    with pytest.raises(K._lib.MiError) as e:
+    """Invalid descriptors and arguments come back as Lite's status codes with a message, before anything is launched."""
+    import ctypes as C
+    import torch
+    lib = K._lib
+    L = lib.init()
+    assert L.mi_matmul_run(None, None, 1, None, None) == lib.MI_NULL_PTR
+    with pytest.raises(lib.MiError) as e:
         K.MatmulInt8Kernel(np.zeros((4, 8), np.int8), None, QP(0.1, 0), [QP(0.1, 0)] * 3, QP(0.1, 0))
-    assert e.value.code == K._lib.MI_PARAM_INVALID
+    assert e.value.code == lib.MI_PARAM_INVALID
     with pytest.raises(TypeError):
         K.MatmulInt8Kernel(np.zeros((4, 8), np.int8), np.zeros(4, np.float32), QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0))
-
+    # descriptors
+    scales, zps = (C.c_double * 4)(0.1, 0.1, 0.1, 0.1), (C.c_int32 * 4)(0, 0, 0, 0)
+    w = np.zeros((4, 8), np.int8)
+    h = C.c_void_p()
+    for bad in (lib.MatmulDesc(0, 4, 1, 0, 0.1, 0, 0.1, 0, 1, scales, zps),      # deep 0
+                lib.MatmulDesc(8, -1, 1, 0, 0.1, 0, 0.1, 0, 1, scales, zps),     # negative col
+                lib.MatmulDesc(8, 4, 1, 2, 0.1, 0, 0.1, 0, 1, scales, zps),      # activation 2 (sigmoid) unsupported
+                lib.MatmulDesc(8, 4, 1, 0, 0.1, 0, 0.1, 0, 3, scales, zps)):     # 3 filter params for 4 channels
+        assert L.mi_matmul_create(C.byref(bad), w.ctypes.data, None, C.byref(h)) == lib.MI_PARAM_INVALID
+        assert h.value is None and L.mi_last_error() != b""
+    assert L.mi_matmul_create(C.byref(lib.MatmulDesc(8, 4, 1, 0, 0.1, 0, 0.1, 0, 1, None, None)), w.ctypes.data, None,
+                              C.byref(h)) == lib.MI_NULL_PTR
+    assert L.mi_dynmm_create(C.byref(lib.DynmmDesc(8, 4, 1, 7, 1, scales, zps)), w.ctypes.data, None,
+                             C.byref(h)) == lib.MI_PARAM_INVALID
+    # runs
+    kern = K.MatmulInt8Kernel(w, None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0))
+    a = torch.zeros((2, 8), dtype=torch.int8, device="cuda")
+    c = torch.zeros((2, 4), dtype=torch.int8, device="cuda")
+    assert L.mi_matmul_run(kern._h, a.data_ptr(), -1, c.data_ptr(), None) == lib.MI_PARAM_INVALID
+    assert L.mi_matmul_run(kern._h, a.data_ptr(), 0, c.data_ptr(), None) == lib.MI_OK          # empty batch: nothing to do
+    assert L.mi_matmul_run(kern._h, None, 2, c.data_ptr(), None) == lib.MI_NULL_PTR
+    dq = K.DynamicQuantKernel(False)
+    assert L.mi_dynquant_run(dq._h, None, 0, None, None) == lib.MI_OK                            # empty tensor
+    assert L.mi_dynquant_run(dq._h, None, 16, None, None) == lib.MI_NULL_PTR
+    assert L.mi_dynquant_run(dq._h, a.data_ptr(), -4, c.data_ptr(), None) == lib.MI_PARAM_INVALID
+    assert L.mi_dynquant_run_segments(dq._h, a.data_ptr(), 0, 8, c.data_ptr(), c.data_ptr(), None) == lib.MI_PARAM_INVALID
+    # convolution: declined shapes are MI_NOT_SUPPORT (the provider falls back), broken ones MI_PARAM_INVALID
+    with pytest.raises(lib.MiError) as e:
+        K.ConvolutionInt8Kernel(np.zeros((8, 3, 3, 4), np.int8), None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0),
+                                (0, 1), (1, 1), (0, 0, 0, 0), 1, 0)
+    assert e.value.code == lib.MI_PARAM_INVALID
+    conv = K.ConvolutionInt8Kernel(np.zeros((8, 1, 1, 4), np.int8), None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0),
+                                   (1, 1), (1, 1), (0, 0, 0, 0), 1, 0)
+    x = torch.zeros((1, 5, 5, 4), dtype=torch.int8, device="cuda")
+    y = torch.zeros((1, 5, 5, 8), dtype=torch.int8, device="cuda")
+    assert L.mi_conv_run(conv._h, x.data_ptr(), 1, 0, 5, y.data_ptr(), None) == lib.MI_PARAM_INVALID
+    assert L.mi_conv_run(conv._h, x.data_ptr(), 1, 5, 5, None, None) == lib.MI_NULL_PTR
 
 def test_first_decode_call_inside_a_graph_capture(orc):
     """The matrix-core decode kernel wants a blocked copy of the weights that is built on first use (an allocation and
