@@ -293,3 +293,39 @@ def test_dynamic_quant_and_dynamic_matmul_through_the_provider(H, orc):
     assert np.array_equal(yr.view(np.uint32), wantr.view(np.uint32))
     for n in (dq, mm, dqr):
         n.close()
+
+
+@pytest.mark.gpu
+def test_configuration_2_block_through_the_provider(H, orc):
+    """The MobileNetV2-style block of benchmark configuration 2 (3x3 s2 stem, 1x1 expand, 3x3 depthwise, 1x1 project,
+    ReLU6 fused) as four provider kernels in a row, tensors handed over on the host as a "CPU"-arch provider gets
+    them: every layer's output equals the oracle's, and the last one the committed golden hash."""
+    import hashlib
+    import json
+    from mindspore_amd import workloads as wl
+    from oracle.pyoracle import conv_shape
+    hashes = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "config_hashes.json")))["c2"]
+    orc.set_threads(16)
+    x, layers = wl.mobilenet_c2()
+    cur = x
+    for L in layers:
+        dw = L["kind"] == "dw"
+        w = L["w"].reshape(L["oc"], L["kernel"], L["kernel"], 1) if dw else L["w"]
+        node_op = op(CONV, kernel=(L["kernel"],) * 2, stride=(L["stride"],) * 2, dilation=(1, 1), pad_mode=0,
+                     pad_list=L["pad"], has_pad_list=1, group=L["oc"] if dw else 1, in_channel=L["ic"],
+                     out_channel=L["oc"], act=L["act"])
+        ins = [tensor(I8, cur.shape, None, False, [(L["sx"], L["zx"])]),
+               tensor(I8, w.shape, w, True, [(s, z) for s, z in zip(L["sw"], L["zw"])])]
+        if L["bias"] is not None:
+            ins.append(tensor(I32, (L["oc"],), L["bias"], True))
+        node = Node(H, node_op, ins, I8, [(L["so"], L["zo"])])
+        assert node.stage == OK, (L["name"], node.stage, node.code)
+        got, _ = node.run(cur)
+        shape = conv_shape(cur.shape[0], cur.shape[1], cur.shape[2], L["ic"], L["oc"], (L["kernel"],) * 2,
+                           (L["stride"],) * 2, (1, 1), L["pad"])
+        fn = orc.conv_dw_int8 if dw else orc.conv_int8
+        want = fn(cur, L["w"], L["bias"], shape, L["sx"], L["zx"], L["sw"], L["zw"], L["so"], L["zo"], L["act"])
+        assert got.shape == want.shape and np.array_equal(got, want), L["name"]
+        assert hashlib.sha256(np.ascontiguousarray(got).tobytes()).hexdigest() == hashes[L["name"]], L["name"]
+        node.close()
+        cur = got
