@@ -24,6 +24,7 @@
 #ifndef MI355X_INT8_H_
 #define MI355X_INT8_H_
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -259,6 +260,18 @@ typedef struct mi_conv_infer {
  * output extent to 1.  Updates p (kernel size, group, SAME-mode pads) as the reference updates its ConvParameter. */
 int mi_infer_conv2d(const int32_t *in_shape, int32_t in_dims, const int32_t *w_shape, int32_t w_dims,
                     mi_conv_infer *p, int32_t *out_shape, int32_t *out_dims);
+
+/* ---- device memory for tensors that stay on the GPU between provider kernels ------------------------------------------
+ * What a provider needs to keep an activation in HBM from one of its kernels to the next and publish the address on
+ * the tensor with MSTensor::SetDeviceData (include/api/types.h:295-305; the consumer reads it with GetDeviceData):
+ * the role a device Allocator's Malloc / Free (include/api/allocator.h:33,48) and the OpenCL kernels' host<->device
+ * copies play in the reference.  Copies are ordered on `stream` like the *_run entry points and return when they
+ * are complete (the host buffer may be reused at once).  All of them act on the device given to mi_init. */
+int mi_device_malloc(size_t bytes, void **out_dev);
+int mi_device_free(void *dev); /* NULL is allowed */
+int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream);
+int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream);
+int mi_stream_synchronize(void *stream);
 
 /* ---- measurement aids (no counterpart in the reference) ---------------------------------------------------------
  * Two plain HBM movers with a known byte count and a matrix-pipe exerciser, used by the benchmark: the read stream gives the bandwidth a

@@ -385,6 +385,56 @@ int mi_init(int device) {
   return MI_OK;
 }
 
+int mi_device_malloc(size_t bytes, void **out_dev) {
+  if (out_dev == nullptr) return MI_NULL_PTR;
+  *out_dev = nullptr;
+  if (bytes == 0) {
+    set_error("mi_device_malloc: zero bytes");
+    return MI_PARAM_INVALID;
+  }
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  const size_t sz = (bytes + 255) & ~(size_t)255;
+  if (hipMalloc(out_dev, sz) != hipSuccess) {
+    *out_dev = nullptr;
+    set_error("hipMalloc(%zu) failed", sz);
+    return MI_MEMORY_FAILED;
+  }
+  return MI_OK;
+}
+
+int mi_device_free(void *dev) {
+  if (dev == nullptr) return MI_OK;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  MI_HIP_CHECK(hipFree(dev));
+  return MI_OK;
+}
+
+int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream) {
+  if (bytes == 0) return MI_OK;
+  if (dst_dev == nullptr || src_host == nullptr) return MI_NULL_PTR;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI_HIP_CHECK(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, s));
+  MI_HIP_CHECK(hipStreamSynchronize(s));  // the caller may reuse src_host at once (the runtime recycles tensor memory)
+  return MI_OK;
+}
+
+int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream) {
+  if (bytes == 0) return MI_OK;
+  if (dst_host == nullptr || src_dev == nullptr) return MI_NULL_PTR;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI_HIP_CHECK(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, s));
+  MI_HIP_CHECK(hipStreamSynchronize(s));
+  return MI_OK;
+}
+
+int mi_stream_synchronize(void *stream) {
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  MI_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return MI_OK;
+}
+
 int mi_diag_stream_read(const void *src_dev, int64_t bytes, void *stream) {
   if (src_dev == nullptr) return MI_NULL_PTR;
   if (bytes <= 0 || (bytes & 15) != 0 || (reinterpret_cast<uintptr_t>(src_dev) & 15) != 0) {

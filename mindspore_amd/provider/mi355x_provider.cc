@@ -16,12 +16,21 @@
 // An application selects it with CPUDeviceInfo::SetProvider("mi355x") (+ SetProviderDevice("CPU")); the stock
 // benchmark tool with --provider=mi355x (it leaves the provider device empty, hence the second registration under "").
 //
-// Tensors are host-resident (arch "CPU": the kernels live in the ordinary CPU subgraph), so Execute() uses the
-// *_run_host entry points, which copy into and out of device buffers the handle owns.  A creator returns nullptr for everything the library
-// does not reproduce bit-exactly; the scheduler then falls back to the builtin CPU kernel
-// (mindspore/lite/src/litert/scheduler.cc:1173-1177).
+// Tensors are host-resident (arch "CPU": the kernels live in the ordinary CPU subgraph).  Every kernel computes into
+// a device buffer of its own, publishes that address on its output tensor (MSTensor::SetDeviceData,
+// include/api/types.h:295-305) and copies the result to the tensor's host memory; a kernel whose input carries an
+// address published by another kernel of this provider reads it in place and skips the upload.  The session config
+//   [mi355x]
+//   device_only_outputs=<tensor name>,<tensor name>,...      (or * for every output)
+// (Model::LoadConfig / UpdateConfig, delivered through Kernel::GetConfig, include/api/kernel_api.h:112-126) names
+// outputs that only kernels of this provider consume: their host copy is skipped as well.
+// A creator returns nullptr for everything the library does not reproduce bit-exactly; the scheduler then falls back
+// to the builtin CPU kernel (mindspore/lite/src/litert/scheduler.cc:1173-1177).
+#include <map>
 #include <memory>
+#include <mutex>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 #include "include/api/kernel.h"
@@ -64,6 +73,122 @@ int64_t RowsOf(const MSTensor &t) {
 }
 }  // namespace
 
+// Device addresses this provider has published on tensors.  GetDeviceData() of an input is trusted only when it is
+// one of them: an application may have attached memory of some other device to a graph input.
+class Published {
+ public:
+  static void Add(void *p) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    Set().insert(p);
+  }
+  static void Remove(void *p) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    Set().erase(p);
+  }
+  static bool Has(void *p) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    return Set().count(p) != 0;
+  }
+
+ private:
+  static std::mutex &Mutex() {
+    static std::mutex m;
+    return m;
+  }
+  static std::unordered_set<void *> &Set() {
+    static std::unordered_set<void *> s;
+    return s;
+  }
+};
+
+// Device memory a kernel owns; grows, never shrinks.
+class DeviceBuffer {
+ public:
+  DeviceBuffer() = default;
+  DeviceBuffer(const DeviceBuffer &) = delete;
+  DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+  ~DeviceBuffer() { Release(); }
+  void *Reserve(size_t bytes) {
+    if (bytes > cap_) {
+      Release();
+      if (mi_device_malloc(bytes, &p_) != MI_OK) return nullptr;
+      cap_ = bytes;
+    }
+    return p_;
+  }
+  void *get() const { return p_; }
+
+ private:
+  void Release() {
+    if (p_ != nullptr) {
+      Published::Remove(p_);
+      mi_device_free(p_);
+    }
+    p_ = nullptr;
+    cap_ = 0;
+  }
+  void *p_ = nullptr;
+  size_t cap_ = 0;
+};
+
+// What every kernel of this provider does around its launch: find input 0 on the device (in place when a kernel of
+// this provider left it there, uploaded otherwise) and hand the output on.
+class DeviceIo {
+ public:
+  // reads [mi355x] device_only_outputs for the given output tensor
+  void Configure(const std::map<std::string, std::string> &section, const std::string &output_name) {
+    const auto it = section.find("device_only_outputs");
+    if (it == section.end()) return;
+    const std::string &list = it->second;
+    size_t pos = 0;
+    while (pos <= list.size()) {
+      size_t end = list.find(',', pos);
+      if (end == std::string::npos) end = list.size();
+      size_t b = pos, e = end;
+      while (b < e && list[b] == ' ') ++b;
+      while (e > b && list[e - 1] == ' ') --e;
+      const std::string name = list.substr(b, e - b);
+      if (name == "*" || (!name.empty() && name == output_name)) host_copy_ = false;
+      pos = end + 1;
+    }
+  }
+
+  const void *Input(MSTensor *t) {
+    void *dev = t->GetDeviceData();
+    if (dev != nullptr && Published::Has(dev)) return dev;
+    const auto host = t->Data();
+    const size_t bytes = t->DataSize();
+    if (host == nullptr || bytes == 0) return nullptr;
+    void *staged = in_.Reserve(bytes);
+    if (staged == nullptr || mi_copy_to_device(staged, host.get(), bytes, nullptr) != MI_OK) return nullptr;
+    return staged;
+  }
+
+  void *Output(size_t bytes) {
+    void *p = out_.Reserve(bytes);
+    if (p != nullptr) Published::Add(p);
+    return p;
+  }
+
+  // after the launch: publish the device address; copy to the host unless the output was declared device-only
+  int Deliver(MSTensor *t) {
+    t->SetDeviceData(out_.get());
+    if (!host_copy_) return kSuccess;
+    void *host = t->MutableData();
+    if (host == nullptr) return kLiteNullptr;
+    return mi_copy_to_host(host, out_.get(), t->DataSize(), nullptr) == MI_OK ? static_cast<int>(kSuccess)
+                                                                              : static_cast<int>(kLiteError);
+  }
+
+  void Withdraw(MSTensor *t) {
+    if (t->GetDeviceData() == out_.get()) t->SetDeviceData(nullptr);
+  }
+
+ private:
+  DeviceBuffer in_, out_;
+  bool host_copy_ = true;
+};
+
 // ---- MatMulFusion / FullConnection, int8 in -> int8 out (full quant) or fp32 out (dynamic quant) ----------------
 class MatmulKernel : public kernel::Kernel {
  public:
@@ -71,11 +196,13 @@ class MatmulKernel : public kernel::Kernel {
                const Context *ctx, bool b_transpose, int act)
       : Kernel(in, out, prim, ctx), b_transpose_(b_transpose), act_(act) {}
   ~MatmulKernel() override {
+    io_.Withdraw(&outputs_[0]);
     mi_matmul_destroy(full_);
     mi_dynmm_destroy(dyn_);
   }
 
   int Prepare() override {
+    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
     const MSTensor &w = inputs_[kWeightIndex];
     const auto wshape = w.Shape();
     if (wshape.size() != 2 || w.Data() == nullptr) return kLiteError;
@@ -101,23 +228,35 @@ class MatmulKernel : public kernel::Kernel {
   int ReSize() override { return kSuccess; }  // the row count is read from the input tensor at every Execute
 
   int Execute() override {
-    const auto *a = static_cast<const int8_t *>(inputs_[0].Data().get());
-    void *c = outputs_[0].MutableData();
-    if (a == nullptr || c == nullptr) return kLiteNullptr;
     const int32_t rows = static_cast<int32_t>(RowsOf(inputs_[0]));
-    if (full_ != nullptr) return ToStatus(mi_matmul_run_host(full_, a, rows, static_cast<int8_t *>(c)));
-    // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
-    // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
-    const auto iqs = inputs_[0].QuantParams();
-    if (iqs.size() == 1) {
-      return ToStatus(mi_dynmm_run_host(dyn_, a, rows, iqs[0].scale, iqs[0].zero_point, static_cast<float *>(c)));
+    if (rows == 0) return kSuccess;
+    const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
+    void *c = io_.Output(outputs_[0].DataSize());
+    if (a == nullptr || c == nullptr) return kLiteNullptr;
+    int rc = MI_ERROR;
+    if (full_ != nullptr) {
+      rc = mi_matmul_run(full_, a, rows, static_cast<int8_t *>(c), nullptr);
+    } else {
+      // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
+      // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
+      const auto iqs = inputs_[0].QuantParams();
+      if (iqs.size() == 1) {
+        rc = mi_dynmm_run(dyn_, a, rows, iqs[0].scale, iqs[0].zero_point, static_cast<float *>(c), nullptr);
+      } else {
+        // one scale per row (input_per_channel_, :152-171), narrowed to float (:168-171); the zero point used is
+        // the first one (matmul_dynamic_int8.cc:61)
+        if (iqs.size() != static_cast<size_t>(rows)) return kLiteError;
+        std::vector<mi_dq_params> ps(iqs.size());
+        for (size_t i = 0; i < iqs.size(); ++i) {
+          ps[i] = mi_dq_params{iqs[i].scale, static_cast<float>(iqs[i].scale), iqs[0].zero_point, 0.0f, 0.0f};
+        }
+        const size_t bytes = ps.size() * sizeof(mi_dq_params);
+        void *dev = row_params_.Reserve(bytes);
+        if (dev == nullptr || mi_copy_to_device(dev, ps.data(), bytes, nullptr) != MI_OK) return kLiteError;
+        rc = mi_dynmm_run_rows(dyn_, a, rows, static_cast<const mi_dq_params *>(dev), static_cast<float *>(c), nullptr);
+      }
     }
-    // one scale per row (input_per_channel_, :152-171); the zero point used is the first one (matmul_dynamic_int8.cc:61)
-    if (iqs.size() != static_cast<size_t>(rows)) return kLiteError;
-    std::vector<double> scales(iqs.size());
-    for (size_t i = 0; i < iqs.size(); ++i) scales[i] = iqs[i].scale;
-    return ToStatus(
-      mi_dynmm_run_rows_host(dyn_, a, rows, scales.data(), iqs[0].zero_point, static_cast<float *>(c)));
+    return rc == MI_OK ? io_.Deliver(&outputs_[0]) : static_cast<int>(kLiteError);
   }
 
  private:
@@ -125,6 +264,8 @@ class MatmulKernel : public kernel::Kernel {
   int act_;
   mi_matmul *full_ = nullptr;
   mi_dynmm *dyn_ = nullptr;
+  DeviceIo io_;
+  DeviceBuffer row_params_;
 };
 
 std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
@@ -160,9 +301,15 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
 class ConvKernel : public kernel::Kernel {
  public:
   using Kernel::Kernel;
-  ~ConvKernel() override { mi_conv_destroy(conv_); }
+  ~ConvKernel() override {
+    io_.Withdraw(&outputs_[0]);
+    mi_conv_destroy(conv_);
+  }
 
-  int Prepare() override { return Build(); }
+  int Prepare() override {
+    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
+    return Build();
+  }
 
   // Weights and quant parameters do not depend on the image size; SAME-mode padding does (the builtin kernel gets
   // it from shape inference at every resize, conv2d_infer.c:34-50), so the handle is rebuilt only when it moved.
@@ -178,11 +325,16 @@ class ConvKernel : public kernel::Kernel {
 
   int Execute() override {
     const auto s = inputs_[0].Shape();
-    const auto *x = static_cast<const int8_t *>(inputs_[0].Data().get());
-    auto *y = static_cast<int8_t *>(outputs_[0].MutableData());
-    if (x == nullptr || y == nullptr || s.size() != 4) return kLiteNullptr;
-    return ToStatus(mi_conv_run_host(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]),
-                                     static_cast<int32_t>(s[2]), y));
+    if (s.size() != 4) return kLiteError;
+    if (inputs_[0].ElementNum() == 0 || outputs_[0].ElementNum() == 0) return kSuccess;
+    const auto *x = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
+    auto *y = static_cast<int8_t *>(io_.Output(outputs_[0].DataSize()));
+    if (x == nullptr || y == nullptr) return kLiteNullptr;
+    if (mi_conv_run(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]), static_cast<int32_t>(s[2]), y,
+                    nullptr) != MI_OK) {
+      return kLiteError;
+    }
+    return io_.Deliver(&outputs_[0]);
   }
 
  private:
@@ -239,6 +391,7 @@ class ConvKernel : public kernel::Kernel {
 
   int32_t pads_[4] = {0, 0, 0, 0};
   mi_conv *conv_ = nullptr;
+  DeviceIo io_;
 };
 
 std::shared_ptr<kernel::Kernel> ConvCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
@@ -273,23 +426,35 @@ std::shared_ptr<kernel::Kernel> ConvCreator(const std::vector<MSTensor> &in, con
 class DynamicQuantKernel : public kernel::Kernel {
  public:
   using Kernel::Kernel;
-  ~DynamicQuantKernel() override { mi_dynquant_destroy(dq_); }
+  ~DynamicQuantKernel() override {
+    io_.Withdraw(&outputs_[0]);
+    mi_dynquant_destroy(dq_);
+  }
 
   int Prepare() override {
+    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
     const auto *p = primitive_->value_as_DynamicQuant();
     per_row_ = p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0;
     return ToStatus(mi_dynquant_create(p->symmetric() ? 1 : 0, &dq_));
   }
   int ReSize() override { return kSuccess; }
   int Execute() override {
-    const auto *x = static_cast<const float *>(inputs_[0].Data().get());
-    auto *q = static_cast<int8_t *>(outputs_[0].MutableData());
+    const int64_t n = inputs_[0].ElementNum();
+    if (n == 0) return kSuccess;
+    const auto *x = static_cast<const float *>(io_.Input(&inputs_[0]));
+    auto *q = static_cast<int8_t *>(io_.Output(outputs_[0].DataSize()));
     if (x == nullptr || q == nullptr) return kLiteNullptr;
+    // the scales and zero points always travel to the host: the consumer, builtin or not, reads them from the tensor
     if (per_row_) {  // the creator admitted only "every axis but the last": one run per row of the last axis
       const int64_t unit = inputs_[0].Shape().back();
-      const int64_t segments = inputs_[0].ElementNum() / unit;
+      const int64_t segments = n / unit;
       std::vector<mi_dq_params> ps(static_cast<size_t>(segments));
-      if (mi_dynquant_run_segments_host(dq_, x, segments, unit, q, ps.data()) != MI_OK) return kLiteError;
+      const size_t bytes = ps.size() * sizeof(mi_dq_params);
+      auto *dev = static_cast<mi_dq_params *>(row_params_.Reserve(bytes));
+      if (dev == nullptr || mi_dynquant_run_segments(dq_, x, segments, unit, q, dev, nullptr) != MI_OK ||
+          mi_copy_to_host(ps.data(), dev, bytes, nullptr) != MI_OK) {
+        return kLiteError;
+      }
       std::vector<QuantParam> qps(ps.size());
       for (size_t i = 0; i < ps.size(); ++i) {
         qps[i].bit_num = 8;
@@ -299,11 +464,12 @@ class DynamicQuantKernel : public kernel::Kernel {
         qps[i].max = ps[i].real_max;
       }
       outputs_[0].SetQuantParams(qps);
-      return kSuccess;
+      return io_.Deliver(&outputs_[0]);
     }
     mi_dq_params p{};
-    const int rc = mi_dynquant_run_host(dq_, x, inputs_[0].ElementNum(), q, &p);
-    if (rc != MI_OK) return kLiteError;
+    if (mi_dynquant_run(dq_, x, n, q, nullptr) != MI_OK || mi_dynquant_get_params(dq_, nullptr, &p) != MI_OK) {
+      return kLiteError;
+    }
     // what DynamicQuantCPUKernel::CalculatePerlayerScaleZp publishes on the output tensor (dynamic_quant.cc:156-186)
     QuantParam qp{};
     qp.bit_num = 8;
@@ -312,12 +478,14 @@ class DynamicQuantKernel : public kernel::Kernel {
     qp.min = p.real_min;
     qp.max = p.real_max;
     outputs_[0].SetQuantParams({qp});
-    return kSuccess;
+    return io_.Deliver(&outputs_[0]);
   }
 
  private:
   mi_dynquant *dq_ = nullptr;
   bool per_row_ = false;
+  DeviceIo io_;
+  DeviceBuffer row_params_;
 };
 
 std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,

@@ -5,6 +5,7 @@
 // runs when this library is loaded.
 #include <string.h>
 
+#include <map>
 #include <memory>
 #include <string>
 #include <vector>
@@ -50,6 +51,7 @@ struct Session {
   std::shared_ptr<mindspore::kernel::Kernel> kernel;
   std::shared_ptr<mindspore::kernel::KernelInterface> infer;
   mindspore::Context ctx;
+  std::map<std::string, std::map<std::string, std::string>> config;  // the session's config file sections
 };
 
 std::vector<mindspore::QuantParam> Quant(int n, const double *scales, const int32_t *zps) {
@@ -101,15 +103,28 @@ int Infer(Session *s) {
 extern "C" {
 // Builds the node: tensors, shape inference, creator lookup and call, Prepare().  *stage tells how far it got;
 // *code is the status of the failing call (0 otherwise).  Returns NULL unless the kernel is ready to execute.
-void *ph_create(const ph_op *op, const char *arch, const char *provider, const ph_tensor *inputs, int32_t n_in,
-                int32_t out_dtype, int32_t out_nquant, const double *out_scales, const int32_t *out_zps,
-                int32_t *stage, int32_t *code) {
+// `producer` (optional): a node made earlier whose output tensor becomes this node's input 0 -- the same tensor
+// object, as in a graph, so that what the producer leaves on it (data, quant params, device address) is what this
+// node finds.  `out_name` names the output tensor; `device_only_outputs` (optional) is the value of that key in the
+// [mi355x] section of the session config.
+void *ph_create_node(const ph_op *op, const char *arch, const char *provider, const ph_tensor *inputs, int32_t n_in,
+                     int32_t out_dtype, int32_t out_nquant, const double *out_scales, const int32_t *out_zps,
+                     void *producer, const char *out_name, const char *device_only_outputs, int32_t *stage,
+                     int32_t *code) {
   auto s = std::make_unique<Session>();
   *stage = kOk;
   *code = 0;
   Fill(*op, &s->prim);
-  for (int i = 0; i < n_in; ++i) s->inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
-  MSTensor out("out", static_cast<mindspore::DataType>(out_dtype), {}, nullptr, 0, false);
+  if (device_only_outputs != nullptr) s->config["mi355x"]["device_only_outputs"] = device_only_outputs;
+  for (int i = 0; i < n_in; ++i) {
+    if (i == 0 && producer != nullptr) {
+      s->inputs.push_back(static_cast<Session *>(producer)->outputs[0]);
+    } else {
+      s->inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
+    }
+  }
+  MSTensor out(out_name != nullptr ? out_name : "out", static_cast<mindspore::DataType>(out_dtype), {}, nullptr, 0,
+               false);
   out.SetQuantParams(Quant(out_nquant, out_scales, out_zps));
   s->outputs.push_back(out);
   s->infer = mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &s->prim);
@@ -125,11 +140,40 @@ void *ph_create(const ph_op *op, const char *arch, const char *provider, const p
     *stage = kDeclined;  // the scheduler would now take the builtin CPU kernel
     return nullptr;
   }
+  s->kernel->SetConfig(&s->config);  // scheduler.cc:1455-1457
   if ((*code = s->kernel->Prepare()) != 0) {
     *stage = kPrepareFailed;
     return nullptr;
   }
   return s.release();
+}
+
+void *ph_create(const ph_op *op, const char *arch, const char *provider, const ph_tensor *inputs, int32_t n_in,
+                int32_t out_dtype, int32_t out_nquant, const double *out_scales, const int32_t *out_zps,
+                int32_t *stage, int32_t *code) {
+  return ph_create_node(op, arch, provider, inputs, n_in, out_dtype, out_nquant, out_scales, out_zps, nullptr, nullptr,
+                        nullptr, stage, code);
+}
+
+// Executes a node whose input 0 is its producer's output tensor, as that producer left it.  The shape is taken from
+// that tensor; when it differs from the last run the output shape is inferred again and ReSize() is called.
+int32_t ph_execute_linked(void *h, int32_t *code) {
+  auto *s = static_cast<Session *>(h);
+  *code = 0;
+  const std::vector<int64_t> before = s->outputs[0].Shape();
+  if (Infer(s) != kOk) return kInferFailed;
+  if (before != s->outputs[0].Shape() && (*code = s->kernel->ReSize()) != 0) return kResizeFailed;
+  if ((*code = s->kernel->Execute()) != 0) return kExecuteFailed;
+  return kOk;
+}
+
+// Attaches an address to input 0 as an application could with MSTensor::SetDeviceData.
+void ph_set_input_device_data(void *h, void *address) { static_cast<Session *>(h)->inputs[0].SetDeviceData(address); }
+
+// bit 0: the output tensor has host memory; bit 1: it carries a device address.
+int32_t ph_output_state(void *h) {
+  auto *s = static_cast<Session *>(h);
+  return (s->outputs[0].HasHostData() ? 1 : 0) | (s->outputs[0].GetDeviceData() != nullptr ? 2 : 0);
 }
 
 // Sets input 0 (new shape allowed: the output shape is inferred again and ReSize() is called, as the runtime does on

@@ -2,6 +2,8 @@
 // life-cycle calls the runtime makes and the protected tensor lists (reference: MSKernel :29-140, IKernel :143-166).
 #ifndef TESTS_LITE_STUB_INCLUDE_API_KERNEL_API_H_
 #define TESTS_LITE_STUB_INCLUDE_API_KERNEL_API_H_
+#include <map>
+#include <string>
 #include <vector>
 
 #include "include/api/status.h"
@@ -16,6 +18,14 @@ class MSKernel {
   virtual int Prepare() = 0;
   virtual int ReSize() = 0;
   virtual int Execute() = 0;
+  // the session's config file sections (Model::LoadConfig / UpdateConfig), handed over by the scheduler after the
+  // creator has run (scheduler.cc:1455-1457)
+  void SetConfig(const std::map<std::string, std::map<std::string, std::string>> *config) { config_ = config; }
+  std::map<std::string, std::string> GetConfig(const std::string &section) const {
+    if (config_ == nullptr) return {};
+    const auto it = config_->find(section);
+    return it == config_->end() ? std::map<std::string, std::string>() : it->second;
+  }
 
  protected:
   MSKernel() = default;
@@ -23,6 +33,7 @@ class MSKernel {
       : context_(ctx), inputs_(in), outputs_(out) {}
   const Context *context_ = nullptr;
   std::vector<MSTensor> inputs_, outputs_;
+  const std::map<std::string, std::map<std::string, std::string>> *config_ = nullptr;
 };
 
 template <typename Primitive>

@@ -32,6 +32,7 @@ class MSTensor {
     std::shared_ptr<std::vector<char>> data;  // null until allocated
     std::vector<QuantParam> quant;
     bool is_const = false;
+    void *device_data = nullptr;  // an address only: the tensor never frees it (lite::Tensor::device_data_)
   };
   MSTensor() : impl_(std::make_shared<Impl>()) {}
   // harness-side constructor (the real class is created by the runtime)
@@ -73,6 +74,9 @@ class MSTensor {
   std::vector<QuantParam> QuantParams() const { return impl_->quant; }
   void SetQuantParams(std::vector<QuantParam> quant_params) { impl_->quant = std::move(quant_params); }
   std::string Name() const { return impl_->name; }
+  void SetDeviceData(void *data) { impl_->device_data = data; }
+  void *GetDeviceData() { return impl_->device_data; }
+  bool HasHostData() const { return impl_->data != nullptr; }  // harness-side
 
  private:
   size_t ElementSize() const {

@@ -414,3 +414,38 @@ def test_first_decode_call_inside_a_graph_capture(orc):
         want = orc.matmul_int8(**case)
         assert np.array_equal(out.cpu().numpy(), want), rep
         assert np.array_equal(kern.run(a).cpu().numpy(), want)   # eager: builds and uses the blocked copy
+
+
+def test_device_memory_entry_points(orc):
+    """mi_device_malloc / mi_copy_to_device / mi_copy_to_host / mi_device_free: what a provider keeps a tensor in HBM
+    with.  A buffer from them feeds a kernel launch like any device pointer."""
+    import ctypes as C
+    lib = K._lib
+    L = lib.init()
+    p = C.c_void_p()
+    assert L.mi_device_malloc(0, C.byref(p)) == lib.MI_PARAM_INVALID and p.value is None
+    assert L.mi_device_malloc(64, None) == lib.MI_NULL_PTR
+    assert L.mi_device_free(None) == lib.MI_OK
+    assert L.mi_copy_to_device(None, None, 0, None) == lib.MI_OK
+    assert L.mi_copy_to_device(None, None, 8, None) == lib.MI_NULL_PTR
+    assert L.mi_copy_to_host(None, None, 8, None) == lib.MI_NULL_PTR
+    rng = np.random.default_rng(21)
+    m, k, n = 7, 200, 52
+    a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    bias = rng.integers(-3000, 3000, n).astype(np.int32)
+    sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
+    kern = K.MatmulInt8Kernel(w, bias, QP(0.03, 4), [QP(s, 0) for s in sw], QP(0.07, -2))
+    a_dev, c_dev = C.c_void_p(), C.c_void_p()
+    assert L.mi_device_malloc(a.nbytes, C.byref(a_dev)) == lib.MI_OK and a_dev.value
+    assert L.mi_device_malloc(m * n, C.byref(c_dev)) == lib.MI_OK and c_dev.value
+    assert L.mi_copy_to_device(a_dev, a.ctypes.data, a.nbytes, None) == lib.MI_OK
+    back = np.empty_like(a)
+    assert L.mi_copy_to_host(back.ctypes.data, a_dev, a.nbytes, None) == lib.MI_OK and np.array_equal(back, a)
+    assert L.mi_matmul_run(kern._h, a_dev, m, c_dev, None) == lib.MI_OK
+    assert L.mi_stream_synchronize(None) == lib.MI_OK
+    got = np.empty((m, n), np.int8)
+    assert L.mi_copy_to_host(got.ctypes.data, c_dev, got.nbytes, None) == lib.MI_OK
+    want = orc.matmul_int8(a, w, bias, 0.03, 4, sw, np.zeros(n, np.int32), 0.07, -2, 0, True)
+    assert np.array_equal(got, want)
+    assert L.mi_device_free(a_dev) == lib.MI_OK and L.mi_device_free(c_dev) == lib.MI_OK

@@ -53,6 +53,12 @@ def H():
     h.ph_infer.argtypes = [C.POINTER(PhOp), C.c_char_p, C.POINTER(PhTensor), C.c_int32, C.POINTER(C.c_int64)]
     h.ph_destroy.argtypes = [C.c_void_p]
     h.ph_destroy.restype = None
+    h.ph_create_node.restype = C.c_void_p
+    h.ph_create_node.argtypes = h.ph_create.argtypes[:9] + [C.c_void_p, C.c_char_p, C.c_char_p] + h.ph_create.argtypes[9:]
+    h.ph_execute_linked.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    h.ph_set_input_device_data.argtypes = [C.c_void_p, C.c_void_p]
+    h.ph_set_input_device_data.restype = None
+    h.ph_output_state.argtypes = [C.c_void_p]
     return h
 
 
@@ -91,14 +97,18 @@ def op(type_, **kw):
 
 
 class Node:
-    def __init__(self, H, o, inputs, out_dtype, out_quant=(), arch=b"CPU", provider=b"mi355x"):
+    def __init__(self, H, o, inputs, out_dtype, out_quant=(), arch=b"CPU", provider=b"mi355x", producer=None,
+                 out_name=None, device_only=None):
+        """producer: the node whose output tensor is this node's input 0 (inputs[0] then only fills the slot);
+        device_only: value of device_only_outputs in the [mi355x] section of the session config."""
         self.H = H
         arr = (PhTensor * len(inputs))(*inputs)
         scales = (C.c_double * max(len(out_quant), 1))(*[float(q[0]) for q in out_quant])
         zps = (C.c_int32 * max(len(out_quant), 1))(*[int(q[1]) for q in out_quant])
         stage, code = C.c_int32(-1), C.c_int32(0)
-        self.h = H.ph_create(C.byref(o), arch, provider, arr, len(inputs), out_dtype, len(out_quant), scales, zps,
-                             C.byref(stage), C.byref(code))
+        self.h = H.ph_create_node(C.byref(o), arch, provider, arr, len(inputs), out_dtype, len(out_quant), scales, zps,
+                                  producer.h if producer is not None else None, out_name, device_only,
+                                  C.byref(stage), C.byref(code))
         self.stage, self.code, self.out_dtype = stage.value, code.value, out_dtype
 
     def run(self, x, quant=()):
@@ -109,6 +119,20 @@ class Node:
         code = C.c_int32(0)
         st = self.H.ph_execute(self.h, x.ctypes.data, shape, x.ndim, len(quant), scales, zps, C.byref(code))
         assert st == OK, (st, code.value)
+        return self.output()
+
+    def run_linked(self):
+        """Executes on the producer's output tensor as the producer left it."""
+        code = C.c_int32(0)
+        st = self.H.ph_execute_linked(self.h, C.byref(code))
+        assert st == OK, (st, code.value)
+
+    def state(self):
+        """(output has host memory, output carries a device address)"""
+        st = self.H.ph_output_state(self.h)
+        return bool(st & 1), bool(st & 2)
+
+    def output(self):
         oshape, dims, nq = (C.c_int64 * 8)(), C.c_int32(0), C.c_int32(0)
         qs, qz = (C.c_double * 65536)(), (C.c_int32 * 65536)()
         nbytes = self.H.ph_output(self.h, oshape, C.byref(dims), None, 0, qs, qz, 65536, C.byref(nq))
@@ -329,3 +353,129 @@ def test_configuration_2_block_through_the_provider(H, orc):
         assert hashlib.sha256(np.ascontiguousarray(got).tobytes()).hexdigest() == hashes[L["name"]], L["name"]
         node.close()
         cur = got
+
+
+def _c2_nodes(H, x_shape, layers, device_only):
+    """The four convolutions as a graph: each node's input 0 is the tensor the node before wrote."""
+    from oracle.pyoracle import conv_shape
+    nodes, shape = [], x_shape
+    for i, L in enumerate(layers):
+        dw = L["kind"] == "dw"
+        w = L["w"].reshape(L["oc"], L["kernel"], L["kernel"], 1) if dw else L["w"]
+        node_op = op(CONV, kernel=(L["kernel"],) * 2, stride=(L["stride"],) * 2, dilation=(1, 1), pad_mode=0,
+                     pad_list=L["pad"], has_pad_list=1, group=L["oc"] if dw else 1, in_channel=L["ic"],
+                     out_channel=L["oc"], act=L["act"])
+        ins = [tensor(I8, shape, None, False, [(L["sx"], L["zx"])]),
+               tensor(I8, w.shape, w, True, [(s, z) for s, z in zip(L["sw"], L["zw"])]),
+               tensor(I32, (L["oc"],), L["bias"], True)]
+        node = Node(H, node_op, ins, I8, [(L["so"], L["zo"])], producer=nodes[-1] if nodes else None,
+                    out_name=L["name"].encode(), device_only=device_only)
+        assert node.stage == OK, (L["name"], node.stage, node.code)
+        nodes.append(node)
+        g = conv_shape(shape[0], shape[1], shape[2], L["ic"], L["oc"], (L["kernel"],) * 2, (L["stride"],) * 2, (1, 1),
+                       L["pad"])
+        shape = (g.batch, g.out_h, g.out_w, L["oc"])
+    return nodes
+
+
+def _c2_oracle(orc, x, layers):
+    from oracle.pyoracle import conv_shape
+    outs, cur = [], x
+    for L in layers:
+        shape = conv_shape(cur.shape[0], cur.shape[1], cur.shape[2], L["ic"], L["oc"], (L["kernel"],) * 2,
+                           (L["stride"],) * 2, (1, 1), L["pad"])
+        fn = orc.conv_dw_int8 if L["kind"] == "dw" else orc.conv_int8
+        cur = fn(cur, L["w"], L["bias"], shape, L["sx"], L["zx"], L["sw"], L["zw"], L["so"], L["zo"], L["act"])
+        outs.append(cur)
+    return outs
+
+
+@pytest.mark.gpu
+def test_activations_stay_on_the_device_between_provider_kernels(H, orc):
+    """Configuration 2 as a graph of four provider kernels whose intermediate tensors are shared objects.  By default
+    every kernel publishes its device buffer on the output tensor and also fills the host copy; the next kernel reads
+    the device buffer in place.  With the interior outputs declared device-only the host copies never come into being
+    and only the last output travels back.  Both ways, run twice (second time on another image, of another size):
+    every host-visible output equals the oracle's, the first image's last output the committed golden hash."""
+    import hashlib
+    import json
+    from mindspore_amd import workloads as wl
+    hashes = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "config_hashes.json")))["c2"]
+    orc.set_threads(16)
+    x, layers = wl.mobilenet_c2()
+    x2 = np.random.default_rng(9).integers(-128, 128, (2, 97, 61, 3), dtype=np.int8)
+    want = {0: _c2_oracle(orc, x, layers), 1: _c2_oracle(orc, x2, layers)}
+    for device_only in (None, b"stem, expand,dw", b"*"):
+        nodes = _c2_nodes(H, x.shape, layers, device_only)
+        for which, image in ((0, x), (1, x2), (0, x)):
+            nodes[0].run(image)
+            for node in nodes[1:]:
+                node.run_linked()
+            for i, node in enumerate(nodes):
+                host, dev = node.state()
+                interior = i + 1 < len(nodes)
+                assert dev, (device_only, i)
+                if device_only is None:
+                    assert host
+                    got, _ = node.output()
+                    assert got.shape == want[which][i].shape and np.array_equal(got, want[which][i]), (which, i)
+                elif interior or device_only == b"*":
+                    assert not host, (device_only, i)  # never allocated: nothing was copied back
+            if device_only != b"*":
+                got, _ = nodes[-1].output()
+                assert np.array_equal(got, want[which][-1]), (device_only, which)
+                if which == 0:
+                    assert hashlib.sha256(np.ascontiguousarray(got).tobytes()).hexdigest() == hashes["project"]
+        for node in reversed(nodes):
+            node.close()
+
+
+@pytest.mark.gpu
+def test_dynamic_quant_feeds_the_dynamic_matmul_on_the_device(H, orc):
+    """DynamicQuant -> dynamic MatMul sharing the int8 tensor: the bytes stay in device memory (declared device-only),
+    the scale and zero point still reach the host tensor, where the MatMul reads them at Execute."""
+    rng = np.random.default_rng(14)
+    w = rng.integers(-127, 128, (80, 96), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, 80).astype(np.float32).astype(np.float64)
+    bias = rng.standard_normal(80).astype(np.float32)
+    zw = np.zeros(80, np.int32)
+    for per_row in (False, True):
+        dq_op = op(DYNQUANT, symmetric=1, n_prefer_axes=1, prefer_axes=(0,)) if per_row else op(DYNQUANT)
+        dq = Node(H, dq_op, [tensor(F32, (37, 96), None)], I8, out_name=b"q", device_only=b"q")
+        assert dq.stage == OK, (dq.stage, dq.code)
+        mm = Node(H, op(MATMUL, transpose_b=1),
+                  [tensor(I8, (37, 96), None), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+                   tensor(F32, (80,), bias, True)], F32, producer=dq, out_name=b"y", device_only=b"q")
+        assert mm.stage == OK, (mm.stage, mm.code)
+        for rows in (37, 5, 64):
+            x = (rng.standard_normal((rows, 96)) * 3).astype(np.float32)
+            _, qp = dq.run(x)
+            assert dq.state() == (False, True)
+            mm.run_linked()
+            y, _ = mm.output()
+            if per_row:
+                q_ref, scales_ref, _ = orc.dynamic_quant_segments(x, True)
+                assert [p[0] for p in qp] == list(scales_ref)
+                ref = orc.dynamic_matmul_rows(q_ref, w, bias, scales_ref, 0, sw, zw)
+            else:
+                q_ref, s_ref, z_ref = orc.dynamic_quant(x, False)
+                assert qp == [(s_ref, z_ref)]
+                ref = orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw)
+            assert y.shape == ref.shape and np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (per_row, rows)
+        mm.close()
+        dq.close()
+
+
+@pytest.mark.gpu
+def test_a_foreign_device_address_on_an_input_is_not_followed(H, orc):
+    """An address on the input tensor that no kernel of this provider published (an application may attach memory of
+    another device) is ignored: the kernel reads the host data."""
+    rng = np.random.default_rng(15)
+    m, n, k = 9, 40, 64
+    a, w, sw, b, ins = _fc_inputs(rng, m, n, k)
+    node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)])
+    assert node.stage == OK, (node.stage, node.code)
+    H.ph_set_input_device_data(node.h, 0x1000)
+    got, _ = node.run(a)
+    assert np.array_equal(got, orc.matmul_int8(a, w, b, 0.02, -3, sw, np.zeros(n, np.int32), 0.05, 5, 0, True))
+    node.close()
