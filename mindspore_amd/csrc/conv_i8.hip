@@ -16,6 +16,7 @@
 namespace mi {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
 
 __global__ __launch_bounds__(256) void pad_rows_kernel(const int8_t *__restrict__ src, int64_t src_ld, int rows,
                                                        int k, int8_t *__restrict__ dst, int k16) {
@@ -200,40 +201,54 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const int8_t *__restrict__
   }
 }
 
-// Channel-vectorised variant for C % 16 == 0: one thread produces 16 consecutive channels of one output pixel, so
-// every tap is one 16-byte activation load and two 16-byte weight loads, and the store is one 16-byte row segment.
+// Channel-vectorised variant for C % 8 == 0: one thread produces CG = 16 (or 8, when C is not a multiple of 16)
+// consecutive channels of one output pixel, so every tap is one CG-byte activation load and 2 * CG bytes of weights,
+// and the store is one CG-byte row segment.
 // A tap outside the image reads as the input zero point (the matching -zx * w is already in bias_folded), so the
 // inner product is sum_t x_t * w_t with no subtraction.  TAPS > 0 (kernel_h * kernel_w known at compile time): the
-// loads of all taps are issued before the first multiply.  TAPS == 0: any kernel size, tap by tap.
-template <int TAPS>
+// loads of all taps are issued before the first multiply.  TAPS == 0: any kernel size, tap by tap.  FAST: the host
+// proved the cheap rounding form exact for every channel (no left shifts to fetch).
+template <int TAPS, int CG, bool FAST>
 __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict__ in, ConvGeom g,
                                                         const int16_t *__restrict__ w16,
                                                         const int32_t *__restrict__ bias_folded, int zx8,
                                                         RequantParams rq, int8_t *__restrict__ out) {
-  const int ch = g.out_c, groups = ch >> 4;
+  static_assert(CG == 8 || CG == 16, "channels per thread");
+  constexpr int XW = CG / 4;  // dwords of activations per tap
+  constexpr int WQ = CG / 8;  // 16-byte vectors of int16 weights per tap
+  const int ch = g.out_c, groups = ch / CG;
   const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * groups;
   const int zsplat = (zx8 & 0xff) * 0x01010101;
   union XV {
-    v4i v;
-    int8_t b[16];
+    int32_t d[XW];
+    int8_t b[CG];
   };
   union WV {
-    v4i v[2];
-    int16_t h[16];
+    v4i v[WQ];
+    int16_t h[CG];
+  };
+  auto load_x = [](const int8_t *p, XV *x) {
+    if constexpr (CG == 16) {
+      const v4i v = *reinterpret_cast<const v4i *>(p);
+      x->d[0] = v.x, x->d[1] = v.y, x->d[2] = v.z, x->d[3] = v.w;
+    } else {
+      const v2i v = *reinterpret_cast<const v2i *>(p);
+      x->d[0] = v.x, x->d[1] = v.y;
+    }
   };
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
     const int64_t p = idx / groups;
-    const int c0 = (int)(idx - p * groups) << 4;
+    const int c0 = (int)(idx - p * groups) * CG;
     const int b = (int)(p / ((int64_t)g.out_h * g.out_w));
     const int rem = (int)(p - (int64_t)b * g.out_h * g.out_w);
     const int oh = rem / g.out_w, ow = rem - oh * g.out_w;
     const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * ch + c0;
-    uint32_t acc[16];
+    uint32_t acc[CG];
     {
       const v4i *bp = reinterpret_cast<const v4i *>(bias_folded + c0);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < CG / 4; ++q) {
         const v4i bv = bp[q];
         acc[4 * q + 0] = (uint32_t)bv.x;
         acc[4 * q + 1] = (uint32_t)bv.y;
@@ -242,12 +257,10 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
       }
     }
     auto mac = [&](XV xv, const WV &wv, bool inside) {
-      xv.v.x = inside ? xv.v.x : zsplat;
-      xv.v.y = inside ? xv.v.y : zsplat;
-      xv.v.z = inside ? xv.v.z : zsplat;
-      xv.v.w = inside ? xv.v.w : zsplat;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[j] += (uint32_t)((int32_t)xv.b[j] * (int32_t)wv.h[j]);  // 8 bit x 10 bit
+      for (int q = 0; q < XW; ++q) xv.d[q] = inside ? xv.d[q] : zsplat;
+#pragma unroll
+      for (int j = 0; j < CG; ++j) acc[j] += (uint32_t)((int32_t)xv.b[j] * (int32_t)wv.h[j]);  // 8 bit x 10 bit
     };
     auto tap_address = [&](int kh, int kw, bool *inside) -> const int8_t * {
       const int ih = oh * g.stride_h - g.pad_u + kh * g.dilation_h;
@@ -264,10 +277,10 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) {
         const int kh = t / g.kernel_w, kw = t - kh * g.kernel_w;
-        xv[t].v = *reinterpret_cast<const v4i *>(tap_address(kh, kw, &inside[t]));
+        load_x(tap_address(kh, kw, &inside[t]), &xv[t]);
         const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)t * ch + c0);
-        wv[t].v[0] = wp[0];
-        wv[t].v[1] = wp[1];
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) wv[t].v[q] = wp[q];
       }
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) mac(xv[t], wv[t], inside[t]);
@@ -277,26 +290,27 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
           XV xv;
           WV wv;
           bool inside;
-          xv.v = *reinterpret_cast<const v4i *>(tap_address(kh, kw, &inside));
+          load_x(tap_address(kh, kw, &inside), &xv);
           const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)(kh * g.kernel_w + kw) * ch + c0);
-          wv.v[0] = wp[0];
-          wv.v[1] = wp[1];
+#pragma unroll
+          for (int q = 0; q < WQ; ++q) wv.v[q] = wp[q];
           mac(xv, wv, inside);
         }
     }
     union {
-      v4i v;
-      int8_t b[16];
+      int32_t d[XW];
+      int8_t b[CG];
     } o;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const v4i ls4 = *reinterpret_cast<const v4i *>(rq.lshift + c0 + 4 * q);
+    for (int q = 0; q < CG / 4; ++q) {
       const v4i m4 = *reinterpret_cast<const v4i *>(rq.mult + c0 + 4 * q);
       const v4i rs4 = *reinterpret_cast<const v4i *>(rq.rshift + c0 + 4 * q);
+      v4i ls4 = {0, 0, 0, 0};
+      if (!FAST) ls4 = *reinterpret_cast<const v4i *>(rq.lshift + c0 + 4 * q);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         int32_t y;
-        if (rq.fast) {
+        if (FAST) {
           y = rdiv_pot_fast(srdhm_nosat((int32_t)acc[4 * q + e], m4[e]), rs4[e], (1 << rs4[e]) >> 1);
         } else {
           y = rdiv_pot(srdhm((int32_t)(acc[4 * q + e] << ls4[e]), m4[e]), rs4[e]);
@@ -307,21 +321,44 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
         o.b[4 * q + e] = (int8_t)y;
       }
     }
-    *reinterpret_cast<v4i *>(out + p * ch + c0) = o.v;
+    if constexpr (CG == 16) {
+      *reinterpret_cast<v4i *>(out + p * ch + c0) = v4i{o.d[0], o.d[1], o.d[2], o.d[3]};
+    } else {
+      *reinterpret_cast<v2i *>(out + p * ch + c0) = v2i{o.d[0], o.d[1]};
+    }
+  }
+}
+
+template <int TAPS, int CG>
+static void launch_dw_vec(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias_folded, int zx8,
+                          const RequantParams &rq, int8_t *out, hipStream_t stream) {
+  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * (g.out_c / CG);
+  const int64_t want = (total + 255) / 256;
+  const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
+  if (rq.fast) {
+    hipLaunchKernelGGL((conv_dw16_kernel<TAPS, CG, true>), dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded,
+                       zx8, rq, out);
+  } else {
+    hipLaunchKernelGGL((conv_dw16_kernel<TAPS, CG, false>), dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded,
+                       zx8, rq, out);
   }
 }
 
 int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias,
                    const int32_t *bias_folded, int zx8, const RequantParams &rq, int8_t *out, hipStream_t stream) {
-  const bool vec = (g.out_c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
-  const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * (vec ? g.out_c >> 4 : g.out_c);
-  const int64_t want = (total + 255) / 256;
-  const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
-  if (vec && g.kernel_h * g.kernel_w == 9) {
-    hipLaunchKernelGGL(conv_dw16_kernel<9>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded, zx8, rq, out);
-  } else if (vec) {
-    hipLaunchKernelGGL(conv_dw16_kernel<0>, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias_folded, zx8, rq, out);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const bool vec16 = aligned && (g.out_c & 15) == 0, vec8 = aligned && (g.out_c & 7) == 0;
+  const bool taps9 = g.kernel_h * g.kernel_w == 9;
+  if (vec8 && !vec16) {  // 8, 24, 40, ... channels
+    if (taps9) launch_dw_vec<9, 8>(in, g, w16, bias_folded, zx8, rq, out, stream);
+    else launch_dw_vec<0, 8>(in, g, w16, bias_folded, zx8, rq, out, stream);
+  } else if (vec16) {
+    if (taps9) launch_dw_vec<9, 16>(in, g, w16, bias_folded, zx8, rq, out, stream);
+    else launch_dw_vec<0, 16>(in, g, w16, bias_folded, zx8, rq, out, stream);
   } else {
+    const int64_t total = (int64_t)g.batch * g.out_h * g.out_w * g.out_c;
+    const int64_t want = (total + 255) / 256;
+    const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
     hipLaunchKernelGGL(conv_dw_kernel, dim3(blocks), dim3(256), 0, stream, in, g, w16, bias, zx8, rq, out);
   }
   MI_HIP_CHECK(hipGetLastError());

@@ -203,6 +203,8 @@ DW_CASES = [
     (1, 15, 18, 16, (5, 5), (1, 2), (1, 1), (2, 2, 2, 2)),
     (2, 11, 9, 32, (3, 3), (2, 1), (2, 2), (2, 2, 2, 2)),
     (1, 4, 4, 48, (3, 3), (1, 1), (1, 1), (2, 2, 2, 2)),
+    (1, 28, 28, 24, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1)),   # 8 channels per thread
+    (2, 10, 12, 40, (5, 5), (2, 2), (1, 1), (2, 2, 2, 2)),
 ]
 
 
