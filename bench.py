@@ -419,7 +419,7 @@ def main():
         if ceiling and "gemv_decode_m1" in extra:
             extra["gemv_decode_m1"]["frac_of_read_stream"] = extra["gemv_decode_m1"]["gbps"] / ceiling
         extra.update(section("bert", lambda: bench_bert(max(5, args.steps // 2), 3)) or {})
-        extra.update(section("small_configs", lambda: bench_small_configs(max(5, args.steps // 2), 3)) or {})
+        extra.update(section("small_configs", lambda: bench_small_configs(max(200, args.steps), 20)) or {})
     result = {
         "metric": "int8 GEMM TOPS + % i8 MFMA peak; decode GEMV HBM GB/s; vs nnacl CPU",
         "value": g["tops"], "unit": "TOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -747,6 +747,11 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
   int k16 = 0;
   if (h->direct_1x1) {
     if ((rc = prepare_rows(in_dev, (int)pixels, k, &h->col_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  } else if (k <= 64 && d.out_channel <= 128 && (d.out_channel & 3) == 0 &&
+             (reinterpret_cast<uintptr_t>(out_dev) & 3) == 0) {
+    // a first-layer convolution: gathered straight from the image, no im2col buffer
+    return launch_conv_smallk(in_dev, g, h->fill, k, static_cast<const int8_t *>(h->st.w.p), h->st.ldw, h->st.params(),
+                              out_dev, s);
   } else {
     k16 = round_up(k, 16);
     if ((rc = h->col_ws.ensure((size_t)pixels * k16)) != MI_OK) return rc;

@@ -99,6 +99,10 @@ struct ConvGeom {
 };
 // im2col into [batch*out_h*out_w][k16] with K order (kh, kw, ic); out-of-image taps are `fill`, the K tail is zero.
 int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, int k16, hipStream_t stream);
+// Dense convolution with kernel_h * kernel_w * in_c <= 64 and out_c <= 128, out_c % 4 == 0, straight from the image
+// (no im2col buffer); w: packed row-major weights with row stride ldw, K order (kh, kw, ic).
+int launch_conv_smallk(const int8_t *in, const ConvGeom &g, int fill, int k_true, const int8_t *w, int ldw,
+                       const RequantParams &rq, int8_t *out, hipStream_t stream);
 // Depthwise conv + requantisation, weights pre-offset to int16 [KH*KW][C].  bias_folded = bias - zx8 * sum_t w16[t][c]
 // (used by the channel-vectorised kernel, which reads out-of-image taps as zx8); rq.fast: the host proved the cheap
 // rounding form exact for every channel.

@@ -8,7 +8,8 @@
 //              convolution_1x1_int8.cc:396)
 //   conv_dw  : depthwise conv + requantisation (ConvDwInt8 / ConvDwInt8Post,
 //              .../nnacl/int8/conv_depthwise_int8.c:24-140)
-// All three are HBM/latency bound byte movers: one thread produces 16 contiguous output bytes (or one output
+//   conv_smallk : dense convolution with kernel_h * kernel_w * in_c <= 64 in one launch, gathered from the image
+// The first three are HBM/latency bound byte movers: one thread produces 16 contiguous output bytes (or one output
 // element for the depthwise kernel, consecutive threads on consecutive channels) so stores coalesce.
 #include "common.h"
 #include "quant_math.h"
@@ -17,6 +18,7 @@ namespace mi {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 
 __global__ __launch_bounds__(256) void pad_rows_kernel(const int8_t *__restrict__ src, int64_t src_ld, int rows,
                                                        int k, int8_t *__restrict__ dst, int k16) {
@@ -162,6 +164,153 @@ int launch_im2col(const int8_t *in, const ConvGeom &g, int fill, int8_t *dst, in
   const int64_t want = (total + 255) / 256;
   const int blocks = (int)(want < 1 ? 1 : (want > 1048576 ? 1048576 : want));
   hipLaunchKernelGGL(im2col_kernel, dim3(blocks), dim3(256), 0, stream, in, g, fill, dst, k16);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+// Dense convolution with a short contraction (kernel_h * kernel_w * in_c <= 64, the first layer of an image network:
+// 3x3 on 3 channels is K = 27) without an im2col buffer and its extra launch.  One wave produces 32 output pixels x
+// all output channels with v_mfma_i32_32x32x32_i8: lane (r, h) gathers bytes [16h, 16h + 16) of every 32-byte K step
+// of pixel r straight from the image, in the K order (kh, kw, ic) of Im2ColPackUnitInt8Opt (conv_int8.c:758-807),
+// taps outside the image read as `fill` (conv_int8.c:877), bytes past K as 0; the weights come from the packed
+// row-major copy (zero filled past K).  Same exact epilogue as the GEMM.
+template <int KSTEPS, int OCB>
+__global__ __launch_bounds__(256) void conv_smallk_kernel(const int8_t *__restrict__ in, ConvGeom g, int fill,
+                                                          int k_true, const int8_t *__restrict__ w, int ldw,
+                                                          RequantParams rq, int8_t *__restrict__ out) {
+  const int lane = threadIdx.x & 63, r = lane & 31, h = lane >> 5;
+  const int64_t first = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 32;
+  const int64_t pixels = (int64_t)g.batch * g.out_h * g.out_w;
+  if (first >= pixels) return;  // the whole wave
+  const bool live = first + r < pixels;
+  const int64_t p = live ? first + r : pixels - 1;
+  const int b = (int)(p / ((int64_t)g.out_h * g.out_w));
+  const int rem = (int)(p - (int64_t)b * g.out_h * g.out_w);
+  const int oh = rem / g.out_w, ow = rem - oh * g.out_w;
+  const int ih0 = oh * g.stride_h - g.pad_u, iw0 = ow * g.stride_w - g.pad_l;
+  const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * g.in_c;
+
+  union Frag {
+    v4i v;
+    int8_t b[16];
+  };
+  Frag x[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s) {
+    const int k0 = 32 * s + 16 * h;
+    int tap = k0 / g.in_c, ic = k0 - tap * g.in_c;
+    int kh = tap / g.kernel_w, kw = tap - kh * g.kernel_w;
+    // no load is predicated: a byte that is not wanted is fetched from the pixel's image origin and replaced, so
+    // that all sixteen loads are in flight together
+    int8_t raw[16];
+    int other[16];  // -1: take the loaded byte; otherwise the value to use instead
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int ih = ih0 + kh * g.dilation_h, iw = iw0 + kw * g.dilation_w;
+      const bool in_k = k0 + i < k_true;
+      const bool inside = ih >= 0 && ih < g.in_h && iw >= 0 && iw < g.in_w;
+      const int64_t off = (in_k && inside) ? ((int64_t)ih * g.in_w + iw) * g.in_c + ic : 0;
+      raw[i] = img[off];
+      other[i] = in_k ? (inside ? -1 : (fill & 0xff)) : 0;
+      const bool wrap_c = ic + 1 == g.in_c;
+      const bool wrap_w = wrap_c && kw + 1 == g.kernel_w;
+      ic = wrap_c ? 0 : ic + 1;
+      kw = wrap_w ? 0 : (wrap_c ? kw + 1 : kw);
+      kh = wrap_w ? kh + 1 : kh;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[s].b[i] = other[i] < 0 ? raw[i] : (int8_t)other[i];
+  }
+
+  v16i acc[OCB];
+#pragma unroll
+  for (int ob = 0; ob < OCB; ++ob)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[ob][e] = 0;
+#pragma unroll
+  for (int s = 0; s < KSTEPS; ++s)
+#pragma unroll
+    for (int ob = 0; ob < OCB; ++ob) {
+      const v4i wf = *reinterpret_cast<const v4i *>(w + (int64_t)(ob * 32 + r) * ldw + 32 * s + 16 * h);
+      acc[ob] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf, x[s].v, acc[ob], 0, 0, 0);
+    }
+  int rowsum = 0;
+  if (rq.has_zw) {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      rowsum = __builtin_amdgcn_sdot4(x[s].v.x, 0x01010101, rowsum, false);
+      rowsum = __builtin_amdgcn_sdot4(x[s].v.y, 0x01010101, rowsum, false);
+      rowsum = __builtin_amdgcn_sdot4(x[s].v.z, 0x01010101, rowsum, false);
+      rowsum = __builtin_amdgcn_sdot4(x[s].v.w, 0x01010101, rowsum, false);
+    }
+    rowsum += __shfl_xor(rowsum, 32);
+  }
+
+  // acc[ob][4 * q + e] is output channel 32 * ob + 8 * q + 4 * h + e of pixel r
+#pragma unroll
+  for (int ob = 0; ob < OCB; ++ob) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int nb = ob * 32 + q * 8 + h * 4;
+      if (nb >= g.out_c) continue;
+      const v4i mult4 = *reinterpret_cast<const v4i *>(rq.mult + nb);
+      const v4i bias4 = *reinterpret_cast<const v4i *>(rq.bias2 + nb);
+      const v4i e4 = *reinterpret_cast<const v4i *>(rq.rshift + nb);
+      v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0};
+      if (rq.has_zw) zw4 = *reinterpret_cast<const v4i *>(rq.zw + nb);
+      if (!rq.fast) ls4 = *reinterpret_cast<const v4i *>(rq.lshift + nb);
+      union {
+        uint32_t u;
+        int8_t b[4];
+      } o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t v = (uint32_t)acc[ob][q * 4 + e];
+        if (rq.has_zw) v -= (uint32_t)rowsum * (uint32_t)zw4[e];
+        v += (uint32_t)bias4[e];
+        int32_t t;
+        if (rq.fast) {
+          t = rdiv_pot_fast(srdhm_nosat((int32_t)v, mult4[e]), e4[e], (1 << e4[e]) >> 1);
+        } else {
+          t = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
+        }
+        t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
+        t = t < rq.amax ? t : rq.amax;
+        t = t > rq.amin ? t : rq.amin;
+        o.b[e] = (int8_t)t;
+      }
+      if (live) *reinterpret_cast<uint32_t *>(out + p * g.out_c + nb) = o.u;
+    }
+  }
+}
+
+int launch_conv_smallk(const int8_t *in, const ConvGeom &g, int fill, int k_true, const int8_t *w, int ldw,
+                       const RequantParams &rq, int8_t *out, hipStream_t stream) {
+  const int64_t pixels = (int64_t)g.batch * g.out_h * g.out_w;
+  if (k_true < 1 || k_true > 64 || g.out_c < 4 || g.out_c > 128 || (g.out_c & 3) != 0 ||
+      (reinterpret_cast<uintptr_t>(out) & 3) != 0 || (reinterpret_cast<uintptr_t>(w) & 15) != 0 || (ldw & 15) != 0 ||
+      ldw < 64 || pixels < 1) {
+    set_error("conv_smallk: unsupported geometry k=%d oc=%d", k_true, g.out_c);
+    return MI_PARAM_INVALID;
+  }
+  const int64_t waves = (pixels + 31) / 32;
+  const int blocks = (int)((waves + 3) / 4);
+  const int ocb = (g.out_c + 31) / 32, ksteps = (k_true + 31) / 32;
+#define MI_SMALLK(KS, OB)                                                                                       \
+  hipLaunchKernelGGL((conv_smallk_kernel<KS, OB>), dim3(blocks), dim3(256), 0, stream, in, g, fill, k_true, w, ldw, \
+                     rq, out)
+  if (ksteps == 1) {
+    if (ocb == 1) MI_SMALLK(1, 1);
+    else if (ocb == 2) MI_SMALLK(1, 2);
+    else if (ocb == 3) MI_SMALLK(1, 3);
+    else MI_SMALLK(1, 4);
+  } else {
+    if (ocb == 1) MI_SMALLK(2, 1);
+    else if (ocb == 2) MI_SMALLK(2, 2);
+    else if (ocb == 3) MI_SMALLK(2, 3);
+    else MI_SMALLK(2, 4);
+  }
+#undef MI_SMALLK
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }

@@ -153,6 +153,11 @@ CONV_CASES = [
     (1, 40, 40, 32, 64, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1)),
     (3, 28, 28, 64, 300, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0)),
     (1, 30, 30, 24, 16, (7, 7), (2, 2), (1, 1), (3, 3, 3, 3)),
+    # short contraction (K <= 64): gathered straight from the image
+    (2, 13, 11, 4, 96, (4, 4), (1, 1), (1, 1), (1, 2, 2, 1)),
+    (1, 9, 9, 3, 128, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1)),
+    (1, 9, 9, 1, 36, (5, 5), (1, 1), (2, 2), (4, 4, 4, 4)),
+    (1, 64, 48, 3, 32, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1)),
 ]
 
 
