@@ -26,6 +26,8 @@
 // outputs that only kernels of this provider consume: their host copy is skipped as well.
 // A creator returns nullptr for everything the library does not reproduce bit-exactly; the scheduler then falls back
 // to the builtin CPU kernel (mindspore/lite/src/litert/scheduler.cc:1173-1177).
+#include <stdlib.h>
+
 #include <map>
 #include <memory>
 #include <mutex>
@@ -48,8 +50,12 @@ namespace {
 constexpr int kWeightIndex = 1;
 constexpr int kBiasIndex = 2;
 
+// The GPU the provider runs on: HIP device 0, or the one MI355X_DEVICE names (a CPUDeviceInfo has no device id).
 bool LibraryReady() {
-  static const bool ok = (mi_init(0) == MI_OK);
+  static const bool ok = [] {
+    const char *device = getenv("MI355X_DEVICE");
+    return mi_init(device != nullptr ? atoi(device) : 0) == MI_OK;
+  }();
   return ok;
 }
 
@@ -91,13 +97,14 @@ class Published {
   }
 
  private:
+  // never destroyed: kernels owned by a session with static storage may be torn down after this file's statics
   static std::mutex &Mutex() {
-    static std::mutex m;
-    return m;
+    static std::mutex *m = new std::mutex;
+    return *m;
   }
   static std::unordered_set<void *> &Set() {
-    static std::unordered_set<void *> s;
-    return s;
+    static std::unordered_set<void *> *s = new std::unordered_set<void *>;
+    return *s;
   }
 };
 
