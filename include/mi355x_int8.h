@@ -119,9 +119,13 @@ void mi_matmul_destroy(mi_matmul *h);
  * (NN/int8/conv1x1_int8.c:31-40), Conv1x1InputPack (NN/base/conv1x1_base.c:19-40), ConvInt8 /
  * Im2ColPackUnitInt8Opt (NN/int8/conv_int8.c:758-913), MatMulInt8_8x8_r (NN/int8/matmul_int8.c:333-364),
  * ConvDwInt8 / ConvDwInt8Post (NN/int8/conv_depthwise_int8.c:24-140).
- * mi_conv_create returns MI_NOT_SUPPORT for what the provider must leave to the builtin kernels: 3x3 stride-1
- * dilation-1 dense convolutions (the reference runs an integer Winograd there on x86, which is not an exact
- * convolution) and grouped convolutions other than depthwise. */
+ * mi_conv_create returns MI_NOT_SUPPORT for what the provider must leave to the builtin kernels: grouped
+ * convolutions other than depthwise, and 3x3 stride-1 dilation-1 dense convolutions unless MI_CONV_3X3_EXACT is set.
+ * For those the reference's choice of kernel depends on the CPU (LK/int8/convolution_int8_creator.cc:81-94): ARM64
+ * cores with the dot-product extension run ConvolutionInt8CPUKernel, the exact convolution this library computes,
+ * every other build (x86 included) runs Convolution3x3Int8CPUKernel, an integer Winograd whose results differ from
+ * the exact convolution.  With the flag the library reproduces the former; without it it declines. */
+#define MI_CONV_3X3_EXACT 1
 typedef struct mi_conv mi_conv;
 
 typedef struct mi_conv_desc {
@@ -137,6 +141,7 @@ typedef struct mi_conv_desc {
   int32_t filter_quant_num;    /* 1 or out_channel */
   const double *filter_scales;
   const int32_t *filter_zps;
+  int32_t flags; /* 0 or MI_CONV_3X3_EXACT */
 } mi_conv_desc;
 
 /* weight_host: [OC][KH][KW][IC] for group 1, [C][KH][KW] for depthwise; bias_host int32 [OC] or NULL. */

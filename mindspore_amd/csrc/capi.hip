@@ -630,9 +630,14 @@ static int mi_conv_create_impl(const mi_conv_desc *d, const int8_t *weight_host,
     set_error("grouped convolution (group=%d) is left to the builtin kernel", d->group);
     return MI_NOT_SUPPORT;
   }
+  if ((d->flags & ~MI_CONV_3X3_EXACT) != 0) {
+    set_error("mi_conv_create: unknown flags 0x%x", d->flags);
+    return MI_PARAM_INVALID;
+  }
   if (!depthwise && d->kernel_h == 3 && d->kernel_w == 3 && d->stride_h == 1 && d->stride_w == 1 &&
-      d->dilation_h == 1 && d->dilation_w == 1) {
-    set_error("3x3 stride-1 dilation-1 convolution is left to the builtin (Winograd) kernel");
+      d->dilation_h == 1 && d->dilation_w == 1 && (d->flags & MI_CONV_3X3_EXACT) == 0) {
+    set_error("3x3 stride-1 dilation-1 convolution is left to the builtin (Winograd) kernel; MI_CONV_3X3_EXACT "
+              "selects the exact convolution the reference runs on ARM64 cores with dot-product instructions");
     return MI_NOT_SUPPORT;
   }
   int rc = check_filter_quant(d->filter_quant_num, d->out_channel, d->filter_scales, d->filter_zps);

@@ -133,11 +133,13 @@ class FullconnectionInt8Kernel(MatmulInt8Kernel):
 
 class ConvolutionInt8Kernel(_Handle):
     """Conv2DFusion int8, NHWC.  weight [OC, KH, KW, IC] (group 1) or [C, KH, KW] (depthwise, group == C).
-    pad = (up, down, left, right).  Raises MiError with code MI_NOT_SUPPORT for the cases a provider must decline."""
+    pad = (up, down, left, right).  Raises MiError with code MI_NOT_SUPPORT for the cases a provider must decline.
+    exact_3x3: take dense 3x3 stride-1 convolutions too, computing the exact convolution as the reference does on
+    ARM64 cores with dot-product instructions (other builds of the reference run an integer Winograd there)."""
     _destroy = "mi_conv_destroy"
 
     def __init__(self, weight, bias, in_quant, weight_quant, out_quant, stride=(1, 1), dilation=(1, 1),
-                 pad=(0, 0, 0, 0), group=1, act=ACT_NONE, device=0):
+                 pad=(0, 0, 0, 0), group=1, act=ACT_NONE, device=0, exact_3x3=False):
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)
@@ -160,7 +162,8 @@ class ConvolutionInt8Kernel(_Handle):
         nq, scales, zps = _quant_arrays(weight_quant)
         d = _lib.ConvDesc(ic, oc, kh, kw, stride[0], stride[1], dilation[0], dilation[1], pad[0], pad[1], pad[2],
                           pad[3], group, act, float(in_quant.scale), int(in_quant.zero_point),
-                          float(out_quant.scale), int(out_quant.zero_point), nq, scales, zps)
+                          float(out_quant.scale), int(out_quant.zero_point), nq, scales, zps,
+                          _lib.CONV_3X3_EXACT if exact_3x3 else 0)
         _lib.check(L.mi_conv_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                     C.byref(self._h)), "mi_conv_create")
 

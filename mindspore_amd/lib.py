@@ -39,7 +39,10 @@ class ConvDesc(C.Structure):
         "pad_u", "pad_d", "pad_l", "pad_r", "group", "act_type")] + [
         ("in_scale", C.c_double), ("in_zp", C.c_int32), ("out_scale", C.c_double), ("out_zp", C.c_int32),
         ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
-        ("filter_zps", C.POINTER(C.c_int32))]
+        ("filter_zps", C.POINTER(C.c_int32)), ("flags", C.c_int32)]
+
+
+CONV_3X3_EXACT = 1
 
 
 class DynmmDesc(C.Structure):

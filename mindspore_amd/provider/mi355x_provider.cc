@@ -24,6 +24,10 @@
 //   device_only_outputs=<tensor name>,<tensor name>,...      (or * for every output)
 // (Model::LoadConfig / UpdateConfig, delivered through Kernel::GetConfig, include/api/kernel_api.h:112-126) names
 // outputs that only kernels of this provider consume: their host copy is skipped as well.
+// Dense 3x3 stride-1 convolutions are declined by default: x86 builds of the reference run an integer Winograd there
+// (convolution_int8_creator.cc:81-94), whose results are not those of the exact convolution.  MI355X_CONV3X3=exact in
+// the environment makes the provider take them and compute the exact convolution, which is what the reference runs
+// on ARM64 cores with dot-product instructions -- for models validated on such devices.
 // A creator returns nullptr for everything the library does not reproduce bit-exactly; the scheduler then falls back
 // to the builtin CPU kernel (mindspore/lite/src/litert/scheduler.cc:1173-1177).
 #include <stdlib.h>
@@ -57,6 +61,12 @@ bool LibraryReady() {
     return mi_init(device != nullptr ? atoi(device) : 0) == MI_OK;
   }();
   return ok;
+}
+
+// A creator cannot see the session config (the scheduler hands it over after creation), hence the environment.
+bool Exact3x3() {
+  const char *v = getenv("MI355X_CONV3X3");
+  return v != nullptr && std::string(v) == "exact";
 }
 
 // Per-tensor activation quantisation is all the builtin kernels accept too (convolution_base.cc:334-342,368-375).
@@ -389,6 +399,7 @@ class ConvKernel : public kernel::Kernel {
     d.filter_quant_num = static_cast<int32_t>(scales.size());
     d.filter_scales = scales.data();
     d.filter_zps = zps.data();
+    d.flags = Exact3x3() ? MI_CONV_3X3_EXACT : 0;
     const void *bias = inputs_.size() > kBiasIndex ? inputs_[kBiasIndex].Data().get() : nullptr;
     // MI_NOT_SUPPORT (3x3 stride-1 Winograd case, grouped convolution) surfaces here as an error; the creator
     // below screens those cases out first so that the scheduler falls back instead
@@ -421,9 +432,10 @@ std::shared_ptr<kernel::Kernel> ConvCreator(const std::vector<MSTensor> &in, con
   const bool depthwise = cv->group() > 1 && cv->group() == cv->in_channel() && cv->group() == cv->out_channel();
   if (cv->group() != 1 && !depthwise) return nullptr;
   // on x86 the reference runs its integer Winograd for dense 3x3 stride-1 dilation-1 convolutions
-  // (convolution_int8_creator.cc:41-73), whose results are not those of the exact convolution: leave them to it
+  // (convolution_int8_creator.cc:81-94), whose results are not those of the exact convolution: leave them to it
+  // unless the deployment asked for the exact convolution (the reference's choice on ARM64 with dot product)
   if (!depthwise && kh == 3 && kw == 3 && cv->stride()->Get(0) == 1 && cv->stride()->Get(1) == 1 &&
-      cv->dilation()->Get(0) == 1 && cv->dilation()->Get(1) == 1) {
+      cv->dilation()->Get(0) == 1 && cv->dilation()->Get(1) == 1 && !Exact3x3()) {
     return nullptr;
   }
   return std::make_shared<ConvKernel>(in, out, prim, ctx);

@@ -176,9 +176,10 @@ def _conv_case(rng, b, ih, iw, ic, oc, kernel, stride, dil, pad, peroc, zwnz, hb
     return dict(x=x, w=w, bias=bias, shape=shape, sx=sx, zx=zx, sw=sw, zw=zw, so=so, zo=zo, act=act)
 
 
-def _gpu_conv(case, stride, dil, pad, group=1, device_tensors=False):
+def _gpu_conv(case, stride, dil, pad, group=1, device_tensors=False, exact_3x3=False):
     kern = K.ConvolutionInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
-                                   QP(case["so"], case["zo"]), stride, dil, pad, group, case["act"])
+                                   QP(case["so"], case["zo"]), stride, dil, pad, group, case["act"],
+                                   exact_3x3=exact_3x3)
     if device_tensors:
         import torch
         out = kern.run(torch.from_numpy(case["x"]).cuda())
@@ -233,6 +234,26 @@ def test_conv_declines_what_the_provider_must_not_claim():
     with pytest.raises(K._lib.MiError) as e:  # grouped, not depthwise
         K.ConvolutionInt8Kernel(np.zeros((8, 3, 3), np.int8), None, QP(0.1, 0), [QP(0.1, 0)], QP(0.1, 0), (2, 2),
                                 group=4)
+    assert e.value.code == K._lib.MI_NOT_SUPPORT
+
+
+@pytest.mark.parametrize("shape", [(1, 14, 14, 64, 96), (2, 9, 11, 5, 12), (1, 56, 56, 64, 64), (1, 7, 7, 3, 8)])
+def test_dense_3x3_stride_1_as_the_exact_convolution(orc, shape):
+    """With MI_CONV_3X3_EXACT the library takes the convolutions it otherwise leaves to the reference's Winograd
+    kernel and computes ConvInt8 on them, the kernel the reference itself selects on ARM64 with dot product
+    (convolution_int8_creator.cc:81-94): compared with nnacl's ConvInt8 on the same inputs."""
+    b, ih, iw, ic, oc = shape
+    rng = np.random.default_rng(ih * 100 + ic)
+    orc.set_threads(16)
+    for it in range(4):
+        pad = [(1, 1, 1, 1), (0, 0, 0, 0), (1, 0, 0, 1), (2, 2, 2, 2)][it]
+        case = _conv_case(rng, b, ih, iw, ic, oc, (3, 3), (1, 1), (1, 1), pad, bool(it & 1), bool(it & 2), it != 3,
+                          [0, 1, 3, 0][it])
+        got = _gpu_conv(case, (1, 1), (1, 1), pad, 1, device_tensors=bool(it & 1), exact_3x3=True)
+        want = orc.conv_int8(**case)
+        assert got.shape == want.shape and np.array_equal(got, want), (shape, it)
+    with pytest.raises(K._lib.MiError) as e:
+        _gpu_conv(case, (1, 1), (1, 1), pad, 1)
     assert e.value.code == K._lib.MI_NOT_SUPPORT
 
 

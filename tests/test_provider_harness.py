@@ -479,3 +479,28 @@ def test_a_foreign_device_address_on_an_input_is_not_followed(H, orc):
     got, _ = node.run(a)
     assert np.array_equal(got, orc.matmul_int8(a, w, b, 0.02, -3, sw, np.zeros(n, np.int32), 0.05, 5, 0, True))
     node.close()
+
+
+@pytest.mark.gpu
+def test_dense_3x3_stride_1_is_taken_on_request(H, orc, monkeypatch):
+    """Declined by default (x86 builds of the reference run a Winograd kernel there); with MI355X_CONV3X3=exact the
+    provider computes the exact convolution, the reference's own choice on ARM64 with dot product."""
+    from oracle.pyoracle import conv_shape
+    rng = np.random.default_rng(31)
+    x = rng.integers(-128, 128, (1, 12, 10, 16), dtype=np.int8)
+    w = rng.integers(-128, 128, (24, 3, 3, 16), dtype=np.int8)
+    sw = rng.uniform(1e-3, 1e-2, 24).astype(np.float32).astype(np.float64)
+    bias = rng.integers(-3000, 3000, 24).astype(np.int32)
+    conv = op(CONV, kernel=(3, 3), stride=(1, 1), dilation=(1, 1), pad_mode=1, in_channel=16, out_channel=24, act=1)
+    ins = lambda: [tensor(I8, x.shape, None, False, [(0.03, 2)]), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+                   tensor(I32, (24,), bias, True)]
+    monkeypatch.delenv("MI355X_CONV3X3", raising=False)
+    assert Node(H, conv, ins(), I8, [(0.08, -4)]).stage == DECLINED
+    monkeypatch.setenv("MI355X_CONV3X3", "exact")
+    node = Node(H, conv, ins(), I8, [(0.08, -4)])
+    assert node.stage == OK, (node.stage, node.code)
+    got, _ = node.run(x)
+    shape = conv_shape(1, 12, 10, 16, 24, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1))
+    want = orc.conv_int8(x, w, bias, shape, 0.03, 2, sw, np.zeros(24, np.int32), 0.08, -4, 1)
+    assert got.shape == want.shape and np.array_equal(got, want)
+    node.close()
