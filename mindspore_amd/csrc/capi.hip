@@ -334,6 +334,7 @@ struct mi_conv {
   int fill = 0;
   RequantState st;
   DevBuf w16, dw_bias, dw_bias_folded, col_ws, c_ws, h_in, h_out;
+  DevBuf fill16;  // 16 bytes of `fill`: where the gathering GEMM loader reads taps outside the image
 };
 
 struct mi_dynquant {
@@ -694,6 +695,7 @@ static int mi_conv_create_impl(const mi_conv_desc *d, const int8_t *weight_host,
     h->fill = is_1x1 ? 0 : d->in_zp;
     rc = h->st.build(weight_host, oc, kdim, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
                      d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
+    if (rc == MI_OK) rc = upload(&h->fill16, std::vector<int8_t>(16, (int8_t)h->fill));
   }
   if (rc != MI_OK) {
     return rc;
@@ -757,6 +759,10 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
     // a first-layer convolution: gathered straight from the image, no im2col buffer
     return launch_conv_smallk(in_dev, g, h->fill, k, static_cast<const int8_t *>(h->st.w.p), h->st.ldw, h->st.params(),
                               out_dev, s);
+  } else if (pixels > 128 && gemm_conv_supported(g, in_dev, out_dev)) {
+    // 16-channel-aligned images: the GEMM gathers its activation operand from the image, no im2col buffer
+    WeightView w{static_cast<const int8_t *>(h->st.w.p), h->st.k_pad, h->st.ldw, nullptr};
+    return launch_gemm_conv_requant(in_dev, g, static_cast<const int8_t *>(h->fill16.p), w, h->st.params(), out_dev, s);
   } else {
     k16 = round_up(k, 16);
     if ((rc = h->col_ws.ensure((size_t)pixels * k16)) != MI_OK) return rc;

@@ -109,6 +109,12 @@ int launch_conv_smallk(const int8_t *in, const ConvGeom &g, int fill, int k_true
 int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, const int32_t *bias,
                    const int32_t *bias_folded, int zx8, const RequantParams &rq, int8_t *out, hipStream_t stream);
 
+// The requantising GEMM with its activation operand gathered from an NHWC image (in_c % 16 == 0): the im2col
+// convolution without the buffer.  fill16: 16 bytes of the value out-of-image taps take, in device memory.
+bool gemm_conv_supported(const ConvGeom &g, const void *in, const void *out);
+int launch_gemm_conv_requant(const int8_t *in, const ConvGeom &g, const int8_t *fill16, const WeightView &w,
+                             const RequantParams &rq, int8_t *out, hipStream_t stream);
+
 // Measurement aids: read `bytes` and discard them / copy them, 16 bytes per lane.
 int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream);
 int launch_copy16(void *dst, const void *src, int64_t bytes, hipStream_t stream);

@@ -354,8 +354,19 @@ __device__ __forceinline__ void hint_interleave_reads() {
 // OCC = workgroups the register allocation leaves room for on one CU (waves per SIMD): 1 for the 256 x 256 tile, which
 // needs the whole register file, 2 for the 128 x 128 tile.
 // =====================================================================================================================
-template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+// CONV: the activation operand is not a matrix in memory but the im2col view of an NHWC image (in_c % 16 == 0): row m
+// is output pixel m, and the 16-byte chunk at K offset k is 16 channels of tap k / in_c, fetched straight from the
+// image, or from 16 bytes of the fill value when the tap lies outside the image (conv_int8.c:758-807,877).
+struct ConvGather {
+  int in_h, in_w, in_c, out_w, out_hw;
+  int kernel_w, stride_h, stride_w, dil_h, dil_w, pad_u, pad_l;
+  uint32_t magic_ic, magic_kw;  // ceil(2^32 / in_c), ceil(2^32 / kernel_w): exact quotients for dividends < 2^16
+  const int8_t *fill16;
+};
+
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, bool CONV>
+__device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const RequantParams &rq, const DequantParams &dq,
+                                                 const ConvGather &cv) {
   constexpr int BKD = 64, PD = NST - 1;  // PD: prefetch distance in K steps
   static_assert(NST >= 3, "the loop keeps NST - 1 >= 2 tiles in flight");
   auto wrap = [](int x) { return x >= NST ? x - NST : x; };  // stage index after an increment of at most NST
@@ -386,11 +397,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
   const int dchunk = (lane & 3) ^ ((lane >> 3) & 3);
   const int8_t *wsrc = g.w + (int64_t)(n0 + wave * WPW * 16 + drow) * g.ldw + dchunk * 16;
   const int8_t *asrc[APW];
+  int ih0[CONV ? APW : 1], iw0[CONV ? APW : 1];
 #pragma unroll
   for (int i = 0; i < APW; ++i) {
     int m = m0 + (wave * APW + i) * 16 + drow;
     m = m < g.m ? m : g.m - 1;
-    asrc[i] = g.a + (int64_t)m * g.lda;
+    if (CONV) {
+      const int b = m / cv.out_hw, rem = m - b * cv.out_hw;
+      const int oh = rem / cv.out_w, ow = rem - oh * cv.out_w;
+      ih0[i] = oh * cv.stride_h - cv.pad_u;
+      iw0[i] = ow * cv.stride_w - cv.pad_l;
+      // address of (ih0, iw0, channel 0); only dereferenced for taps inside the image
+      asrc[i] = g.a + (((int64_t)b * cv.in_h + ih0[i]) * cv.in_w + iw0[i]) * cv.in_c;
+    } else {
+      asrc[i] = g.a + (int64_t)m * g.lda;
+    }
   }
   // A has exactly K valid bytes per row (the weights are zero padded, A is the caller's): a 16-byte chunk past K is
   // fetched from the row's last chunk instead
@@ -401,6 +422,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
 #pragma unroll
     for (int i = 0; i < WPW; ++i) async_copy16(wsrc + (int64_t)i * 16 * g.ldw + kt * BKD, sw + i * 1024);
     int koff = kt * BKD + dchunk * 16;
+    if (CONV) {
+      const uint32_t tap = __umulhi((uint32_t)koff, cv.magic_ic);
+      const int ic = koff - (int)tap * cv.in_c;
+      const uint32_t kh = cv.kernel_w == 1 ? tap : __umulhi(tap, cv.magic_kw);
+      const int dh = (int)kh * cv.dil_h, dw = ((int)tap - (int)kh * cv.kernel_w) * cv.dil_w;
+      const int tap_off = (dh * cv.in_w + dw) * cv.in_c + ic;
+      const bool in_k = koff < g.k;  // past K the weights are zero: any 16 readable bytes will do
+#pragma unroll
+      for (int i = 0; i < APW; ++i) {
+        const int ih = ih0[i] + dh, iw = iw0[i] + dw;
+        const bool inside = in_k && (unsigned)ih < (unsigned)cv.in_h && (unsigned)iw < (unsigned)cv.in_w;
+        async_copy16(inside ? asrc[i] + tap_off : cv.fill16, sa + i * 1024);
+      }
+      return;
+    }
     koff = koff < a_last ? koff : a_last;
 #pragma unroll
     for (int i = 0; i < APW; ++i) async_copy16(asrc[i] + koff, sa + i * 1024);
@@ -488,6 +524,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
                                                    m0 + wm * WM, r, h);
 }
 
+template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+  gemm_direct_body<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST, false>(g, rq, dq, ConvGather{});
+}
+
+// The same GEMM with the activation operand gathered from an NHWC image (no im2col buffer).
+template <int TILE_N, int TILE_M, bool HAS_ZW, bool FAST, int NST, int OCC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_conv_kernel(GemmArgs g, ConvGather cv, RequantParams rq) {
+  gemm_direct_body<TILE_N, TILE_M, EPI_REQUANT, HAS_ZW, FAST, NST, true>(g, rq, DequantParams{}, cv);
+}
+
 // ---- host side -----------------------------------------------------------------------------------------------
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4, int OCC = 1>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
@@ -563,6 +610,60 @@ int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
   }
   return rq.fast ? launch_pick_tile<EPI_REQUANT, false, true>(g, rq, dq, stream)
                  : launch_pick_tile<EPI_REQUANT, false, false>(g, rq, dq, stream);
+}
+
+template <int TILE_N, int TILE_M, bool HAS_ZW, bool FAST, int NST, int OCC>
+static int launch_conv_cfg(GemmArgs g, const ConvGather &cv, const RequantParams &rq, hipStream_t stream) {
+  g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
+  g.tiles_n = (g.n + TILE_N - 1) / TILE_N;
+  auto kern = gemm_conv_kernel<TILE_N, TILE_M, HAS_ZW, FAST, NST, OCC>;
+  hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g, cv, rq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <bool HAS_ZW, bool FAST>
+static int launch_conv_pick_tile(const GemmArgs &g, const ConvGather &cv, const RequantParams &rq,
+                                 hipStream_t stream) {
+  const int64_t tiles_m = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
+  // up to 64 output channels: half-width tiles (three workgroups per CU) instead of half-empty square ones
+  if (g.n <= 64 && g.m >= 128 * 128) return launch_conv_cfg<64, 128, HAS_ZW, FAST, 4, 3>(g, cv, rq, stream);
+  if (tiles_m >= 128) return launch_conv_cfg<128, 128, HAS_ZW, FAST, 4, 2>(g, cv, rq, stream);
+  return launch_conv_cfg<64, 64, HAS_ZW, FAST, 4, 1>(g, cv, rq, stream);
+}
+
+bool gemm_conv_supported(const ConvGeom &cg, const void *in, const void *out) {
+  const int64_t k = (int64_t)cg.kernel_h * cg.kernel_w * cg.in_c;
+  return (cg.in_c & 15) == 0 && k <= 65536 - 128 && (int64_t)cg.in_h * cg.in_w * cg.in_c < ((int64_t)1 << 31) &&
+         (int64_t)cg.batch * cg.out_h * cg.out_w < ((int64_t)1 << 31) && (cg.out_c & 3) == 0 &&
+         (reinterpret_cast<uintptr_t>(in) & 15) == 0 && (reinterpret_cast<uintptr_t>(out) & 3) == 0;
+}
+
+int launch_gemm_conv_requant(const int8_t *in, const ConvGeom &cg, const int8_t *fill16, const WeightView &w,
+                             const RequantParams &rq, int8_t *out, hipStream_t stream) {
+  const int64_t k64 = (int64_t)cg.kernel_h * cg.kernel_w * cg.in_c;
+  const int64_t m64 = (int64_t)cg.batch * cg.out_h * cg.out_w;
+  if (in == nullptr || fill16 == nullptr || w.w == nullptr || out == nullptr) {
+    set_error("gemm_conv: null pointer");
+    return MI_NULL_PTR;
+  }
+  if (!gemm_conv_supported(cg, in, out) || m64 <= 0 || cg.out_c <= 0 || w.k_pad % kKPad != 0 || w.k_pad < k64 ||
+      w.ldw < w.k_pad || (w.ldw & 15) != 0) {
+    set_error("gemm_conv: unsupported geometry ic=%d k=%lld pixels=%lld oc=%d", cg.in_c, (long long)k64,
+              (long long)m64, cg.out_c);
+    return MI_PARAM_INVALID;
+  }
+  const auto magic = [](int d) { return d <= 1 ? 0u : (uint32_t)((((uint64_t)1 << 32) + d - 1) / (uint64_t)d); };
+  ConvGather cv{cg.in_h,     cg.in_w,       cg.in_c,       cg.out_w,  cg.out_h * cg.out_w, cg.kernel_w, cg.stride_h,
+                cg.stride_w, cg.dilation_h, cg.dilation_w, cg.pad_u,  cg.pad_l,            magic(cg.in_c),
+                magic(cg.kernel_w), fill16};
+  GemmArgs g{in, 0, (int)m64, (int)k64, w.w, w.ldw, w.k_pad, cg.out_c, 0, 0, out, cg.out_c};
+  if (rq.has_zw) {
+    return rq.fast ? launch_conv_pick_tile<true, true>(g, cv, rq, stream)
+                   : launch_conv_pick_tile<true, false>(g, cv, rq, stream);
+  }
+  return rq.fast ? launch_conv_pick_tile<false, true>(g, cv, rq, stream)
+                 : launch_conv_pick_tile<false, false>(g, cv, rq, stream);
 }
 
 int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,

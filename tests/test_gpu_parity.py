@@ -158,6 +158,13 @@ CONV_CASES = [
     (1, 9, 9, 3, 128, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1)),
     (1, 9, 9, 1, 36, (5, 5), (1, 1), (2, 2), (4, 4, 4, 4)),
     (1, 64, 48, 3, 32, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1)),
+    # 16-channel-aligned images with more than 128 output pixels: the GEMM gathers from the image, no im2col buffer
+    (1, 33, 31, 32, 20, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2)),
+    (2, 30, 30, 80, 36, (1, 1), (2, 2), (1, 1), (1, 1, 1, 1)),
+    (1, 20, 20, 16, 8, (5, 5), (1, 1), (1, 1), (2, 2, 2, 2)),
+    (1, 20, 24, 16, 8, (3, 1), (1, 2), (1, 1), (1, 1, 0, 0)),
+    (2, 96, 96, 16, 132, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1)),
+    (1, 23, 17, 48, 64, (2, 4), (1, 1), (3, 2), (3, 3, 4, 4)),
 ]
 
 
@@ -237,7 +244,8 @@ def test_conv_declines_what_the_provider_must_not_claim():
     assert e.value.code == K._lib.MI_NOT_SUPPORT
 
 
-@pytest.mark.parametrize("shape", [(1, 14, 14, 64, 96), (2, 9, 11, 5, 12), (1, 56, 56, 64, 64), (1, 7, 7, 3, 8)])
+@pytest.mark.parametrize("shape", [(1, 14, 14, 64, 96), (2, 9, 11, 5, 12), (1, 56, 56, 64, 64), (1, 7, 7, 3, 8),
+                                   (4, 64, 64, 16, 128), (4, 64, 66, 16, 40)])
 def test_dense_3x3_stride_1_as_the_exact_convolution(orc, shape):
     """With MI_CONV_3X3_EXACT the library takes the convolutions it otherwise leaves to the reference's Winograd
     kernel and computes ConvInt8 on them, the kernel the reference itself selects on ARM64 with dot product
