@@ -207,6 +207,7 @@ def bench_bert(steps, warmup):
 def bench_small_configs(steps, warmup):
     """Configuration 1 (FullConnection 128x768x768) and configuration 2 (MobileNetV2-style block, device-resident
     chain of stem 3x3 s2, 1x1 expand, 3x3 depthwise, 1x1 project): latency per layer, algorithmic bytes moved."""
+    import numpy as np
     import torch
     from mindspore_amd import kernels as K
     from mindspore_amd import workloads as wl
@@ -250,6 +251,26 @@ def bench_small_configs(steps, warmup):
     ms, _ = time_steps(graph.replay, steps, warmup)
     total_us = ms * 1e3
     out["c2_block_graph_us"] = total_us
+    # a mid-network 3x3 convolution (batch 32, 56 x 56 x 64 -> 64, stride 1; taken with MI_CONV_3X3_EXACT): the GEMM
+    # gathers its activation operand from the image.  Ten calls per graph.
+    rng = np.random.default_rng(3)
+    xin = torch.from_numpy(rng.integers(-128, 128, (32, 56, 56, 64), dtype=np.int8)).cuda()
+    wt = rng.integers(-128, 128, (64, 3, 3, 64), dtype=np.int8)
+    qp = [K.QuantParam(float(sc), 0) for sc in rng.uniform(1e-3, 1e-2, 64)]
+    kern = K.ConvolutionInt8Kernel(wt, None, K.QuantParam(0.02, 3), qp, K.QuantParam(0.5, -2), (1, 1), (1, 1),
+                                   (1, 1, 1, 1), 1, 0, exact_3x3=True)
+    yout = kern.run(xin)
+    with torch.cuda.stream(side):
+        kern.run(xin, out=yout)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(10):
+                kern.run(xin, out=yout)
+    torch.cuda.synchronize()
+    ms, _ = time_steps(graph.replay, max(10, steps // 10), 3)
+    us = ms * 1e3 / 10
+    out["conv3x3_b32_56x56x64"] = dict(us=us, tops=2.0 * yout.numel() * 9 * 64 / (us * 1e-6) / 1e12,
+                                       algorithmic_bytes=int(xin.numel() + yout.numel() + wt.size))
     return out
 
 
