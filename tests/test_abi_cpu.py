@@ -106,6 +106,10 @@ def test_device_entry_points_fail_cleanly_without_init(L):
     assert L.mi_diag_stream_read(None, 16, None) == lib.MI_NULL_PTR
     assert L.mi_diag_copy(None, None, 16, None) == lib.MI_NULL_PTR
     assert L.mi_diag_mfma_rate(None, 1, 1, None, None) == lib.MI_NULL_PTR
+    assert L.mi_device_malloc(64, None) == lib.MI_NULL_PTR
+    assert L.mi_copy_to_device(None, None, 8, None) == lib.MI_NULL_PTR
+    assert L.mi_copy_to_host(None, None, 8, None) == lib.MI_NULL_PTR
+    assert L.mi_copy_to_device(None, None, 0, None) == lib.MI_OK and L.mi_device_free(None) == lib.MI_OK
     h = C.c_void_p()
     assert L.mi_matmul_create(None, None, None, C.byref(h)) == lib.MI_NULL_PTR
     import torch
@@ -116,4 +120,10 @@ def test_device_entry_points_fail_cleanly_without_init(L):
         w = np.zeros((4, 8), np.int8)
         rc = L.mi_matmul_create(C.byref(d), w.ctypes.data, None, C.byref(h))
         assert rc == lib.MI_ERROR and b"mi_init" in L.mi_last_error()
+        p = C.c_void_p()
+        assert L.mi_device_malloc(64, C.byref(p)) == lib.MI_ERROR and p.value is None
+        assert L.mi_stream_synchronize(None) == lib.MI_ERROR
+        d3 = lib.ConvDesc(4, 8, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0.1, 0, 0.1, 0, 1, scales, zps, 2)
+        assert L.mi_conv_create(C.byref(d3), np.zeros((8, 3, 3, 4), np.int8).ctypes.data, None,
+                                C.byref(h)) == lib.MI_PARAM_INVALID  # unknown flag bit
         assert L.mi_init(0) == lib.MI_NOT_SUPPORT
