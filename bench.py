@@ -8,7 +8,7 @@ requantising epilogue); the decode GEMV (configuration 4, batch 1), DynamicQuant
 timed region.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm4096|gemm8192] [--no-cpu] [--no-extra]
-                    [--calibrate]
+                    [--calibrate] [--conv3x3]
 """
 import argparse
 import json
@@ -268,8 +268,19 @@ def bench_small_configs(steps, warmup):
     ms, _ = time_steps(graph.replay, steps, warmup)
     total_us = ms * 1e3
     out["c2_block_graph_us"] = total_us
-    # a mid-network 3x3 convolution (batch 32, 56 x 56 x 64 -> 64, stride 1; taken with MI_CONV_3X3_EXACT): the GEMM
-    # gathers its activation operand from the image.  Ten calls per graph.
+    # a mid-network 3x3 convolution: the GEMM gathers its activation operand from the image
+    kern, xin, yout, nbytes = make_conv3x3()
+    us = time_in_graph(lambda: kern.run(xin, out=yout), steps, 3) * 1e3
+    out["conv3x3_b32_56x56x64"] = dict(us=us, tops=2.0 * yout.numel() * 9 * 64 / (us * 1e-6) / 1e12,
+                                       algorithmic_bytes=nbytes)
+    return out
+
+
+def make_conv3x3():
+    """Batch 32, 56 x 56 x 64 -> 64 channels, 3x3, stride 1, pad 1 (taken with MI_CONV_3X3_EXACT)."""
+    import numpy as np
+    import torch
+    from mindspore_amd import kernels as K
     rng = np.random.default_rng(3)
     xin = torch.from_numpy(rng.integers(-128, 128, (32, 56, 56, 64), dtype=np.int8)).cuda()
     wt = rng.integers(-128, 128, (64, 3, 3, 64), dtype=np.int8)
@@ -277,18 +288,7 @@ def bench_small_configs(steps, warmup):
     kern = K.ConvolutionInt8Kernel(wt, None, K.QuantParam(0.02, 3), qp, K.QuantParam(0.5, -2), (1, 1), (1, 1),
                                    (1, 1, 1, 1), 1, 0, exact_3x3=True)
     yout = kern.run(xin)
-    with torch.cuda.stream(side):
-        kern.run(xin, out=yout)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            for _ in range(10):
-                kern.run(xin, out=yout)
-    torch.cuda.synchronize()
-    ms, _ = time_steps(graph.replay, max(10, steps // 10), 3)
-    us = ms * 1e3 / 10
-    out["conv3x3_b32_56x56x64"] = dict(us=us, tops=2.0 * yout.numel() * 9 * 64 / (us * 1e-6) / 1e12,
-                                       algorithmic_bytes=int(xin.numel() + yout.numel() + wt.size))
-    return out
+    return kern, xin, yout, int(xin.numel() + yout.numel() + wt.size)
 
 
 def cpu_baseline(case, size):
@@ -394,6 +394,8 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch the library's 256 MiB device copy three times (known traffic, for scaling "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--conv3x3", action="store_true",
+                    help="also launch the batch-32 3x3 convolution of the extras 20 times (for profiling that kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this hot path is a single-GPU path; only --gpus 1 is supported (got %d)" % args.gpus,
@@ -475,6 +477,11 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             lib.check(L.mi_diag_copy(dst.data_ptr(), src.data_ptr(), 256 << 20, _stream()), "mi_diag_copy")
+        torch.cuda.synchronize()
+    if args.conv3x3:
+        kern, xin, yout, _ = make_conv3x3()
+        for _ in range(20):
+            kern.run(xin, out=yout)
         torch.cuda.synchronize()
     if "mfma_only" in extra:
         # the matrix pipe alone on operands drawn like this GEMM's: the shader clock it sustains depends on the data
