@@ -627,6 +627,8 @@ static int launch_conv_pick_tile(const GemmArgs &g, const ConvGather &cv, const 
                                  hipStream_t stream) {
   const int64_t tiles_m = (int64_t)((g.m + 127) / 128) * ((g.n + 127) / 128);
   // up to 64 output channels: half-width tiles (three workgroups per CU) instead of half-empty square ones
+  // (more such tiles than three per CU: a fourth workgroup per CU on three stages saves the second round)
+  if (g.n <= 64 && (g.m + 127) / 128 > 768) return launch_conv_cfg<64, 128, HAS_ZW, FAST, 3, 4>(g, cv, rq, stream);
   if (g.n <= 64 && g.m >= 128 * 128) return launch_conv_cfg<64, 128, HAS_ZW, FAST, 4, 3>(g, cv, rq, stream);
   if (tiles_m >= 128) return launch_conv_cfg<128, 128, HAS_ZW, FAST, 4, 2>(g, cv, rq, stream);
   return launch_conv_cfg<64, 64, HAS_ZW, FAST, 4, 1>(g, cv, rq, stream);

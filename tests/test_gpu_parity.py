@@ -245,7 +245,7 @@ def test_conv_declines_what_the_provider_must_not_claim():
 
 
 @pytest.mark.parametrize("shape", [(1, 14, 14, 64, 96), (2, 9, 11, 5, 12), (1, 56, 56, 64, 64), (1, 7, 7, 3, 8),
-                                   (4, 64, 64, 16, 128), (4, 64, 66, 16, 40)])
+                                   (4, 64, 64, 16, 128), (4, 64, 66, 16, 40), (32, 56, 56, 16, 8)])
 def test_dense_3x3_stride_1_as_the_exact_convolution(orc, shape):
     """With MI_CONV_3X3_EXACT the library takes the convolutions it otherwise leaves to the reference's Winograd
     kernel and computes ConvInt8 on them, the kernel the reference itself selects on ARM64 with dot product
