@@ -245,7 +245,10 @@ int orc_matmul_int8(const int8_t *a, const int8_t *w, const int32_t *bias, int8_
  * otherwise -> ConvolutionInt8CPUKernel: im2col rows are pre-filled with zx (NN/int8/conv_int8.c:877) so an
  *   out-of-image tap contributes nothing; K order is (kh, kw, ic) (:794,802); bias fold
  *   LK/int8/convolution_int8.cc:131-142.
- * (3x3 stride 1 dilation 1 goes to an integer Winograd kernel on x86 in the reference and is NOT covered.) */
+ * 3x3 stride 1 dilation 1: the reference's choice depends on the CPU (LK/int8/convolution_int8_creator.cc:81-94).
+ *   ARM64 cores with the dot-product extension run ConvolutionInt8CPUKernel as above, and that is what this function
+ *   computes; every other build (x86 included) runs an integer Winograd kernel, which is NOT restated here (the
+ *   product declines those convolutions unless asked for the exact form). */
 int orc_conv_int8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const orc_conv_shape *s,
                   double sx, int zx, const double *sw, const int32_t *zw, int nfilt, double so, int zo, int act_type) {
   if (nfilt < 1 || (nfilt > 1 && nfilt != s->out_c)) return -1;

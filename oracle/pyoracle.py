@@ -105,6 +105,13 @@ class _Base:
     def conv_int8(self, x, w, bias, shape, sx, zx, sw, zw, so, zo, act=ACT_NONE):
         return self._conv("conv_int8", x, w, bias, shape, sx, zx, sw, zw, so, zo, act)
 
+    def conv_int8_as_arm64_sdot(self, x, w, bias, shape, sx, zx, sw, zw, so, zo, act=ACT_NONE):
+        """ConvInt8 whatever the kernel size: the compiled reference refuses dense 3x3 stride-1 convolutions through
+        conv_int8 (x86 selects a Winograd kernel for them), this entry runs ConvInt8 on them as ARM64 cores with dot
+        product do.  The restatement computes the exact convolution either way."""
+        name = "conv_int8_as_arm64_sdot" if self.prefix == "ref_" else "conv_int8"
+        return self._conv(name, x, w, bias, shape, sx, zx, sw, zw, so, zo, act)
+
     def conv_dw_int8(self, x, w, bias, shape, sx, zx, sw, zw, so, zo, act=ACT_NONE):
         return self._conv("conv_dw_int8", x, w, bias, shape, sx, zx, sw, zw, so, zo, act)
 

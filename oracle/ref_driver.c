@@ -420,12 +420,12 @@ static int ref_conv_1x1(const int8_t *in, const int8_t *w, const int32_t *bias, 
   return 0;
 }
 
-int ref_conv_int8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const ref_conv_shape *s,
-                  double sx, int zx, const double *sw, const int32_t *zw, int nfilt, double so, int zo, int act_type,
-                  int threads, double *run_seconds) {
+static int conv_int8_impl(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const ref_conv_shape *s,
+                          double sx, int zx, const double *sw, const int32_t *zw, int nfilt, double so, int zo,
+                          int act_type, int threads, double *run_seconds, int winograd_guard) {
   if (nfilt < 1 || (nfilt > 1 && nfilt != s->out_c)) return -1;
-  if (s->kernel_h == 3 && s->kernel_w == 3 && s->stride_h == 1 && s->stride_w == 1 && s->dilation_h == 1 &&
-      s->dilation_w == 1)
+  if (winograd_guard && s->kernel_h == 3 && s->kernel_w == 3 && s->stride_h == 1 && s->stride_w == 1 &&
+      s->dilation_h == 1 && s->dilation_w == 1)
     return -2; /* Winograd branch of the reference: not an exact integer convolution */
   if (threads < 1) threads = 1;
   ConvParameter cp;
@@ -439,6 +439,22 @@ int ref_conv_int8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t
   }
   free_conv_quant(&qs);
   return rc;
+}
+
+/* Kernel selection as on x86 (mindspore/lite/src/litert/kernel/cpu/int8/convolution_int8_creator.cc:81-94): dense
+ * 3x3 stride-1 dilation-1 goes to the Winograd kernel there and is refused here. */
+int ref_conv_int8(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out, const ref_conv_shape *s,
+                  double sx, int zx, const double *sw, const int32_t *zw, int nfilt, double so, int zo, int act_type,
+                  int threads, double *run_seconds) {
+  return conv_int8_impl(in, w, bias, out, s, sx, zx, sw, zw, nfilt, so, zo, act_type, threads, run_seconds, 1);
+}
+
+/* Kernel selection as on ARM64 cores with the dot-product extension (same lines: ConvolutionInt8CPUKernel for every
+ * dense kernel size): ConvInt8 also for 3x3 stride 1.  The C code of ConvInt8 is the same on every platform. */
+int ref_conv_int8_as_arm64_sdot(const int8_t *in, const int8_t *w, const int32_t *bias, int8_t *out,
+                                const ref_conv_shape *s, double sx, int zx, const double *sw, const int32_t *zw,
+                                int nfilt, double so, int zo, int act_type, int threads, double *run_seconds) {
+  return conv_int8_impl(in, w, bias, out, s, sx, zx, sw, zw, nfilt, so, zo, act_type, threads, run_seconds, 0);
 }
 
 /* ------------------------------------------------------------------------------------------------------------

@@ -64,8 +64,16 @@ def small_cases(ref):
         (1, 6, 6, 7, 5, (1, 1), (2, 2), (1, 1), (1, 0, 1, 0), 1, 0, 0, 0, 0),
         (1, 10, 10, 4, 6, (5, 3), (1, 1), (2, 1), (4, 4, 1, 1), 0, 0, 1, 3, 0),
         (2, 9, 7, 12, 12, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 1, 1, 1, 3, 1),
-        (1, 8, 8, 5, 5, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), 0, 0, 0, 0, 1)]:
+        (1, 8, 8, 5, 5, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), 0, 0, 0, 0, 1),
+        # 16-channel-aligned images with more than 128 output pixels (the GEMM gathers from the image), the second one
+        # a dense 3x3 stride-1 convolution computed as ConvInt8 (what the reference runs on ARM64 with dot product);
+        # drawn from a generator of their own so that the cases before and after keep their values
+        (1, 24, 24, 16, 12, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), 1, 1, 1, 3, 0),
+        (1, 12, 13, 32, 8, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), 1, 0, 1, 1, 0)]:
         shape = conv_shape(b, ih, iw, ic, oc, kern, st, dil, pad)
+        main_rng = rng
+        if idx >= 7:
+            rng = np.random.default_rng(4242 + idx)
         x = rng.integers(-128, 128, (b, ih, iw, ic), dtype=np.int8)
         w = rng.integers(-128, 128, (oc, kern[0], kern[1]) if dw else (oc, kern[0], kern[1], ic), dtype=np.int8)
         nf = oc if peroc else 1
@@ -76,13 +84,14 @@ def small_cases(ref):
         kdim = kern[0] * kern[1] * (1 if dw else ic)
         so, zo = float(sx * sw.mean() * np.sqrt(kdim) * 100), int(rng.integers(-20, 21))
         ref.threads = 1 + idx % 3
-        fn = ref.conv_dw_int8 if dw else ref.conv_int8
+        fn = ref.conv_dw_int8 if dw else ref.conv_int8_as_arm64_sdot
         y = fn(x, w, bias if hb else None, shape, sx, zx, sw, zw, so, zo, act)
         p = "cv%d_" % idx
         geom = np.array([kern[0], kern[1], st[0], st[1], dil[0], dil[1], pad[0], pad[1], pad[2], pad[3], dw], np.int32)
         out.update({p + "x": x, p + "w": w, p + "bias": bias, p + "sw": sw, p + "zw": zw, p + "geom": geom,
                     p + "meta": np.array([sx, zx, so, zo, act, hb], np.float64), p + "y": y})
         idx += 1
+        rng = main_rng
     out["cv_count"] = np.array([idx])
     # dynamic quant + dynamic matmul
     idx = 0

@@ -8,6 +8,7 @@ import pytest
 
 from mindspore_amd import kernels as K
 from mindspore_amd.kernels import QuantParam as QP
+from oracle import pyoracle
 from oracle.pyoracle import conv_shape
 
 pytestmark = pytest.mark.gpu
@@ -123,7 +124,8 @@ def test_golden_small_cases(orc):
         w = g[p + "w"]
         kern = K.ConvolutionInt8Kernel(w, g[p + "bias"] if hb else None, QP(sx, int(zx)),
                                        _qps(g[p + "sw"], g[p + "zw"]), QP(so, int(zo)), (sh, sw_), (dh, dw_),
-                                       (pu, pd, pl, pr), w.shape[0] if depthwise else 1, int(act))
+                                       (pu, pd, pl, pr), w.shape[0] if depthwise else 1, int(act),
+                                       exact_3x3=not depthwise and (kh, kw, sh, sw_, dh, dw_) == (3, 3, 1, 1, 1, 1))
         assert np.array_equal(kern.run(g[p + "x"]), g[p + "y"]), p
     for i in range(int(g["dq_count"][0])):
         p = "dq%d_" % i
@@ -258,8 +260,12 @@ def test_dense_3x3_stride_1_as_the_exact_convolution(orc, shape):
         case = _conv_case(rng, b, ih, iw, ic, oc, (3, 3), (1, 1), (1, 1), pad, bool(it & 1), bool(it & 2), it != 3,
                           [0, 1, 3, 0][it])
         got = _gpu_conv(case, (1, 1), (1, 1), pad, 1, device_tensors=bool(it & 1), exact_3x3=True)
-        want = orc.conv_int8(**case)
+        want = orc.conv_int8_as_arm64_sdot(**case)
         assert got.shape == want.shape and np.array_equal(got, want), (shape, it)
+        if it == 0 and pyoracle.Reference.available():  # the compiled ConvInt8 itself
+            r = pyoracle.reference()
+            r.threads = 16
+            assert np.array_equal(got, r.conv_int8_as_arm64_sdot(**case)), (shape, "compiled nnacl")
     with pytest.raises(K._lib.MiError) as e:
         _gpu_conv(case, (1, 1), (1, 1), pad, 1)
     assert e.value.code == K._lib.MI_NOT_SUPPORT

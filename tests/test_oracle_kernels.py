@@ -149,6 +149,32 @@ def test_conv_closed_form_and_nnacl(orc, idx):
             assert np.array_equal(got, r.conv_int8(**case)), (idx, it)
 
 
+@pytest.mark.parametrize("geom", [(1, 6, 7, 3, 5), (2, 9, 8, 16, 12), (1, 14, 14, 32, 24), (1, 3, 3, 1, 1)])
+def test_dense_3x3_stride_1_is_conv_int8_when_the_reference_selects_it(orc, geom):
+    """Dense 3x3 stride-1 convolutions: the reference runs ConvInt8 on them on ARM64 cores with dot product and a
+    Winograd kernel elsewhere (convolution_int8_creator.cc:81-94).  The oracle restates ConvInt8; it is checked here
+    against the closed form and against the compiled ConvInt8 itself, reached without the x86 kernel selection."""
+    from oracle import pyoracle
+    b, ih, iw, ic, oc = geom
+    rng = np.random.default_rng(500 + ih + ic)
+    for it in range(6):
+        pad = [(1, 1, 1, 1), (0, 0, 0, 0), (2, 1, 0, 2)][it % 3]
+        if ih + pad[0] + pad[1] < 3 or iw + pad[2] + pad[3] < 3:
+            continue
+        case = _conv_case(rng, b, ih, iw, ic, oc, (3, 3), (1, 1), (1, 1), pad, bool(it & 1), bool(it & 2), it != 3,
+                          [0, 1, 3][it % 3])
+        got = orc.conv_int8_as_arm64_sdot(**case)
+        want = cf.conv_int8(case["x"], case["w"], case["bias"], case["shape"], case["sx"], case["zx"], case["sw"],
+                            case["zw"], case["so"], case["zo"], case["act"])
+        assert np.array_equal(got, want), (geom, it)
+        if pyoracle.Reference.available():
+            r = pyoracle.reference()
+            r.threads = 1 + it % 3
+            assert np.array_equal(got, r.conv_int8_as_arm64_sdot(**case)), (geom, it)
+            with pytest.raises(RuntimeError):  # the x86 selection refuses: Winograd there
+                r.conv_int8(**case)
+
+
 def test_conv1x1_input_pack_reference_vectors(orc):
     """Input1x1PrePack1/2 of the reference (mindspore/lite/test/ut/src/runtime/kernel/arm/int8/
     conv_1x1_int8_tests.cc:32-71) pin the strided/padded 1x1 gather with its zero fill.  With an identity 1x1
