@@ -208,6 +208,10 @@ def test_conv_cases(orc, idx):
         got = _gpu_conv(case, stride, dil, pad, 1, device_tensors=bool(it & 1))
         want = orc.conv_int8(**case)
         assert np.array_equal(got, want), (idx, it, int((got != want).sum()))
+        if it == 2 and pyoracle.Reference.available():  # and the compiled nnacl itself
+            r = pyoracle.reference()
+            r.threads = 16
+            assert np.array_equal(got, r.conv_int8(**case)), (idx, "compiled nnacl")
 
 
 DW_CASES = [
