@@ -127,3 +127,19 @@ def test_device_entry_points_fail_cleanly_without_init(L):
         assert L.mi_conv_create(C.byref(d3), np.zeros((8, 3, 3, 4), np.int8).ctypes.data, None,
                                 C.byref(h)) == lib.MI_PARAM_INVALID  # unknown flag bit
         assert L.mi_init(0) == lib.MI_NOT_SUPPORT
+
+
+def test_public_header_is_plain_c(tmp_path):
+    """include/mi355x_int8.h is the drop-in boundary: it has to compile as C99 and as C++11 on its own."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "mi355x_int8.h"\n'
+                   "int main(void) { mi_conv_desc d = {0}; mi_matmul_desc m = {0}; return d.flags + m.deep; }\n")
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include")
+    for cmd in (["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror"],
+                ["g++", "-std=c++11", "-Wall", "-Werror", "-x", "c++"]):
+        p = subprocess.run(cmd + ["-I", inc, "-fsyntax-only", str(src)], capture_output=True, text=True)
+        assert p.returncode == 0, p.stderr
