@@ -273,6 +273,12 @@ int mi_infer_conv2d(const int32_t *in_shape, int32_t in_dims, const int32_t *w_s
  * copies play in the reference.  Copies are ordered on `stream` like the *_run entry points and return when they
  * are complete (the host buffer may be reused at once).  All of them act on the device given to mi_init. */
 int mi_device_malloc(size_t bytes, void **out_dev);
+/* Page-locked host memory, which the GPU copies from and to directly: what a host-side Allocator for the device info
+ * (Allocator::Malloc / Free, include/api/allocator.h:33,48; DeviceInfoContext::SetAllocator, include/api/context.h:217)
+ * hands to tensors so that graph inputs and outputs cross PCIe without a bounce buffer.
+ * mindspore_amd/provider/mi355x_allocator.h builds such an allocator on these two. */
+int mi_host_malloc(size_t bytes, void **out_host);
+int mi_host_free(void *host); /* NULL is allowed */
 int mi_device_free(void *dev); /* NULL is allowed */
 int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream);
 int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream);

@@ -410,6 +410,29 @@ int mi_device_free(void *dev) {
   return MI_OK;
 }
 
+int mi_host_malloc(size_t bytes, void **out_host) {
+  if (out_host == nullptr) return MI_NULL_PTR;
+  *out_host = nullptr;
+  if (bytes == 0) {
+    set_error("mi_host_malloc: zero bytes");
+    return MI_PARAM_INVALID;
+  }
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  if (hipHostMalloc(out_host, bytes, hipHostMallocDefault) != hipSuccess) {
+    *out_host = nullptr;
+    set_error("hipHostMalloc(%zu) failed", bytes);
+    return MI_MEMORY_FAILED;
+  }
+  return MI_OK;
+}
+
+int mi_host_free(void *host) {
+  if (host == nullptr) return MI_OK;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  MI_HIP_CHECK(hipHostFree(host));
+  return MI_OK;
+}
+
 int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream) {
   if (bytes == 0) return MI_OK;
   if (dst_dev == nullptr || src_host == nullptr) return MI_NULL_PTR;

@@ -22,6 +22,7 @@ EXPORTS = [
     "mi_dynmm_destroy",
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
     "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize",
+    "mi_host_malloc", "mi_host_free",
     "mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate",
 ]
 
@@ -134,6 +135,8 @@ def load():
     L.mi_infer_conv2d.argtypes = [pi32, i32, pi32, i32, C.POINTER(ConvInfer), pi32, pi32]
     L.mi_device_malloc.argtypes = [C.c_size_t, C.POINTER(vp)]
     L.mi_device_free.argtypes = [vp]
+    L.mi_host_malloc.argtypes = [C.c_size_t, C.POINTER(vp)]
+    L.mi_host_free.argtypes = [vp]
     L.mi_copy_to_device.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_copy_to_host.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_stream_synchronize.argtypes = [vp]

@@ -24,11 +24,16 @@ def syntax_check_against_reference_headers():
     flatc-generated schema header is the stand-in.  Returns compiler output ('' = clean) or None without the tree."""
     if not os.path.isdir(os.path.join(REFERENCE, "include", "api")):
         return None
-    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-I" + REFERENCE, "-I" + os.path.join(REFERENCE, "mindspore", "lite"),
-           "-I" + os.path.join(REFERENCE, "mindspore", "core"), "-I" + HERE, "-I" + os.path.join(ROOT, "include"),
-           os.path.join(ROOT, "mindspore_amd", "provider", "mi355x_provider.cc")]
-    p = subprocess.run(cmd, capture_output=True, text=True)
-    return (p.stdout + p.stderr).strip() if p.returncode != 0 or p.stderr.strip() else ""
+    out = ""
+    for src in ("mi355x_provider.cc", "mi355x_allocator.h"):
+        cmd = ["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-I" + REFERENCE,
+               "-I" + os.path.join(REFERENCE, "mindspore", "lite"), "-I" + os.path.join(REFERENCE, "mindspore", "core"),
+               "-I" + HERE, "-I" + os.path.join(ROOT, "include"), "-x", "c++",
+               os.path.join(ROOT, "mindspore_amd", "provider", src)]
+        p = subprocess.run(cmd, capture_output=True, text=True)
+        if p.returncode != 0 or p.stderr.strip():
+            out += (p.stdout + p.stderr).strip() + "\n"
+    return out.strip()
 
 
 if __name__ == "__main__":

@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "../../mindspore_amd/provider/mi355x_allocator.h"
 #include "../../mindspore_amd/provider/mi355x_provider.cc"
 
 using mindspore::MSTensor;
@@ -232,4 +233,39 @@ int32_t ph_infer(const ph_op *op, const char *provider, const ph_tensor *inputs,
 }
 
 void ph_destroy(void *h) { delete static_cast<Session *>(h); }
+
+// The pinned allocator as the runtime would use it for tensor data (lite::Tensor::MallocData / FreeData with the
+// reference counting of the executor).  Returns 0, or the number of the first check that failed.
+int32_t ph_allocator_selftest(void) {
+  std::shared_ptr<mindspore::Allocator> a = mindspore::mi355x::MakePinnedAllocator();
+  void *p = a->Malloc(1000);
+  if (p == nullptr) return 1;
+  if (a->RefCount(p) != 0 || a->SetRefCount(p, 2) != 2 || a->DecRefCount(p, 1) != 1 || a->IncRefCount(p, 3) != 4) return 2;
+  int dummy = 0;
+  if (a->RefCount(&dummy) != -1 || a->RefCount(nullptr) != -1 || a->IncRefCount(&dummy, 1) != -1) return 3;
+  memset(p, 0x5a, 1000);
+  a->Free(p);
+  if (a->RefCount(p) != -1) return 4;
+  void *q = a->Malloc(900);  // fits the freed block and is not 64 times smaller: reused, count reset
+  if (q != p || a->RefCount(q) != 0) return 5;
+  void *tiny = a->Malloc(8);  // 1000 > 8 << 6: too wasteful, a new block
+  a->Free(q);
+  void *tiny2 = a->Malloc(8);
+  if (tiny == nullptr || tiny2 == nullptr || tiny2 == q || tiny2 == tiny) return 6;
+  void *big = a->Malloc(size_t{1} << 22);
+  if (big == nullptr) return 7;
+  // the memory is usable by the copies the provider makes
+  void *dev = nullptr;
+  if (mi_device_malloc(size_t{1} << 22, &dev) != MI_OK) return 8;
+  memset(big, 0x3c, size_t{1} << 22);
+  void *back = a->Malloc(size_t{1} << 22);
+  if (back == nullptr || mi_copy_to_device(dev, big, size_t{1} << 22, nullptr) != MI_OK ||
+      mi_copy_to_host(back, dev, size_t{1} << 22, nullptr) != MI_OK || memcmp(big, back, size_t{1} << 22) != 0) {
+    return 9;
+  }
+  mi_device_free(dev);
+  a->Free(nullptr);
+  a->Free(&dummy);  // unknown pointers are left alone
+  return 0;  // everything still allocated is released by the destructor
+}
 }

@@ -504,3 +504,11 @@ def test_dense_3x3_stride_1_is_taken_on_request(H, orc, monkeypatch):
     want = orc.conv_int8(x, w, bias, shape, 0.03, 2, sw, np.zeros(24, np.int32), 0.08, -4, 1)
     assert got.shape == want.shape and np.array_equal(got, want)
     node.close()
+
+
+@pytest.mark.gpu
+def test_pinned_allocator_for_the_device_info(H):
+    """mindspore_amd/provider/mi355x_allocator.h: DefaultAllocator's contract (reuse of freed blocks within 64x,
+    reference counts from 0, -1 for unknown pointers) on page-locked memory that the GPU copies accept."""
+    H.ph_allocator_selftest.restype = C.c_int32
+    assert H.ph_allocator_selftest() == 0
