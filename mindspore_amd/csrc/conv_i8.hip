@@ -355,7 +355,7 @@ __global__ __launch_bounds__(256) void conv_dw_kernel(const int8_t *__restrict__
 // and the store is one CG-byte row segment.
 // A tap outside the image reads as the input zero point (the matching -zx * w is already in bias_folded), so the
 // inner product is sum_t x_t * w_t with no subtraction.  TAPS > 0 (kernel_h * kernel_w known at compile time): the
-// loads of all taps are issued before the first multiply.  TAPS == 0: any kernel size, tap by tap.  FAST: the host
+// loads of all taps are issued before the first multiply.  TAPS == 0: any kernel size, five taps per batch of loads.  FAST: the host
 // proved the cheap rounding form exact for every channel (no left shifts to fetch).
 template <int TAPS, int CG, bool FAST>
 __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict__ in, ConvGeom g,
@@ -434,17 +434,31 @@ __global__ __launch_bounds__(256) void conv_dw16_kernel(const int8_t *__restrict
 #pragma unroll
       for (int t = 0; t < TAPS; ++t) mac(xv[t], wv[t], inside[t]);
     } else {
-      for (int kh = 0; kh < g.kernel_h; ++kh)
-        for (int kw = 0; kw < g.kernel_w; ++kw) {
-          XV xv;
-          WV wv;
-          bool inside;
-          load_x(tap_address(kh, kw, &inside), &xv);
-          const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)(kh * g.kernel_w + kw) * ch + c0);
+      // five taps at a time (a row of a 5x5 kernel): their loads are issued together, so a kernel of T taps costs
+      // T / 5 memory round trips instead of T
+      constexpr int B = 5;
+      const int taps = g.kernel_h * g.kernel_w;
+      int kh = 0, kw = 0;  // of tap t0 + u, kept by stepping (no division per tap)
+      for (int t0 = 0; t0 < taps; t0 += B) {
+        XV xv[B];
+        WV wv[B];
+        bool inside[B];
 #pragma unroll
-          for (int q = 0; q < WQ; ++q) wv.v[q] = wp[q];
-          mac(xv, wv, inside);
+        for (int u = 0; u < B; ++u) {
+          const bool past = t0 + u >= taps;  // past the last tap: a re-read of the last one that is not used
+          const int t = past ? taps - 1 : t0 + u;
+          load_x(tap_address(past ? g.kernel_h - 1 : kh, past ? g.kernel_w - 1 : kw, &inside[u]), &xv[u]);
+          const bool wrap_w = kw + 1 == g.kernel_w;
+          kw = wrap_w ? 0 : kw + 1;
+          kh = wrap_w ? kh + 1 : kh;
+          const v4i *wp = reinterpret_cast<const v4i *>(w16 + (int64_t)t * ch + c0);
+#pragma unroll
+          for (int q = 0; q < WQ; ++q) wv[u].v[q] = wp[q];
         }
+#pragma unroll
+        for (int u = 0; u < B; ++u)
+          if (t0 + u < taps) mac(xv[u], wv[u], inside[u]);
+      }
     }
     union {
       int32_t d[XW];
@@ -498,7 +512,10 @@ int launch_conv_dw(const int8_t *in, const ConvGeom &g, const int16_t *w16, cons
   const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
   const bool vec16 = aligned && (g.out_c & 15) == 0, vec8 = aligned && (g.out_c & 7) == 0;
   const bool taps9 = g.kernel_h * g.kernel_w == 9;
-  if (vec8 && !vec16) {  // 8, 24, 40, ... channels
+  // kernels larger than 3x3 on few pixels: a thread's chain of taps is what the launch lasts, and there are SIMDs to
+  // spare, so half the channels per thread
+  const bool long_chain = !taps9 && (int64_t)g.batch * g.out_h * g.out_w * (g.out_c >> 4) < 65536;
+  if (vec8 && (!vec16 || long_chain)) {  // 8, 24, 40, ... channels
     if (taps9) launch_dw_vec<9, 8>(in, g, w16, bias_folded, zx8, rq, out, stream);
     else launch_dw_vec<0, 8>(in, g, w16, bias_folded, zx8, rq, out, stream);
   } else if (vec16) {
