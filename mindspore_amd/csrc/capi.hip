@@ -199,7 +199,7 @@ struct RequantState {
       const int64_t vmax = std::min<int64_t>((int64_t)1 << 31, (int64_t)k * 16384 + llabs((long long)h_bias2[c]) +
                                                                    (int64_t)k * 128 * llabs((long long)zwv[c]));
       const int64_t xmax = ((vmax * llabs((long long)h_mult[c])) >> 31) + 1;
-      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN || vmax >= ((int64_t)1 << 31) ||
+      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN || vmax + kAccBias >= ((int64_t)1 << 31) ||
           xmax + ((int64_t)1 << (e[c] - 1)) + (llabs((long long)zo) << e[c]) > INT32_MAX)
         fast = false;
     }

@@ -27,6 +27,10 @@ inline int64_t round_up64(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 constexpr int kNPad = 256;
 constexpr int kKPad = 256;
 
+// The value the 256 x 256 GEMM tile's accumulators start from (taken out again in the epilogue); the host's proof that
+// the cheap rounding form cannot overflow includes it.
+constexpr uint32_t kAccBias = 0x2AAAAAAAu;
+
 // ---- int8 requantising epilogue parameters (device arrays are padded to kNPad entries) ----
 struct RequantParams {
   const int32_t *mult;    // 31-bit mantissa per channel

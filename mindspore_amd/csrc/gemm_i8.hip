@@ -20,6 +20,8 @@
 #include "common.h"
 #include "quant_math.h"
 
+#include <type_traits>
+
 namespace mi {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -121,7 +123,9 @@ struct EpiParams {
   }
 };
 
-template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST>
+// ACC0: the value the accumulators started from (see kAccBias); it leaves through the per-channel constants, so it
+// costs nothing here.
+template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST, uint32_t ACC0 = 0>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)[TM], const GemmArgs &g,
                                               const RequantParams &rq, const DequantParams &dq, const int *p,
                                               char *cstage, int n_tile, int n_w, int m_w, int r, int h) {
@@ -146,7 +150,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         if (nb >= g.n) continue;
         const int *pl = p + (nb - n_tile);
         const v4i mult4 = *reinterpret_cast<const v4i *>(pl);
-        const v4i bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+        v4i bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
         const v4i e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
         v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
         int64_t c64[4] = {0, 0, 0, 0};
@@ -158,10 +162,15 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             pre4[e] = ((1 << e4[e]) >> 1) + (int32_t)((uint32_t)rq.zo << e4[e]);
-            c64[e] = (int64_t)bias4[e] * (int64_t)mult4[e] + ((int64_t)1 << 30);
+            // (acc + ACC0 - ACC0 + bias2) * mult + 2^30, the ACC0 term moved into the constant; 64-bit wrap-around
+            // arithmetic, the true value fits
+            c64[e] = (int64_t)((uint64_t)((int64_t)bias4[e] * (int64_t)mult4[e]) + ((uint64_t)1 << 30) -
+                               (uint64_t)ACC0 * (uint64_t)(int64_t)mult4[e]);
           }
         } else {
           ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) bias4[e] = (int32_t)((uint32_t)bias4[e] - ACC0);
         }
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
@@ -172,7 +181,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
             if (FAST) {
               int32_t v = acc[i][j][q * 4 + e];
               if (HAS_ZW) v -= rowsum[j] * zw4[e];
-              const int64_t p = (int64_t)v * (int64_t)mult4[e] + c64[e];
+              const int64_t p = (int64_t)((uint64_t)((int64_t)v * (int64_t)mult4[e]) + (uint64_t)c64[e]);
               const int32_t x = (int32_t)(p >> 31);
               const int32_t t = (x + pre4[e] + (x >> 31)) >> e4[e];
               y[e] = med3_i32(t, amin_v, amax_v);
@@ -259,7 +268,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
         uint32_t corr[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e];
+        for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e] - ACC0;
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
           v4f o;
@@ -535,6 +544,173 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
   gemm_direct_body<TILE_N, TILE_M, EPI_REQUANT, HAS_ZW, FAST, NST, true>(g, rq, DequantParams{}, cv);
 }
 
+// =====================================================================================================================
+// K-block main loop for the 256 x 256 tile (one workgroup per CU, the whole register file).
+//
+// What the compute-bound GEMM pays for is operand delivery: the L2 -> L1 path moves whole 128-byte lines, so a loader
+// that asks for 64 bytes of a row per K step has every line sent twice, one K step apart.  Here K advances in blocks of 128 bytes
+// -- whole cache lines -- so that each line leaves the L2 once: one wave instruction fetches 8 rows x 128 bytes.
+// LDS holds two slots per operand (slot = 256 rows x 128 B = 32 KiB; 128 KiB in all).  A loop iteration is one K
+// block = four 32-byte MFMA sub-steps (quarters) on double-buffered fragments:
+//   Q1  MFMAs on chunks 0-1 | reads chunks 2-3 | issues the loads of A block b+1 (its slot was released by the
+//                                               previous iteration's barrier)
+//   Q2  MFMAs on chunks 2-3 | reads chunks 4-5
+//   Q3  MFMAs on chunks 4-5 | reads chunks 6-7, then waits for its own LDS reads and loads and meets the other
+//       waves: block b+1 is complete in LDS and nobody reads block b any more
+//   Q4  MFMAs on chunks 6-7 | reads chunks 0-1 of block b+1 | issues the loads of W block b+2 into block b's slot
+// One barrier per 128 bytes of K.  In a slot, 16-byte chunk c of row R sits at position c ^ (R & 7): the loader's
+// 1 KiB writes (8 rows x 8 chunks) and the fragment reads (8 consecutive rows, one logical chunk) both cover all
+// 32 banks.
+//
+// kAccBias: the accumulators start from this constant instead of 0 and the epilogue's per-channel constants take it
+// out again (exact: wrap-around arithmetic).  Partial sums of signed products hover around zero, where every sign
+// change flips all upper bits of the 32-bit accumulator; from an alternating bit pattern a sum that crosses it
+// flips at most the bits up to the next 0/1 boundary.  The matrix pipe alone, on operands drawn like this
+// benchmark's, sustains 7-9 % more (power-limited shader clock) with it.  For the same reason consecutive MFMAs
+// share one operand (serpentine order over the 4 x 4 sub-tiles): +5 %.
+// =====================================================================================================================
+template <int EPI, bool HAS_ZW, bool FAST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kblock_kernel(GemmArgs g,
+                                                                                                      RequantParams rq,
+                                                                                                      DequantParams dq) {
+  constexpr int TILE = 256, KB = 128, T = 4;  // wave tile 128 x 128 = T x T MFMA tiles
+  constexpr int SLOT = TILE * KB;             // one operand, one K block
+  constexpr int LPW = 8;                      // loader instructions per wave, operand and block (64 rows)
+  static_assert(4 * SLOT >= kEpiArrays * TILE * 4 + 4 * epi_stage_bytes<EPI, T>(), "the epilogue staging must fit");
+  __shared__ __attribute__((aligned(1024))) char lds[4 * SLOT];  // W slot 0, W slot 1, A slot 0, A slot 1
+
+  int tile_m, tile_n;
+  tile_coords(g, &tile_m, &tile_n);
+  const int m0 = tile_m * TILE, n0 = tile_n * TILE;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wm = wave >> 1;
+  const int r = lane & 31, h = lane >> 5;
+  const int kblocks = (g.k + KB - 1) / KB;
+  const int kchunks = g.k >> 4;
+  EpiParams<TILE, EPI> epi;
+  epi.fetch(rq, dq, n0, tid);
+
+  // loader: instruction i of a wave fills rows 64 * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
+  // L & 7 of its row, i.e. fetches logical chunk (L & 7) ^ (row & 7)
+  const int drow = lane >> 3;
+  const int dchunk = (lane & 7) ^ drow;
+  const int8_t *wsrc = g.w + (int64_t)(n0 + wave * 64 + drow) * g.ldw + dchunk * 16;
+  const int8_t *asrc[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    int m = m0 + wave * 64 + 8 * i + drow;
+    m = m < g.m ? m : g.m - 1;
+    asrc[i] = g.a + (int64_t)m * g.lda;
+  }
+  const int a_last = (kchunks - 1) * 16;
+  auto dma_w = [&](int slot, int kb) {
+    char *dst = lds + slot * SLOT + wave * 64 * KB;
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) async_copy16(wsrc + (int64_t)(8 * i) * g.ldw + kb * KB, dst + i * 1024);
+  };
+  auto dma_a = [&](int slot, int kb) {
+    char *dst = lds + (2 + slot) * SLOT + wave * 64 * KB;
+    int koff = kb * KB + dchunk * 16;
+    koff = koff < a_last ? koff : a_last;  // past K: any valid read will do, the weights are zero there
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) async_copy16(asrc[i] + koff, dst + i * 1024);
+  };
+
+  v16i acc[T][T];
+#pragma unroll
+  for (int i = 0; i < T; ++i)
+#pragma unroll
+    for (int j = 0; j < T; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = (int)kAccBias;
+  int rowsum[T];
+#pragma unroll
+  for (int j = 0; j < T; ++j) rowsum[j] = 0;
+
+  const int swz = r & 7;
+  const int w_off = (wn * 128 + r) * KB, a_off = 2 * SLOT + (wm * 128 + r) * KB;
+  Frag<T, T> f0, f1;
+  auto read_frag = [&](Frag<T, T> &f, int slot, int q) {  // q: 32-byte sub-step inside the block
+    const char *base = lds + slot * SLOT + (((2 * q + h) ^ swz) << 4);
+#pragma unroll
+    for (int i = 0; i < T; ++i) f.w[i] = *reinterpret_cast<const v4i *>(base + w_off + i * 32 * KB);
+#pragma unroll
+    for (int j = 0; j < T; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * KB);
+  };
+  auto mma = [&](const Frag<T, T> &f, int chunk) {
+    if (HAS_ZW) {
+      const int ones = chunk < kchunks ? 0x01010101 : 0;
+#pragma unroll
+      for (int j = 0; j < T; ++j) {
+        int t = rowsum[j];
+        t = __builtin_amdgcn_sdot4(f.a[j].x, ones, t, false);
+        t = __builtin_amdgcn_sdot4(f.a[j].y, ones, t, false);
+        t = __builtin_amdgcn_sdot4(f.a[j].z, ones, t, false);
+        t = __builtin_amdgcn_sdot4(f.a[j].w, ones, t, false);
+        rowsum[j] = t;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+      for (int jj = 0; jj < T; ++jj) {
+        const int j = (i & 1) ? T - 1 - jj : jj;
+        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.a[j], acc[i][j], 0, 0, 0);
+      }
+  };
+  // one LDS read behind each of the first 8 MFMAs of a quarter, then (when the quarter issues loads) one load
+  // behind each of the other 8
+  auto hints = [&](auto with_loads) {
+#pragma unroll
+    for (int i = 0; i < 2 * T; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+    }
+    if constexpr (decltype(with_loads)::value) {
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  dma_w(0, 0);
+  dma_a(0, 0);
+  dma_w(1, kblocks > 1 ? 1 : 0);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LPW) : "memory");
+  read_frag(f0, 0, 0);
+  for (int b = 0; b < kblocks; ++b) {
+    const int slot = b & 1;
+    const int kb_a = b + 1 < kblocks ? b + 1 : kblocks - 1;  // past the end: re-fetch the last block into a slot
+    const int kb_w = b + 2 < kblocks ? b + 2 : kblocks - 1;  // nobody reads again
+    read_frag(f1, slot, 1);
+    dma_a(slot ^ 1, kb_a);
+    mma(f0, b * 8 + h);
+    hints(std::true_type());
+    read_frag(f0, slot, 2);
+    mma(f1, b * 8 + 2 + h);
+    hints(std::false_type());
+    read_frag(f1, slot, 3);
+    mma(f0, b * 8 + 4 + h);
+    hints(std::false_type());
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    read_frag(f0, slot ^ 1, 0);
+    dma_w(slot, kb_w);
+    mma(f1, b * 8 + 6 + h);
+    hints(std::true_type());
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing re-fetches land before the LDS is reused
+  __syncthreads();
+  epi.to_lds(reinterpret_cast<int *>(lds), tid);
+  gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+                                                         lds + kEpiArrays * TILE * 4 + wave * epi_stage_bytes<EPI, T>(),
+                                                         n0, n0 + wn * 128, m0 + wm * 128, r, h);
+}
+
 // ---- host side -----------------------------------------------------------------------------------------------
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4, int OCC = 1>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
@@ -543,6 +719,16 @@ static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &
   const int blocks = g.tiles_m * g.tiles_n;
   auto kern = gemm_direct_kernel<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST, OCC>;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), 0, stream, g, rq, dq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <int EPI, bool HAS_ZW, bool FAST>
+static int launch_kblock(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
+  g.tiles_m = (g.m + 255) / 256;
+  g.tiles_n = (g.n + 255) / 256;
+  hipLaunchKernelGGL((gemm_kblock_kernel<EPI, HAS_ZW, FAST>), dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g, rq,
+                     dq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -557,7 +743,7 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
   // the fp32 epilogue writes four times the bytes: below one 256 x 256 tile per CU it is worth more to overlap it
   // with another workgroup's main loop (two 128 x 128 tiles per CU) than to save operand traffic
-  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192)) return launch_cfg<256, 256, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192)) return launch_kblock<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // a few hundred activation rows against many channels: 256-channel x 128-row tiles keep the weight re-reads of
   // the square 128 tile away while still giving every CU a tile
   if (g.m <= 512 && (int64_t)((g.m + 127) / 128) * ((g.n + 255) / 256) >= 128)

@@ -82,6 +82,23 @@ def test_decode_rows_every_stream_shape(orc, n, k):
         assert np.array_equal(got, want), (m, n, k, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("m,n,k", [(2100, 6144, 1008), (3073, 4100, 144), (4096, 3072, 64), (2049, 6148, 400)])
+def test_matmul_whole_cu_tile_ragged(orc, m, n, k):
+    """The 256 x 256 tile (128-byte K blocks, biased accumulators) with ragged rows, channels and K: K below one
+    block, K that ends inside a block, inside its first half, per-tensor / per-channel, zero and non-zero weight zero
+    points, the generic rounding path."""
+    rng = np.random.default_rng(m + n + k)
+    orc.set_threads(16)
+    for it in range(4):
+        case = _mm_case(rng, m, n, k, bool(it & 1), bool(it & 2), it != 2, [0, 1, 3, 0][it], it != 3,
+                        1e-3 if it == 3 else 100.0)
+        if it == 3:
+            case["bias"] = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+        got, _ = _gpu_matmul(case, device_tensors=True)
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
+
+
 def test_matmul_generic_rounding_paths(orc):
     """Cases the fast epilogue must not take: real multiplier >= 1 (left shift), shift 0, huge bias (wrap)."""
     rng = np.random.default_rng(5)
@@ -313,7 +330,7 @@ def test_dynamic_matmul(orc):
     rng = np.random.default_rng(401)
     orc.set_threads(16)
     for it, (m, n, k) in enumerate([(1, 1, 1), (5, 9, 17), (33, 70, 64), (130, 65, 300), (9, 256, 1000),
-                                    (700, 300, 129), (64, 2304, 768)]):
+                                    (700, 300, 129), (64, 2304, 768), (4100, 4096, 400), (4097, 4100, 208)]):
         a = rng.integers(-128, 128, (m, k), dtype=np.int8)
         w = rng.integers(-128, 128, (n, k), dtype=np.int8)
         nf = n if it & 1 else 1
