@@ -96,11 +96,26 @@ typedef struct mi_matmul_desc {
   int32_t filter_quant_num;    /* 1 (per tensor) or col (per output channel) */
   const double *filter_scales; /* [filter_quant_num] */
   const int32_t *filter_zps;   /* [filter_quant_num] */
+  int32_t flags;               /* 0 or MI_MATMUL_NO_DECODE_PACK */
 } mi_matmul_desc;
+
+/* All weight packing happens in mi_matmul_create (the role of TransferB, LK/int8/matmul_base_int8.cc:360-384: pack
+ * once at Prepare).  Two packed forms are kept: K-contiguous rows (GEMM tiles; up to 2 activation rows) and 1 KiB
+ * blocks of 16 channels x 64 K-bytes in matrix-core operand order (3..32 activation rows, the batched decode
+ * kernel).  MI_MATMUL_NO_DECODE_PACK skips the second form (deep x col bytes of device memory less) for callers
+ * that know they never run with 3..32 rows; such a handle still accepts those row counts and runs them on the GEMM
+ * tiles.  mi_matmul_run never packs, allocates for packing or waits. */
+#define MI_MATMUL_NO_DECODE_PACK 1
 
 /* weight_host: int8 const weight; bias_host: int32 [col] or NULL.  Both are consumed during the call. */
 int mi_matmul_create(const mi_matmul_desc *desc, const int8_t *weight_host, const int32_t *bias_host,
                      mi_matmul **out);
+/* Sizes the handle's workspaces for runs of up to `max_rows` rows, so that later runs allocate nothing: the role of
+ * the buffers MatmulBaseInt8CPUKernel::ReSize allocates (LK/int8/matmul_base_int8.cc:296-325).  Workspaces exist only
+ * for operand shapes the kernels cannot take in place (deep % 16 != 0 or a misaligned activation base: a padded copy
+ * of the activations; col % 4 != 0 or a misaligned output base: a padded output).  Without this call the first run
+ * that needs a larger workspace allocates it (hipFree + hipMalloc: the device idles meanwhile). */
+int mi_matmul_reserve(mi_matmul *h, int32_t max_rows);
 /* a_dev: int8 [rows, deep]; c_dev: int8 [rows, col].  Asynchronous on `stream`. */
 int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
 /* Same with host tensors: copies in, runs, copies out, synchronises. */
@@ -155,6 +170,10 @@ int mi_conv_same_pad(int32_t in, int32_t kernel, int32_t stride, int32_t dilatio
 int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_dev,
                 void *stream);
 int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_host);
+/* Sizes the handle's workspaces (im2col buffer, padded rows / output, where the shape needs them) for this input
+ * geometry, so that later runs of it allocate nothing: the role of ConvolutionInt8CPUKernel::InitTmpBuffer
+ * (LK/int8/convolution_int8.cc:159-197). */
+int mi_conv_reserve(mi_conv *h, int32_t batch, int32_t in_h, int32_t in_w);
 void mi_conv_destroy(mi_conv *h);
 
 /* ---- DynamicQuant (fp32 -> int8, per tensor) --------------------------------------------------------------- */
@@ -225,6 +244,9 @@ int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_d
                       float *c_dev, void *stream);
 int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
                            float *c_host);
+/* As mi_matmul_reserve (the buffers of MatmulDynamicBaseInt8CPUKernel::ReSize, LK/int8/matmul_dynamic_base_int8.cc:
+ * 204-232). */
+int mi_dynmm_reserve(mi_dynmm *h, int32_t max_rows);
 void mi_dynmm_destroy(mi_dynmm *h);
 
 /* ---- shape inference (host arithmetic, no GPU needed) --------------------------------------------------------------

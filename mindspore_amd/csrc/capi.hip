@@ -140,7 +140,7 @@ static int upload(DevBuf *b, const std::vector<T> &v) {
 struct RequantState {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
-  DevBuf w_blocked;  // built by the first run with 3..32 activation rows
+  DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (3..32 activation rows); built in create or absent
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
   bool has_zw = false, fast = false;
@@ -162,7 +162,7 @@ struct RequantState {
 
   // w_nk: [n][k] row-major (already transposed if needed)
   int build(const int8_t *w_nk, int n_, int k_, const int32_t *bias, double sx, int32_t zx, double so, int32_t zo_,
-            int nfilt, const double *sw, const int32_t *zws, int act, bool pack_weights) {
+            int nfilt, const double *sw, const int32_t *zws, int act, bool pack_weights, bool pack_decode = false) {
     n = n_;
     k = k_;
     n_pad = round_up(n, kNPad);
@@ -215,6 +215,13 @@ struct RequantState {
       std::vector<int8_t> packed((size_t)n_pad * ldw, 0);
       for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * ldw, w_nk + (size_t)c * k, (size_t)k);
       if ((rc = upload(&w, packed)) != MI_OK) return rc;
+      if (pack_decode) {
+        if ((rc = w_blocked.ensure((size_t)n_pad * k_pad)) != MI_OK) return rc;
+        rc = launch_block_weights(static_cast<const int8_t *>(w.p), n_pad, k_pad, ldw, static_cast<int8_t *>(w_blocked.p),
+                                  nullptr);
+        if (rc != MI_OK) return rc;
+        MI_HIP_CHECK(hipStreamSynchronize(nullptr));  // runs may come in on any stream
+      }
     }
     return MI_OK;
   }
@@ -283,28 +290,12 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
                             DevBuf *c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
-  bool skinny = rows <= kGemvMaxRows && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024);
-  if (skinny && rows > kGemvDotRows && st.w_blocked.p == nullptr) {
-    // the blocked copy needs an allocation and a wait, neither of which a stream under graph capture allows: such
-    // a call takes the GEMM path (same results), and the copy is built by the first call outside a capture
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) skinny = false;
-  }
+  // up to 2 rows: the dot kernel on the row-major weights; 3..32 rows: the matrix-core decode kernel on the blocked
+  // copy made at create time -- a handle created without it runs those row counts on the GEMM tiles
+  const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
+                                           : rows <= kGemvMaxRows && st.w_blocked.p != nullptr;
   if (skinny) {
-    if (rows > kGemvDotRows) {
-      if (st.w_blocked.p == nullptr) {
-        int rc = st.w_blocked.ensure((size_t)st.n_pad * st.k_pad);
-        if (rc != MI_OK) return rc;
-        rc = launch_block_weights(w.w, st.n_pad, st.k_pad, st.ldw, static_cast<int8_t *>(st.w_blocked.p), stream);
-        if (rc != MI_OK) {
-          st.w_blocked.release();
-          return rc;
-        }
-        // one-time: later runs may come in on other streams and must find the copy complete
-        MI_HIP_CHECK(hipStreamSynchronize(stream));
-      }
-      w.blocked = static_cast<const int8_t *>(st.w_blocked.p);
-    }
+    if (rows > kGemvDotRows) w.blocked = static_cast<const int8_t *>(st.w_blocked.p);
     return launch_gemv_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
   }
   if ((st.n & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 3) == 0)
@@ -546,6 +537,10 @@ static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_h
     set_error("mi_matmul_create: bad shape/activation deep=%d col=%d act=%d", d->deep, d->col, d->act_type);
     return MI_PARAM_INVALID;
   }
+  if ((d->flags & ~MI_MATMUL_NO_DECODE_PACK) != 0) {
+    set_error("mi_matmul_create: unknown flags 0x%x", d->flags);
+    return MI_PARAM_INVALID;
+  }
   int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
   if (rc != MI_OK) return rc;
   if ((rc = ensure_device()) != MI_OK) return rc;
@@ -554,7 +549,8 @@ static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_h
   if (h == nullptr) return MI_MEMORY_FAILED;
   const std::vector<int8_t> w_nk = to_nk(weight_host, d->col, d->deep, d->b_transpose);
   rc = h->st.build(w_nk.data(), d->col, d->deep, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
-                   d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true);
+                   d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true,
+                   (d->flags & MI_MATMUL_NO_DECODE_PACK) == 0);
   if (rc != MI_OK) {
     return rc;
   }
@@ -564,6 +560,16 @@ static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_h
 
 int mi_matmul_create(const mi_matmul_desc *d, const int8_t *weight_host, const int32_t *bias_host, mi_matmul **out) {
   return guarded("mi_matmul_create", [&] { return mi_matmul_create_impl(d, weight_host, bias_host, out); });
+}
+
+int mi_matmul_reserve(mi_matmul *h, int32_t max_rows) {
+  if (h == nullptr) return MI_NULL_PTR;
+  if (max_rows < 0) return MI_PARAM_INVALID;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  // sized for the worst case of either workspace: whether a run needs them also depends on its pointers
+  if ((rc = h->a_ws.ensure((size_t)max_rows * round_up(h->st.k, 16))) != MI_OK) return rc;
+  return h->c_ws.ensure((size_t)max_rows * round_up(h->st.n, 4));
 }
 
 int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream) {
@@ -742,6 +748,21 @@ int mi_conv_out_shape(const mi_conv *h, int32_t in_h, int32_t in_w, int32_t *out
   *out_h = (in_h + d.pad_u + d.pad_d - eh) / d.stride_h + 1;
   *out_w = (in_w + d.pad_l + d.pad_r - ew) / d.stride_w + 1;
   return MI_OK;
+}
+
+int mi_conv_reserve(mi_conv *h, int32_t batch, int32_t in_h, int32_t in_w) {
+  if (h == nullptr) return MI_NULL_PTR;
+  if (batch < 0) return MI_PARAM_INVALID;
+  int oh = 0, ow = 0;
+  int rc = mi_conv_out_shape(h, in_h, in_w, &oh, &ow);
+  if (rc != MI_OK) return rc;
+  if (h->depthwise || batch == 0) return MI_OK;
+  if ((rc = ensure_device()) != MI_OK) return rc;
+  const size_t pixels = (size_t)batch * oh * ow;
+  // the im2col buffer (or, for a 1x1, the padded copy of the image rows) and the padded output, whether or not this
+  // geometry and the run's pointers end up needing them
+  if ((rc = h->col_ws.ensure(pixels * round_up(h->st.k, 16))) != MI_OK) return rc;
+  return h->c_ws.ensure(pixels * round_up(h->st.n, 4));
 }
 
 int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_dev,
@@ -1007,6 +1028,15 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   if ((rc = launch_gemm_dequant(a, lda, rows, k16, w, n4, dq, static_cast<float *>(h->c_ws.p), n4, s)) != MI_OK)
     return rc;
   return launch_copy_rows(h->c_ws.p, (int64_t)n4 * 4, rows, h->n * 4, c_dev, (int64_t)h->n * 4, s);
+}
+
+int mi_dynmm_reserve(mi_dynmm *h, int32_t max_rows) {
+  if (h == nullptr) return MI_NULL_PTR;
+  if (max_rows < 0) return MI_PARAM_INVALID;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  if ((rc = h->a_ws.ensure((size_t)max_rows * round_up(h->k, 16))) != MI_OK) return rc;
+  return h->c_ws.ensure((size_t)max_rows * round_up(h->n, 4) * sizeof(float));
 }
 
 int mi_dynmm_run(mi_dynmm *h, const int8_t *a_dev, int32_t rows, double in_scale, int32_t in_zp, float *c_dev,

@@ -67,8 +67,8 @@ struct WeightView {
   int ldw;
   // Second copy for the matrix-core decode kernel (3..32 activation rows), or nullptr: the same bytes regrouped into
   // 1 KiB blocks [row / 16][k / 64], the 64 16-byte chunks of a block in the order the lanes of the MFMA operand take
-  // them ([(k % 64) / 16][row % 16]), so that a wave instruction fetches 1 KiB front to back.  Built on the device on
-  // first use (launch_block_weights).
+  // them ([(k % 64) / 16][row % 16]), so that a wave instruction fetches 1 KiB front to back.  Built on the device
+  // when the handle is created (launch_block_weights).
   const int8_t *blocked;
 };
 inline int weight_row_stride(int k_pad) { return (k_pad / 256) % 2 == 0 ? k_pad + 256 : k_pad; }

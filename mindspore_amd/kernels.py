@@ -67,10 +67,13 @@ class _Handle:
 
 
 class MatmulInt8Kernel(_Handle):
-    """Full-quant int8 MatMul: C = requant(A x W^T).  weight is [N, K] when transpose_b else [K, N]; bias int32 [N]."""
+    """Full-quant int8 MatMul: C = requant(A x W^T).  weight is [N, K] when transpose_b else [K, N]; bias int32 [N].
+    decode_pack=False skips the second packed form of the weights (the one runs with 3..32 rows use); such rows then
+    run on the GEMM tiles."""
     _destroy = "mi_matmul_destroy"
 
-    def __init__(self, weight, bias, in_quant, weight_quant, out_quant, transpose_b=True, act=ACT_NONE, device=0):
+    def __init__(self, weight, bias, in_quant, weight_quant, out_quant, transpose_b=True, act=ACT_NONE, device=0,
+                 decode_pack=True):
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)
@@ -86,7 +89,7 @@ class MatmulInt8Kernel(_Handle):
         nq, scales, zps = _quant_arrays(weight_quant)
         d = _lib.MatmulDesc(self.k, self.n, 1 if transpose_b else 0, act, float(in_quant.scale),
                             int(in_quant.zero_point), float(out_quant.scale), int(out_quant.zero_point), nq, scales,
-                            zps)
+                            zps, 0 if decode_pack else _lib.MATMUL_NO_DECODE_PACK)
         _lib.check(L.mi_matmul_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                       C.byref(self._h)), "mi_matmul_create")
 
@@ -113,6 +116,10 @@ class MatmulInt8Kernel(_Handle):
         out = np.empty(a.shape[:-1] + (self.n,), np.int8)
         _lib.check(L.mi_matmul_run_host(self._h, a.ctypes.data, rows, out.ctypes.data), "mi_matmul_run_host")
         return out
+
+    def reserve(self, max_rows):
+        """ReSize(): sizes the workspaces so that runs of up to max_rows rows allocate nothing."""
+        _lib.check(_lib.load().mi_matmul_reserve(self._h, int(max_rows)), "mi_matmul_reserve")
 
     def params(self):
         L = _lib.load()

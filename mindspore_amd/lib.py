@@ -14,11 +14,11 @@ ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
 EXPORTS = [
     "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_quantize_multiplier_single", "mi_activation_range", "mi_requant_params",
     "mi_multiply_by_quantized_multiplier",
-    "mi_matmul_create", "mi_matmul_run", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
-    "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_destroy",
+    "mi_matmul_create", "mi_matmul_reserve", "mi_matmul_run", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
+    "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_reserve", "mi_conv_destroy",
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
     "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
-    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host",
+    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
     "mi_dynmm_destroy",
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
     "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize",
@@ -31,7 +31,10 @@ class MatmulDesc(C.Structure):
     _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
                 ("in_scale", C.c_double), ("in_zp", C.c_int32), ("out_scale", C.c_double), ("out_zp", C.c_int32),
                 ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
-                ("filter_zps", C.POINTER(C.c_int32))]
+                ("filter_zps", C.POINTER(C.c_int32)), ("flags", C.c_int32)]
+
+
+MATMUL_NO_DECODE_PACK = 1
 
 
 class ConvDesc(C.Structure):
@@ -100,6 +103,7 @@ def load():
     L.mi_multiply_by_quantized_multiplier.argtypes = [i32, i32, i32, i32]
     L.mi_multiply_by_quantized_multiplier.restype = i32
     L.mi_matmul_create.argtypes = [C.POINTER(MatmulDesc), vp, vp, C.POINTER(vp)]
+    L.mi_matmul_reserve.argtypes = [vp, i32]
     L.mi_matmul_run.argtypes = [vp, vp, i32, vp, vp]
     L.mi_matmul_run_host.argtypes = [vp, vp, i32, vp]
     L.mi_matmul_get_params.argtypes = [vp, vp, vp, vp, vp, pi32, pi32]
@@ -110,6 +114,7 @@ def load():
     L.mi_conv_same_pad.argtypes = [i32, i32, i32, i32, pi32, pi32, pi32]
     L.mi_conv_run.argtypes = [vp, vp, i32, i32, i32, vp, vp]
     L.mi_conv_run_host.argtypes = [vp, vp, i32, i32, i32, vp]
+    L.mi_conv_reserve.argtypes = [vp, i32, i32, i32]
     L.mi_conv_destroy.argtypes = [vp]
     L.mi_conv_destroy.restype = None
     L.mi_dynquant_create.argtypes = [i32, C.POINTER(vp)]
@@ -128,6 +133,7 @@ def load():
     L.mi_dynmm_run_host.argtypes = [vp, vp, i32, dbl, i32, vp]
     L.mi_dynmm_run_rows.argtypes = [vp, vp, i32, vp, vp, vp]
     L.mi_dynmm_run_rows_host.argtypes = [vp, vp, i32, C.POINTER(dbl), i32, vp]
+    L.mi_dynmm_reserve.argtypes = [vp, i32]
     L.mi_dynmm_destroy.argtypes = [vp]
     L.mi_dynmm_destroy.restype = None
     L.mi_infer_matmul.argtypes = [pi32, i32, pi32, i32, pi32, i32, i32, i32, pi32, pi32]

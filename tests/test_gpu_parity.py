@@ -451,32 +451,37 @@ def test_error_paths():
     assert L.mi_conv_run(conv._h, x.data_ptr(), 1, 5, 5, None, None) == lib.MI_NULL_PTR
 
 def test_first_decode_call_inside_a_graph_capture(orc):
-    """The matrix-core decode kernel wants a blocked copy of the weights that is built on first use (an allocation and
-    a wait).  A first call under stream capture must not do either: it takes the GEMM path, the capture stays valid,
-    every replay is right, and a later eager call builds the copy."""
+    """All weight packing happens at create time, so the very first call of a handle may come under stream capture
+    and runs the decode kernel it would run eagerly: the capture stays valid and every replay is right.  A handle
+    created without the decode pack takes the same row counts on the GEMM tiles, with the same results."""
     import torch
     rng = np.random.default_rng(77)
-    case = _mm_case(rng, 8, 200, 512, True, False, True, 0)
-    kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
-                              QP(case["so"], case["zo"]), True, 0)
-    a = torch.from_numpy(case["a"]).cuda()
-    out = torch.zeros((8, 200), dtype=torch.int8, device="cuda")
-    st = torch.cuda.Stream()
-    with torch.cuda.stream(st):
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=st):
-            kern.run(a, out=out)
-    torch.cuda.synchronize()
-    for rep in range(3):
-        a.copy_(torch.from_numpy(rng.integers(-128, 128, (8, 512), dtype=np.int8)))
-        out.zero_()
+    for k, decode_pack in ((512, True), (512, False), (500, True)):   # 500: the run also pads the activation rows
+        case = _mm_case(rng, 8, 200, k, True, False, True, 0)
+        kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
+                                  QP(case["so"], case["zo"]), True, 0, decode_pack=decode_pack)
+        kern.reserve(8)   # ReSize(): the padded-row workspace exists before the capture
+        a = torch.from_numpy(case["a"]).cuda()
+        out = torch.zeros((8, 200), dtype=torch.int8, device="cuda")
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=st):
+                kern.run(a, out=out)
         torch.cuda.synchronize()
-        g.replay()
-        torch.cuda.synchronize()
-        case["a"] = a.cpu().numpy()
-        want = orc.matmul_int8(**case)
-        assert np.array_equal(out.cpu().numpy(), want), rep
-        assert np.array_equal(kern.run(a).cpu().numpy(), want)   # eager: builds and uses the blocked copy
+        for rep in range(3):
+            a.copy_(torch.from_numpy(rng.integers(-128, 128, (8, k), dtype=np.int8)))
+            out.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            case["a"] = a.cpu().numpy()
+            want = orc.matmul_int8(**case)
+            assert np.array_equal(out.cpu().numpy(), want), (k, decode_pack, rep)
+            assert np.array_equal(kern.run(a).cpu().numpy(), want)
+        for m in (3, 17, 32, 2, 40):   # every decode row class on this handle, eager
+            case["a"] = rng.integers(-128, 128, (m, k), dtype=np.int8)
+            assert np.array_equal(kern.run(case["a"]), orc.matmul_int8(**case)), (k, decode_pack, m)
 
 
 def test_device_memory_entry_points(orc):
