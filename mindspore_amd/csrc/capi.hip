@@ -128,6 +128,38 @@ struct DevBuf {
   }
 };
 
+// Where a run takes temporary device memory from: a buffer of the handle that grows on demand, or a fixed region
+// that is never reallocated.
+struct Workspace {
+  DevBuf *grow = nullptr;  // growable buffer, or
+  void *fixed = nullptr;   // fixed region of `capacity` bytes
+  size_t capacity = 0;
+  static Workspace growable(DevBuf *b) {
+    Workspace w;
+    w.grow = b;
+    return w;
+  }
+  static Workspace region(void *p, size_t bytes) {
+    Workspace w;
+    w.fixed = p;
+    w.capacity = bytes;
+    return w;
+  }
+  int get(size_t want, void **out) const {
+    if (grow != nullptr) {
+      int rc = grow->ensure(want);
+      *out = grow->p;
+      return rc;
+    }
+    if (want > capacity) {
+      set_error("this call needs %zu bytes of scratch memory, %zu are available", want, capacity);
+      return MI_PARAM_INVALID;
+    }
+    *out = fixed;
+    return MI_OK;
+  }
+};
+
 template <typename T>
 static int upload(DevBuf *b, const std::vector<T> &v) {
   int rc = b->ensure(v.size() * sizeof(T) + 16);
@@ -265,8 +297,8 @@ static std::vector<int8_t> to_nk(const int8_t *w, int n, int k, int b_transpose)
 
 // Activations must reach the GEMM/GEMV kernels as 16-byte aligned rows of k16 bytes; returns the pointer/stride to
 // use, copying through `ws` when the caller's layout does not qualify.
-static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_t stream, const int8_t **a_out,
-                        int64_t *lda_out, int *k16_out) {
+static int prepare_rows(const int8_t *a, int rows, int k, const Workspace &ws, hipStream_t stream,
+                        const int8_t **a_out, int64_t *lda_out, int *k16_out) {
   const int k16 = round_up(k, 16);
   if (k16 == k && (reinterpret_cast<uintptr_t>(a) & 15) == 0) {
     *a_out = a;
@@ -274,11 +306,12 @@ static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_
     *k16_out = k;
     return MI_OK;
   }
-  int rc = ws->ensure((size_t)rows * k16);
+  void *buf = nullptr;
+  int rc = ws.get((size_t)rows * k16, &buf);
   if (rc != MI_OK) return rc;
-  rc = launch_pad_rows(a, k, rows, k, static_cast<int8_t *>(ws->p), k16, stream);
+  rc = launch_pad_rows(a, k, rows, k, static_cast<int8_t *>(buf), k16, stream);
   if (rc != MI_OK) return rc;
-  *a_out = static_cast<const int8_t *>(ws->p);
+  *a_out = static_cast<const int8_t *>(buf);
   *lda_out = k16;
   *k16_out = k16;
   return MI_OK;
@@ -287,7 +320,7 @@ static int prepare_rows(const int8_t *a, int rows, int k, DevBuf *ws, hipStream_
 // The GEMM kernels write rows with vector stores; when the caller's row length or base address does not allow that,
 // they write to a padded scratch output which is then compacted into the caller's tensor.
 static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int rows, int k16, int8_t *c,
-                            DevBuf *c_ws, hipStream_t stream) {
+                            const Workspace &c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
   // up to 2 rows: the dot kernel on the row-major weights; 3..32 rows: the matrix-core decode kernel on the blocked
@@ -301,12 +334,12 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
   if ((st.n & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 3) == 0)
     return launch_gemm_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
   const int n4 = round_up(st.n, 4);
-  int rc = c_ws->ensure((size_t)rows * n4);
+  void *buf = nullptr;
+  int rc = c_ws.get((size_t)rows * n4, &buf);
   if (rc != MI_OK) return rc;
-  RequantParams rq_pad = rq;
-  rc = launch_gemm_requant(a, lda, rows, k16, w, n4, rq_pad, static_cast<int8_t *>(c_ws->p), n4, stream);
+  rc = launch_gemm_requant(a, lda, rows, k16, w, n4, rq, static_cast<int8_t *>(buf), n4, stream);
   if (rc != MI_OK) return rc;
-  return launch_copy_rows(c_ws->p, n4, rows, st.n, c, st.n, stream);
+  return launch_copy_rows(buf, n4, rows, st.n, c, st.n, stream);
 }
 
 }  // namespace mi
@@ -373,6 +406,8 @@ int mi_init(int device) {
     return MI_NOT_SUPPORT;
   }
   MI_HIP_CHECK(hipSetDevice(device));
+  int rc = gemv_prepare_device();
+  if (rc != MI_OK) return rc;
   g_device = device;
   return MI_OK;
 }
@@ -588,8 +623,8 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
   const int8_t *a = nullptr;
   int64_t lda = 0;
   int k16 = 0;
-  if ((rc = prepare_rows(a_dev, rows, h->st.k, &h->a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
-  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, &h->c_ws, s);
+  if ((rc = prepare_rows(a_dev, rows, h->st.k, Workspace::growable(&h->a_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
+  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, Workspace::growable(&h->c_ws), s);
 }
 
 int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host) {
@@ -797,7 +832,7 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
   int64_t lda = 0;
   int k16 = 0;
   if (h->direct_1x1) {
-    if ((rc = prepare_rows(in_dev, (int)pixels, k, &h->col_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+    if ((rc = prepare_rows(in_dev, (int)pixels, k, Workspace::growable(&h->col_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
   } else if (k <= 64 && d.out_channel <= 128 && (d.out_channel & 3) == 0 &&
              (reinterpret_cast<uintptr_t>(out_dev) & 3) == 0) {
     // a first-layer convolution: gathered straight from the image, no im2col buffer
@@ -814,7 +849,7 @@ int mi_conv_run(mi_conv *h, const int8_t *in_dev, int32_t batch, int32_t in_h, i
     a = static_cast<const int8_t *>(h->col_ws.p);
     lda = k16;
   }
-  return run_requant_gemm(h->st, a, lda, (int)pixels, k16, out_dev, &h->c_ws, s);
+  return run_requant_gemm(h->st, a, lda, (int)pixels, k16, out_dev, Workspace::growable(&h->c_ws), s);
 }
 
 int mi_conv_run_host(mi_conv *h, const int8_t *in_host, int32_t batch, int32_t in_h, int32_t in_w, int8_t *out_host) {
@@ -1008,7 +1043,7 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   const int8_t *a = nullptr;
   int64_t lda = 0;
   int k16 = 0;
-  if ((rc = prepare_rows(a_dev, rows, h->k, &h->a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  if ((rc = prepare_rows(a_dev, rows, h->k, Workspace::growable(&h->a_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
   DequantParams dq;
   dq.wscale = static_cast<const float *>(h->wscale.p);
   dq.bias = h->has_bias ? static_cast<const float *>(h->bias.p) : nullptr;

@@ -87,6 +87,9 @@ constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel (activations st
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
 
+// Per-device set-up of the skinny-M kernels (function attributes); called by mi_init with the device current.
+int gemv_prepare_device();
+
 // Regroups packed row-major weights into the blocked copy described at WeightView::blocked.
 int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t *blocked, hipStream_t stream);
 

@@ -195,19 +195,30 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
 template <int M, int R, int D, bool DIRECT>
 static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
   auto kern = gemv_i8_kernel<M, R, D, DIRECT>;
+  // (more than 64 KiB of dynamic LDS needs the attribute that gemv_prepare_device set when the library was initialised)
   const int lds_bytes = DIRECT ? 0 : M * ((g.kchunks + 63) / 64) * 1024;
-  if (lds_bytes > 64 * 1024) {
-    static bool attr_set = false;
-    if (!attr_set) {
-      MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      attr_set = true;
-    }
-  }
   const int rows_per_block = 4 * R;
   const int blocks = (g.n + rows_per_block - 1) / rows_per_block;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds_bytes, stream, g, rq);
   MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <int M, int R, int D>
+static int allow_big_lds() {
+  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_kernel<M, R, D, false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  return MI_OK;
+}
+
+// Once per device, from mi_init: the kernels that stage long activation rows in LDS may ask for up to 160 KiB.
+int gemv_prepare_device() {
+  int rc;
+  if ((rc = allow_big_lds<1, 4, 4>()) != MI_OK || (rc = allow_big_lds<1, 4, 8>()) != MI_OK ||
+      (rc = allow_big_lds<1, 2, 8>()) != MI_OK || (rc = allow_big_lds<1, 1, 12>()) != MI_OK ||
+      (rc = allow_big_lds<2, 4, 4>()) != MI_OK || (rc = allow_big_lds<2, 4, 8>()) != MI_OK ||
+      (rc = allow_big_lds<2, 2, 8>()) != MI_OK || (rc = allow_big_lds<2, 1, 12>()) != MI_OK)
+    return rc;
   return MI_OK;
 }
 
