@@ -118,6 +118,17 @@ int mi_matmul_create(const mi_matmul_desc *desc, const int8_t *weight_host, cons
 int mi_matmul_reserve(mi_matmul *h, int32_t max_rows);
 /* a_dev: int8 [rows, deep]; c_dev: int8 [rows, col].  Asynchronous on `stream`. */
 int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
+/* mi_matmul_run for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same results; instead of the
+ * handle's growable workspaces it uses one scratch area of MI_NOALLOC_SCRATCH_BYTES of static device memory (held by
+ * every GPU the library is initialised on until the process ends) and calls neither hipMalloc nor hipFree nor any
+ * allocating routine.  Scratch is needed only for operands the kernels cannot take in place: rows x round_up(deep,
+ * 16) bytes when deep % 16 != 0 or a_dev is not 16-byte aligned, plus rows x round_up(col, 4) bytes when col % 4 != 0
+ * or c_dev is not 4-byte aligned; a call that needs more than the maximum returns MI_PARAM_INVALID and launches
+ * nothing.  All handles on a GPU share the scratch area: calls of this entry point that overlap in time on one
+ * GPU (different streams or threads) race on it; calls ordered on one stream do not. */
+#define MI_NOALLOC_SCRATCH_BYTES (8u << 20)
+int mi_matmul_run_noalloc(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
 /* Same with host tensors: copies in, runs, copies out, synchronises. */
 int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host);
 /* Derived per-channel parameters (arrays of `col` entries, any may be NULL): multiplier / shifts, the folded bias

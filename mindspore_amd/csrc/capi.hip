@@ -20,6 +20,14 @@ namespace mi {
 static thread_local char g_err[512] = "";
 static int g_device = -1;
 
+// Scratch memory of mi_matmul_run_noalloc: static device memory, so the entry point never allocates.  Every GPU the
+// library is initialised on holds its own copy of the array at its own address; the array's name is only a host-side
+// stand-in, so host code uses the per-device address that mi_init looked up (g_scratch_ptr), never the name.
+constexpr size_t kScratchBytes = MI_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices] = {};
+
 void set_error(const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -408,6 +416,11 @@ int mi_init(int device) {
   MI_HIP_CHECK(hipSetDevice(device));
   int rc = gemv_prepare_device();
   if (rc != MI_OK) return rc;
+  if (device < kMaxDevices && g_scratch_ptr[device] == nullptr) {
+    void *ptr = nullptr;
+    MI_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));  // this device's copy of the array
+    g_scratch_ptr[device] = ptr;
+  }
   g_device = device;
   return MI_OK;
 }
@@ -625,6 +638,47 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
   int k16 = 0;
   if ((rc = prepare_rows(a_dev, rows, h->st.k, Workspace::growable(&h->a_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
   return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, Workspace::growable(&h->c_ws), s);
+}
+
+int mi_matmul_run_noalloc(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream) {
+  if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
+    set_error("mi_matmul_run_noalloc: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0) {
+    set_error("mi_matmul_run_noalloc: rows=%d", rows);
+    return MI_PARAM_INVALID;
+  }
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  void *base = g_device < kMaxDevices ? g_scratch_ptr[g_device] : nullptr;
+  if (base == nullptr) {
+    set_error("mi_matmul_run_noalloc: no scratch memory on device %d", g_device);
+    return MI_ERROR;
+  }
+  // the padded activation rows first, the padded output behind them; a part is only used when the operand's shape
+  // or address needs it, but the size check does not depend on the pointers of this particular call
+  const size_t a_bytes = round_up64((int64_t)rows * round_up(h->st.k, 16), 256);
+  const size_t c_bytes = (size_t)rows * round_up(h->st.n, 4);
+  const bool a_padded = (h->st.k & 15) != 0, c_padded = (h->st.n & 3) != 0;
+  const bool a_unaligned = (reinterpret_cast<uintptr_t>(a_dev) & 15) != 0;
+  const bool c_unaligned = (reinterpret_cast<uintptr_t>(c_dev) & 3) != 0;
+  const size_t need = ((a_padded || a_unaligned) ? a_bytes : 0) + ((c_padded || c_unaligned) ? c_bytes : 0);
+  if (need > kScratchBytes) {
+    set_error("mi_matmul_run_noalloc: %d rows of this MatMul (deep %d, col %d) need %zu bytes of scratch memory, the "
+              "maximum is %zu; use mi_matmul_run", rows, h->st.k, h->st.n, need, kScratchBytes);
+    return MI_PARAM_INVALID;
+  }
+  unsigned char *p = static_cast<unsigned char *>(base);
+  const Workspace a_ws = Workspace::region(p, a_bytes);
+  const Workspace c_ws = Workspace::region(p + ((a_padded || a_unaligned) ? a_bytes : 0), c_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  if ((rc = prepare_rows(a_dev, rows, h->st.k, a_ws, s, &a, &lda, &k16)) != MI_OK) return rc;
+  return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, c_ws, s);
 }
 
 int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host) {
