@@ -103,7 +103,7 @@ def bench_hbm_read(steps, warmup):
     it is read again."""
     import torch
     from mindspore_amd import lib
-    L = lib.load()
+    L = lib.load_diag()
     slice_bytes, n_slices = 48 << 20, 64
     buf = torch.ones(slice_bytes * n_slices, dtype=torch.int8, device="cuda")
     state = {"i": 0}
@@ -121,7 +121,7 @@ def bench_mfma_rate():
     import numpy as np
     import torch
     from mindspore_amd import lib
-    L = lib.load()
+    L = lib.load_diag()
     clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
     out = {}
     iters, wgs = 40000, 256
@@ -472,7 +472,7 @@ def main():
                      "kernel": "mi::gemm_direct_kernel<256, 256, 0, false, true, 4, 1>", "ops_per_launch": g["ops"]},
     }
     if args.calibrate:
-        L = lib.load()
+        L = lib.load_diag()
         src = torch.ones(256 << 20, dtype=torch.int8, device="cuda")
         dst = torch.empty_like(src)
         for _ in range(3):

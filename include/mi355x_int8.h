@@ -317,19 +317,6 @@ int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *s
 int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream);
 int mi_stream_synchronize(void *stream);
 
-/* ---- measurement aids (no counterpart in the reference) ---------------------------------------------------------
- * Two plain HBM movers with a known byte count and a matrix-pipe exerciser, used by the benchmark: the read stream gives the bandwidth a
- * kernel that only reads (the decode GEMV) can reach on this device, the copy calibrates the profiler's
- * FETCH_SIZE / WRITE_SIZE counters.  bytes must be a multiple of 16, pointers 16-byte aligned. */
-int mi_diag_stream_read(const void *src_dev, int64_t bytes, void *stream);
-int mi_diag_copy(void *dst_dev, const void *src_dev, int64_t bytes, void *stream);
-/* The matrix pipe alone: `workgroups` x 4 waves each issue iters x 16 v_mfma_i32_32x32x32_i8 (65536 ops each) on
- * register operands read once from operands_dev (32 KiB).  The sustained shader clock, and with it the rate,
- * depends on the operand data (bit toggling -> power), so the benchmark passes bytes drawn like the GEMM's.
- * clocks_dev[0] = shader cycles, clocks_dev[1] = 100 MHz ticks spent in the loop (device memory, 16 bytes). */
-int mi_diag_mfma_rate(const void *operands_dev, int32_t iters, int32_t workgroups, uint64_t *clocks_dev,
-                      void *stream);
-
 #ifdef __cplusplus
 }
 #endif

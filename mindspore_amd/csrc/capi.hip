@@ -498,35 +498,6 @@ int mi_stream_synchronize(void *stream) {
   return MI_OK;
 }
 
-int mi_diag_stream_read(const void *src_dev, int64_t bytes, void *stream) {
-  if (src_dev == nullptr) return MI_NULL_PTR;
-  if (bytes <= 0 || (bytes & 15) != 0 || (reinterpret_cast<uintptr_t>(src_dev) & 15) != 0) {
-    set_error("mi_diag_stream_read: bytes and pointer must be multiples of 16");
-    return MI_PARAM_INVALID;
-  }
-  return launch_stream_read(src_dev, bytes, static_cast<hipStream_t>(stream));
-}
-
-int mi_diag_copy(void *dst_dev, const void *src_dev, int64_t bytes, void *stream) {
-  if (src_dev == nullptr || dst_dev == nullptr) return MI_NULL_PTR;
-  if (bytes <= 0 || (bytes & 15) != 0 || ((reinterpret_cast<uintptr_t>(src_dev) | reinterpret_cast<uintptr_t>(dst_dev)) & 15) != 0) {
-    set_error("mi_diag_copy: bytes and pointers must be multiples of 16");
-    return MI_PARAM_INVALID;
-  }
-  return launch_copy16(dst_dev, src_dev, bytes, static_cast<hipStream_t>(stream));
-}
-
-int mi_diag_mfma_rate(const void *operands_dev, int32_t iters, int32_t workgroups, uint64_t *clocks_dev,
-                      void *stream) {
-  if (operands_dev == nullptr || clocks_dev == nullptr) return MI_NULL_PTR;
-  if (iters <= 0 || workgroups <= 0 || workgroups > 65536 || (reinterpret_cast<uintptr_t>(operands_dev) & 15) != 0) {
-    set_error("mi_diag_mfma_rate: bad iteration / workgroup count or unaligned operands");
-    return MI_PARAM_INVALID;
-  }
-  return launch_mfma_rate(operands_dev, iters, workgroups, reinterpret_cast<unsigned long long *>(clocks_dev),
-                          static_cast<hipStream_t>(stream));
-}
-
 const char *mi_last_error(void) { return g_err; }
 const char *mi_version(void) { return "mi355x_int8 0.1 (gfx950)"; }
 

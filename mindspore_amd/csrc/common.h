@@ -122,15 +122,6 @@ bool gemm_conv_supported(const ConvGeom &g, const void *in, const void *out);
 int launch_gemm_conv_requant(const int8_t *in, const ConvGeom &g, const int8_t *fill16, const WeightView &w,
                              const RequantParams &rq, int8_t *out, hipStream_t stream);
 
-// Measurement aids: read `bytes` and discard them / copy them, 16 bytes per lane.
-int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream);
-int launch_copy16(void *dst, const void *src, int64_t bytes, hipStream_t stream);
-
-// Measurement aid: `iters` x 16 v_mfma_i32_32x32x32_i8 per wave on the given operand bytes (32 KiB), 4 waves per
-// workgroup; clocks[0..1] (device memory) receive shader cycles and 100 MHz ticks of the loop.
-int launch_mfma_rate(const void *operands, int iters, int workgroups, unsigned long long *clocks,
-                     hipStream_t stream);
-
 // DynamicQuant: per-block min/max partials, then quantise (every block re-reduces the partials).
 constexpr int kDqMaxBlocks = 1024;
 int launch_dynquant(const float *x, int64_t n, int symmetric, float2 *partials, mi_dq_params *params, int8_t *q,

@@ -71,51 +71,6 @@ int launch_copy_rows(const void *src, int64_t src_ld, int rows, int row_bytes, v
   return MI_OK;
 }
 
-// Reads 8 KiB per wave (8 x 16 bytes per lane, all requested before the first use) and keeps nothing: the shape
-// of the decode GEMV's weight stream without its arithmetic.
-__global__ __launch_bounds__(256) void stream_read_kernel(const v4i *__restrict__ src, int64_t chunks,
-                                                          int *__restrict__ sink) {
-  const int lane = threadIdx.x & 63;
-  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  v4i buf[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int64_t c = wave * 512 + i * 64 + lane;
-    c = c < chunks ? c : chunks - 1;
-    buf[i] = __builtin_nontemporal_load(src + c);  // as the decode kernels read their weights
-  }
-  int s = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s += buf[i].x ^ buf[i].y ^ buf[i].z ^ buf[i].w;
-  if (s == 0x5ca1ab1e && sink != nullptr) sink[0] = s;  // never true for the benchmark's data; keeps the loads alive
-}
-
-int launch_stream_read(const void *src, int64_t bytes, hipStream_t stream) {
-  const int64_t chunks = bytes / 16;
-  const int64_t blocks = (chunks + 2047) / 2048;
-  if (chunks <= 0 || blocks > 0x7fffffff) return MI_PARAM_INVALID;
-  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, static_cast<const v4i *>(src),
-                     chunks, static_cast<int *>(nullptr));
-  MI_HIP_CHECK(hipGetLastError());
-  return MI_OK;
-}
-
-__global__ __launch_bounds__(256) void copy16_kernel(const v4i *__restrict__ src, v4i *__restrict__ dst,
-                                                     int64_t chunks) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < chunks; i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = src[i];
-}
-
-int launch_copy16(void *dst, const void *src, int64_t bytes, hipStream_t stream) {
-  const int64_t chunks = bytes / 16;
-  if (chunks <= 0) return MI_PARAM_INVALID;
-  const int64_t want = (chunks + 255) / 256;
-  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)(want > 65536 ? 65536 : want)), dim3(256), 0, stream,
-                     static_cast<const v4i *>(src), static_cast<v4i *>(dst), chunks);
-  MI_HIP_CHECK(hipGetLastError());
-  return MI_OK;
-}
-
 __global__ __launch_bounds__(256) void im2col_kernel(const int8_t *__restrict__ in, ConvGeom g, int fill,
                                                      int8_t *__restrict__ dst, int k16) {
   const int kdim = g.kernel_h * g.kernel_w * g.in_c;

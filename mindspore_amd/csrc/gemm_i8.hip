@@ -870,49 +870,4 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
             : launch_pick_tile<EPI_DEQUANT, false, false>(g, rq, dq, stream);
 }
 
-// Measurement aid: nothing but back-to-back MFMAs on register operands taken from `operands` (256 threads x 8 x 16
-// bytes), one workgroup per CU, one wave per SIMD -- the rate the matrix pipe sustains for THAT operand data.  The
-// sustained shader clock depends on how many operand bits toggle, so the caller passes data like the GEMM's.
-// clocks[0] = shader cycles, clocks[1] = 100 MHz ticks spent in the loop by workgroup 0.
-__global__ __launch_bounds__(256) void mfma_rate_kernel(const v4i *__restrict__ operands, int iters,
-                                                        unsigned long long *__restrict__ clocks,
-                                                        int *__restrict__ sink) {
-  v16i acc[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) acc[i][e] = 0;
-  v4i fa[4], fb[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    fa[i] = operands[threadIdx.x * 8 + i];
-    fb[i] = operands[threadIdx.x * 8 + 4 + i];
-  }
-  const unsigned long long c0 = clock64(), w0 = wall_clock64();
-  for (int it = 0; it < iters; ++it) {
-#pragma unroll
-    for (int i = 0; i < 16; ++i)
-      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i & 3], fb[i >> 2], acc[i], 0, 0, 0);
-  }
-  const unsigned long long c1 = clock64(), w1 = wall_clock64();
-  int t = 0;
-#pragma unroll
-  for (int i = 0; i < 16; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) t += acc[i][e];
-  if (t == 0x5ca1ab1e && iters < 0) sink[0] = t;  // never true; keeps the accumulators alive
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    clocks[0] = c1 - c0;
-    clocks[1] = w1 - w0;
-  }
-}
-
-int launch_mfma_rate(const void *operands, int iters, int workgroups, unsigned long long *clocks,
-                     hipStream_t stream) {
-  hipLaunchKernelGGL(mfma_rate_kernel, dim3(workgroups), dim3(256), 0, stream, static_cast<const v4i *>(operands),
-                     iters, clocks, static_cast<int *>(nullptr));
-  MI_HIP_CHECK(hipGetLastError());
-  return MI_OK;
-}
-
 }  // namespace mi

@@ -14,6 +14,7 @@
 #include <cstring>
 #include <vector>
 
+#include "../../include/mi355x_diag.h"
 #include "../../include/mi355x_int8.h"
 
 #define CHECK_HIP(x)                                                          \

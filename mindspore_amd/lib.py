@@ -23,8 +23,10 @@ EXPORTS = [
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
     "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize",
     "mi_host_malloc", "mi_host_free",
-    "mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate",
 ]
+# libmi355x_diag.so (include/mi355x_diag.h): the benchmark's measurement aids, not part of the product library
+DIAG_LIB_PATH = os.path.join(HERE, "libmi355x_diag.so")
+DIAG_EXPORTS = ["mi_diag_stream_read", "mi_diag_copy", "mi_diag_mfma_rate"]
 
 
 class MatmulDesc(C.Structure):
@@ -147,11 +149,28 @@ def load():
     L.mi_copy_to_device.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_copy_to_host.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_stream_synchronize.argtypes = [vp]
-    L.mi_diag_stream_read.argtypes = [vp, i64, vp]
-    L.mi_diag_copy.argtypes = [vp, vp, i64, vp]
-    L.mi_diag_mfma_rate.argtypes = [vp, i32, i32, vp, vp]
     _lib = L
     return L
+
+
+_diag = None
+
+
+def load_diag():
+    """Loads the benchmark's measurement aids (libmi355x_diag.so)."""
+    global _diag
+    if _diag is not None:
+        return _diag
+    load()  # settles which HIP runtime the process holds
+    if not os.path.exists(DIAG_LIB_PATH):
+        raise RuntimeError("%s is not built: run `python -m mindspore_amd.build`" % DIAG_LIB_PATH)
+    D = C.CDLL(DIAG_LIB_PATH)
+    vp, i32, i64 = C.c_void_p, C.c_int32, C.c_int64
+    D.mi_diag_stream_read.argtypes = [vp, i64, vp]
+    D.mi_diag_copy.argtypes = [vp, vp, i64, vp]
+    D.mi_diag_mfma_rate.argtypes = [vp, i32, i32, vp, vp]
+    _diag = D
+    return D
 
 
 def check(code, what):

@@ -31,6 +31,20 @@ def test_exports_match_header(L):
     assert b"gfx950" in L.mi_version()
 
 
+def test_measurement_aids_live_in_their_own_library(L):
+    """The benchmark's probes are declared in include/mi355x_diag.h and built into libmi355x_diag.so: the header an
+    integrator reads and the product library carry none of them."""
+    header = open(os.path.join(ROOT, "include", "mi355x_diag.h")).read()
+    declared = set(re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(lib.DIAG_EXPORTS), declared ^ set(lib.DIAG_EXPORTS)
+    D = lib.load_diag()
+    for name in declared:
+        assert hasattr(D, name) and not hasattr(L, name), name
+    assert D.mi_diag_stream_read(None, 16, None) == lib.MI_NULL_PTR
+    assert D.mi_diag_copy(None, None, 16, None) == lib.MI_NULL_PTR
+    assert D.mi_diag_mfma_rate(None, 1, 1, None, None) == lib.MI_NULL_PTR
+
+
 def test_quantize_multiplier_matches_oracle(L, orc):
     rnd = random.Random(11)
     vals = [0.0, 1.0, 0.5, 0.9999999999999999, 1e-9, 123.0, -0.3, 5e-324, float("inf"), float("nan")]
@@ -103,9 +117,6 @@ def test_device_entry_points_fail_cleanly_without_init(L):
     assert L.mi_dynquant_run_segments_host(None, None, 4, 4, None, None) == lib.MI_NULL_PTR
     assert L.mi_dynmm_run_rows(None, None, 1, None, None, None) == lib.MI_NULL_PTR
     assert L.mi_dynmm_run_rows_host(None, None, 1, None, 0, None) == lib.MI_NULL_PTR
-    assert L.mi_diag_stream_read(None, 16, None) == lib.MI_NULL_PTR
-    assert L.mi_diag_copy(None, None, 16, None) == lib.MI_NULL_PTR
-    assert L.mi_diag_mfma_rate(None, 1, 1, None, None) == lib.MI_NULL_PTR
     assert L.mi_device_malloc(64, None) == lib.MI_NULL_PTR
     assert L.mi_copy_to_device(None, None, 8, None) == lib.MI_NULL_PTR
     assert L.mi_copy_to_host(None, None, 8, None) == lib.MI_NULL_PTR
