@@ -22,10 +22,38 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA peak, TOP/s (5.0 POP/s)
 PEAK_HBM_GBPS = 8000.0   # MI355X HBM3E peak, GB/s
 
-# HBM-side bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
-# this script, each scaled by what the same counter reads for the 256 MiB copy of --calibrate (FETCH_SIZE x 2.000,
-# WRITE_SIZE x 1.000; summary in profiles/gemm_direct_kernel_gemm4096.txt): (99337 + 16640) KiB.  None = not measured.
-MEASURED_TRAFFIC_BYTES = {"gemm4096": (99337 + 16640) * 1024, "gemm8192": None}
+HEADLINE_KERNEL = "mi::gemm_kblock_kernel<0, false, true>"
+# HBM-side bytes per launch of the dominant kernel come from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` runs of
+# this script, each scaled by what the same counter reads for the 256 MiB copy of --calibrate.  The figures are read
+# from the committed summary of those runs, which also names the kernel and the commit it was measured at, so that
+# a number that no longer belongs to the current kernel shows.
+TRAFFIC_SUMMARY = {"gemm4096": os.path.join(ROOT, "profiles", "gemm_kblock_kernel_gemm4096.txt"), "gemm8192": None}
+
+
+def measured_traffic(workload):
+    """{bytes, kernel, commit} from the `key: value` lines of the profile summary, or None."""
+    path = TRAFFIC_SUMMARY.get(workload)
+    if not path or not os.path.exists(path):
+        return None
+    kv = {}
+    for line in open(path):
+        key, sep, val = line.partition(":")
+        if sep and key.strip() in ("traffic_bytes_per_launch", "kernel", "measured_at_commit"):
+            kv[key.strip()] = val.strip()
+    if "traffic_bytes_per_launch" not in kv:
+        return None
+    return dict(bytes=int(kv["traffic_bytes_per_launch"]), kernel=kv.get("kernel"), commit=kv.get("measured_at_commit"))
+
+
+def host_cores():
+    """Threads the CPU baseline runs on: every core this process may use; a thread-count limit the environment sets
+    (OMP_NUM_THREADS, the box's CPU share) is respected.  Returns (threads used, what nproc reports)."""
+    nproc = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    used = nproc
+    limit = os.environ.get("OMP_NUM_THREADS", "")
+    if limit.isdigit() and int(limit) > 0:
+        used = min(used, int(limit))
+    return used, nproc
 
 
 def time_steps(fn, steps, warmup):
@@ -68,7 +96,36 @@ def make_matmul(c):
                               True, c["act"])
 
 
-def bench_gemm(size, steps, warmup, host_path=False):
+def bench_sustained(kern, a, out, size, launches=400):
+    """The same GEMM launched back to back for at least 20 ms: under this load the power management lowers the shader
+    clock within a few milliseconds, so the figure of a short timed region is a burst figure.  The shader clock is
+    read by a 0.3 ms matrix-pipe loop (in-kernel cycle counter against the 100 MHz counter) queued right behind the
+    last launch, on operands drawn like the GEMM's."""
+    import numpy as np
+    import torch
+    from mindspore_amd import lib
+    D = lib.load_diag()
+    ops_t = torch.from_numpy(np.random.default_rng(0).integers(-128, 128, 32768, dtype=np.int8)).cuda()
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    for _ in range(5):
+        kern.run(a, out=out)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(launches):
+        kern.run(a, out=out)
+    stop.record()
+    lib.check(D.mi_diag_mfma_rate(ops_t.data_ptr(), 1024, 256, clocks.data_ptr(), _stream()), "mi_diag_mfma_rate")
+    torch.cuda.synchronize()
+    total_ms = start.elapsed_time(stop)
+    ms = total_ms / launches
+    c = clocks.cpu().numpy()
+    tops = 2.0 * size ** 3 / (ms * 1e-3) / 1e12
+    return dict(launches=launches, total_ms=total_ms, ms_per_launch=ms, tops=tops, frac_of_int8_peak=tops / PEAK_INT8_TOPS,
+                shader_clock_ghz_right_after=float(c[0]) / (float(c[1]) * 10.0))
+
+
+def bench_gemm(size, steps, warmup, host_path=False, sustained=False):
     import torch
     from mindspore_amd import workloads as wl
     c = wl.gemm_c5(size)
@@ -82,6 +139,8 @@ def bench_gemm(size, steps, warmup, host_path=False):
     ev_ms, host_ms = time_steps(lambda: kern.run(a, out=out), steps, warmup)
     ops = 2.0 * size * size * size
     res = dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c, prepare_ms=prepare_ms)
+    if sustained:
+        res["sustained"] = bench_sustained(kern, a, out, size)
     if host_path:
         # the boundary as the provider uses it today: host tensors in and out (pinned staging + PCIe both ways)
         kern.run(c["a"])
@@ -296,7 +355,7 @@ def cpu_baseline(case, size):
     not travel -- on a bounded sample: the first `rows` activation rows of the same GEMM on all host cores (about 20
     core-seconds), and the first 64 rows on one thread."""
     from oracle import pyoracle
-    cores = min(16, os.cpu_count() or 1)
+    cores, nproc = host_cores()
     if pyoracle.Reference.available():
         eng, kind = pyoracle.reference(), "reference"
     else:
@@ -319,7 +378,7 @@ def cpu_baseline(case, size):
     rows = 1024 if size <= 4096 else 256
     tops, secs = run(rows, cores)
     tops1, secs1 = run(64 if size <= 4096 else 16, 1)
-    return dict(value=tops, unit="TOP/s", cores=cores, kind=kind, seconds=secs,
+    return dict(value=tops, unit="TOP/s", cores=cores, nproc=nproc, kind=kind, seconds=secs,
                 sample="first %d of %d activation rows of the same %d^3 GEMM (A-pack + row sums + MatmulInt8Opt "
                        "column stripes on %d threads)" % (rows, size, size, cores),
                 single_thread=dict(value=tops1, unit="TOP/s", cores=1, seconds=secs1,
@@ -332,7 +391,7 @@ def cpu_side_by_side():
     first 256 rows, configuration 1, and the four layers of configuration 2."""
     from oracle import pyoracle
     from mindspore_amd import workloads as wl
-    cores = min(16, os.cpu_count() or 1)
+    cores, _ = host_cores()
     if pyoracle.Reference.available():
         eng, kind = pyoracle.reference(), "reference"
         eng.threads = cores
@@ -409,8 +468,10 @@ def main():
     lib.init(0)  # raises if the HIP library is missing or the GPU is not gfx950
 
     size = 4096 if args.workload == "gemm4096" else 8192
-    g = bench_gemm(size, args.steps, args.warmup, host_path=not args.no_extra)
+    g = bench_gemm(size, args.steps, args.warmup, host_path=not args.no_extra, sustained=not args.no_extra)
     extra = {}
+    if "sustained" in g:
+        extra["gemm%d_sustained" % size] = g["sustained"]
 
     def section(name, fn):
         """An extra must never cost the headline line: a failure is recorded under its name."""
@@ -468,9 +529,15 @@ def main():
         "config": {"workload": "config 5: int8 GEMM M=N=K=%d, per-channel requant to int8 (fused epilogue), zx=7, "
                                "int32 bias" % size},
         "roofline": {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                     "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
-                     "kernel": "mi::gemm_direct_kernel<256, 256, 0, false, true, 4, 1>", "ops_per_launch": g["ops"]},
+                     "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": None,
+                     "kernel": HEADLINE_KERNEL, "ops_per_launch": g["ops"]},
     }
+    tr = measured_traffic(args.workload)
+    if tr:
+        result["roofline"]["traffic"] = tr["bytes"]
+        result["roofline"]["traffic_measured_at_commit"] = tr["commit"]
+        result["roofline"]["traffic_measured_on_kernel"] = tr["kernel"]
+        result["roofline"]["traffic_is_for_this_kernel"] = tr["kernel"] == HEADLINE_KERNEL
     if args.calibrate:
         L = lib.load_diag()
         src = torch.ones(256 << 20, dtype=torch.int8, device="cuda")

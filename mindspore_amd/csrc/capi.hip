@@ -180,13 +180,14 @@ static int upload(DevBuf *b, const std::vector<T> &v) {
 struct RequantState {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
+  DevBuf mult2, c2lo, c2hi, pre;  // the GEMM epilogue's per-channel constants (RequantParams::fast2)
   DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (3..32 activation rows); built in create or absent
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
-  bool has_zw = false, fast = false;
+  bool has_zw = false, fast = false, fast2 = false;
 
   RequantParams params() const {
-    RequantParams rq;
+    RequantParams rq{};
     rq.mult = static_cast<const int32_t *>(mult.p);
     rq.bias2 = static_cast<const int32_t *>(bias2.p);
     rq.rshift = static_cast<const int32_t *>(rshift.p);
@@ -197,6 +198,11 @@ struct RequantState {
     rq.amax = amax;
     rq.has_zw = has_zw ? 1 : 0;
     rq.fast = fast ? 1 : 0;
+    rq.mult2 = static_cast<const uint32_t *>(mult2.p);
+    rq.c2lo = static_cast<const uint32_t *>(c2lo.p);
+    rq.c2hi = static_cast<const uint32_t *>(c2hi.p);
+    rq.pre = static_cast<const int32_t *>(pre.p);
+    rq.fast2 = fast2 ? 1 : 0;
     return rq;
   }
 
@@ -245,7 +251,27 @@ struct RequantState {
     }
     for (int c = n; c < n_pad; ++c) e[c] = 1;
     if (amin > amax) fast = false;
+    // constants of the GEMM's single-multiply rounding form (RequantParams::fast2)
+    fast2 = fast;
+    std::vector<uint32_t> m2(n_pad, 0), lo(n_pad, 0), hi(n_pad, 0);
+    std::vector<int32_t> prev(n_pad, 0);
+    for (int c = 0; c < n && fast2; ++c) {
+      if (h_mult[c] < 0 || (int64_t)k * 16384 + (int64_t)k * 128 * llabs((long long)zwv[c]) > (int64_t)kAccBias) {
+        fast2 = false;
+        break;
+      }
+      m2[c] = (uint32_t)h_mult[c] << 1;
+      const uint64_t c2 = (uint64_t)(2 * ((int64_t)h_bias2[c] - (int64_t)kAccBias)) * (uint64_t)(int64_t)h_mult[c] +
+                          ((uint64_t)1 << 31);
+      lo[c] = (uint32_t)c2;
+      hi[c] = (uint32_t)(c2 >> 32);
+      prev[c] = (int32_t)(((uint32_t)1 << e[c]) >> 1) + (int32_t)((uint32_t)zo << e[c]);
+    }
     int rc;
+    if ((rc = upload(&mult2, m2)) != MI_OK) return rc;
+    if ((rc = upload(&c2lo, lo)) != MI_OK) return rc;
+    if ((rc = upload(&c2hi, hi)) != MI_OK) return rc;
+    if ((rc = upload(&pre, prev)) != MI_OK) return rc;
     if ((rc = upload(&mult, h_mult)) != MI_OK) return rc;
     if ((rc = upload(&bias2, h_bias2)) != MI_OK) return rc;
     if ((rc = upload(&rshift, e)) != MI_OK) return rc;
@@ -274,6 +300,10 @@ struct RequantState {
     rshift.release();
     lshift.release();
     zw.release();
+    mult2.release();
+    c2lo.release();
+    c2hi.release();
+    pre.release();
   }
 };
 

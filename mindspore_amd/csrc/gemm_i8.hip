@@ -84,7 +84,7 @@ __device__ __forceinline__ uint32_t pack4(int y0, int y1, int y2, int y3) {
 //      and an aligned base (it routes other shapes through a padded scratch output). ----
 //      Per-channel parameters are read from LDS (array p of kEpiArrays x TILE_N ints, filled by EpiParams below):
 //      global loads here would share the vmcnt counter with the output stores and serialise on them. ----
-constexpr int kEpiArrays = 5;
+constexpr int kEpiArrays = 6;
 constexpr int kDeqStageRowBytes = 144;  // fp32 output staging: 32 columns (128 B) + 16 B so that rows shift banks
 // bytes of the wave-private output staging tile behind the parameter arrays
 template <int EPI, int TM>
@@ -92,7 +92,7 @@ constexpr int epi_stage_bytes() { return EPI == EPI_REQUANT ? 16384 : TM * 32 * 
 
 // The workgroup's per-channel epilogue parameters: thread t holds channel n0 + t of each array (fetched at kernel
 // start, so the latency is hidden by the main loop) and drops them into LDS once the main loop is done.
-template <int TILE_N, int EPI>
+template <int TILE_N, int EPI, bool FAST>
 struct EpiParams {
   int v[kEpiArrays];
   __device__ __forceinline__ void fetch(const RequantParams &rq, const DequantParams &dq, int n0, int tid) {
@@ -100,7 +100,14 @@ struct EpiParams {
     for (int a = 0; a < kEpiArrays; ++a) v[a] = 0;
     if (tid < TILE_N) {
       const int n = n0 + tid;  // arrays are padded to a multiple of 256 channels
-      if (EPI == EPI_REQUANT) {
+      if (EPI == EPI_REQUANT && FAST) {
+        v[0] = (int)rq.mult2[n];
+        v[1] = (int)rq.c2lo[n];
+        v[2] = (int)rq.c2hi[n];
+        v[3] = rq.pre[n];
+        v[4] = rq.rshift[n];
+        v[5] = rq.zw[n];
+      } else if (EPI == EPI_REQUANT) {
         v[0] = rq.mult[n];
         v[1] = rq.bias2[n];
         v[2] = rq.rshift[n];
@@ -129,6 +136,7 @@ template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST, uint32_t 
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)[TM], const GemmArgs &g,
                                               const RequantParams &rq, const DequantParams &dq, const int *p,
                                               char *cstage, int n_tile, int n_w, int m_w, int r, int h) {
+  static_assert(!(EPI == EPI_REQUANT && FAST) || ACC0 == kAccBias, "the host folds kAccBias into c2");
   if (HAS_ZW) {
 #pragma unroll
     for (int j = 0; j < TM; ++j) rowsum[j] += __shfl_xor(rowsum[j], 32);
@@ -141,94 +149,99 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
     // L2 write path then becomes the bottleneck of the whole kernel.  Wave-private staging tile, 128 rows x 128 B:
     // 16-byte chunk c of row R sits at slot c ^ (R & 7), and inside a chunk dword d sits at (d + (R >> 3)) & 3, which
     // makes both the dword writes (32 rows, one column) and the 16-byte row reads bank-conflict free.
+    // The tile is produced and written out in two halves of 64 rows, so that the stores of the first half are under
+    // way while the second half is being requantised.
     constexpr bool kStageC = (TN == 4 && TM == 4);
+    constexpr int kHalves = kStageC ? 2 : 1, kJ = TM / kHalves;
+    const int lane = h * 32 + r;
+    const bool vec16 = ((g.ldc & 15) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
+    for (int jh = 0; jh < kHalves; ++jh) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int nb = n_w + i * 32 + q * 8 + h * 4;
-        if (nb >= g.n) continue;
-        const int *pl = p + (nb - n_tile);
-        const v4i mult4 = *reinterpret_cast<const v4i *>(pl);
-        v4i bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
-        const v4i e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
-        v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
-        int64_t c64[4] = {0, 0, 0, 0};
-        if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
-        if (FAST) {
-          // y = ((srdhm(v, mult) + half - (x < 0)) >> e) + zo with v = acc + bias2 folds into
-          //   x = (acc * mult + (bias2 * mult + 2^30)) >> 31 ;  y = (x + (half + (zo << e)) + (x >> 31)) >> e
-          // (exact because the host proved that none of the intermediate sums can leave int32 / int64)
+      for (int i = 0; i < TN; ++i) {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            pre4[e] = ((1 << e4[e]) >> 1) + (int32_t)((uint32_t)rq.zo << e4[e]);
-            // (acc + ACC0 - ACC0 + bias2) * mult + 2^30, the ACC0 term moved into the constant; 64-bit wrap-around
-            // arithmetic, the true value fits
-            c64[e] = (int64_t)((uint64_t)((int64_t)bias4[e] * (int64_t)mult4[e]) + ((uint64_t)1 << 30) -
-                               (uint64_t)ACC0 * (uint64_t)(int64_t)mult4[e]);
+        for (int q = 0; q < 4; ++q) {
+          const int nb = n_w + i * 32 + q * 8 + h * 4;
+          if (nb >= g.n) continue;
+          const int *pl = p + (nb - n_tile);
+          v4i mult4, bias4 = {0, 0, 0, 0}, e4, zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
+          v4i c2lo4 = {0, 0, 0, 0}, c2hi4 = {0, 0, 0, 0};
+          mult4 = *reinterpret_cast<const v4i *>(pl);
+          if (FAST) {
+            c2lo4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+            c2hi4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
+            pre4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
+            e4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+            if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 5 * TILE_N);
+          } else {
+            bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+            e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
+            if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
+            ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bias4[e] = (int32_t)((uint32_t)bias4[e] - ACC0);
           }
-        } else {
-          ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bias4[e] = (int32_t)((uint32_t)bias4[e] - ACC0);
-        }
+          for (int jj = 0; jj < kJ; ++jj) {
+            const int j = jh * kJ + jj;
+            const int m = m_w + j * 32 + r;
+            int y[4];
 #pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          const int m = m_w + j * 32 + r;
-          int y[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            if (FAST) {
-              int32_t v = acc[i][j][q * 4 + e];
-              if (HAS_ZW) v -= rowsum[j] * zw4[e];
-              const int64_t p = (int64_t)((uint64_t)((int64_t)v * (int64_t)mult4[e]) + (uint64_t)c64[e]);
-              const int32_t x = (int32_t)(p >> 31);
-              const int32_t t = (x + pre4[e] + (x >> 31)) >> e4[e];
-              y[e] = med3_i32(t, amin_v, amax_v);
-            } else {
-              uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
-              if (HAS_ZW) v -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
-              v += (uint32_t)bias4[e];
-              int32_t t = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
-              t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
-              t = t < rq.amax ? t : rq.amax;
-              y[e] = t > rq.amin ? t : rq.amin;
+            for (int e = 0; e < 4; ++e) {
+              if (FAST) {
+                // the host proved that the accumulator register, read as unsigned, stays below 2^31 and that none
+                // of the sums below leaves its type (RequantParams::fast2)
+                uint32_t a = (uint32_t)acc[i][j][q * 4 + e];
+                if (HAS_ZW) a -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
+                const uint64_t c2 = ((uint64_t)(uint32_t)c2hi4[e] << 32) | (uint32_t)c2lo4[e];
+                const uint64_t p2 = (uint64_t)a * (uint64_t)(uint32_t)mult4[e] + c2;
+                const int32_t x = (int32_t)(p2 >> 32);
+                const int32_t t = (x + pre4[e] + (x >> 31)) >> e4[e];
+                y[e] = med3_i32(t, amin_v, amax_v);
+              } else {
+                uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
+                if (HAS_ZW) v -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
+                v += (uint32_t)bias4[e];
+                int32_t t = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
+                t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
+                t = t < rq.amax ? t : rq.amax;
+                y[e] = t > rq.amin ? t : rq.amin;
+              }
             }
-          }
-          const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
-          if (kStageC) {
-            const int row = j * 32 + r;
-            const int slot = (2 * i + (q >> 1)) ^ (r & 7), d = (2 * q + h + (r >> 3)) & 3;
-            *reinterpret_cast<uint32_t *>(cstage + row * 128 + slot * 16 + d * 4) = packed;
-          } else if (m < g.m) {
-            *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
+            const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
+            if (kStageC) {
+              const int row = j * 32 + r;
+              const int slot = (2 * i + (q >> 1)) ^ (r & 7), d = (2 * q + h + (r >> 3)) & 3;
+              *reinterpret_cast<uint32_t *>(cstage + row * 128 + slot * 16 + d * 4) = packed;
+            } else if (m < g.m) {
+              *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
+            }
           }
         }
       }
-    }
-    if (kStageC) {
-      const int lane = h * 32 + r;
-      const int c16 = lane & 7, lrow = lane >> 3;
-      const int n = n_w + c16 * 16;
-      const bool vec16 = ((g.ldc & 15) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+      if (kStageC) {
+        const int c16 = lane & 7, lrow = lane >> 3;
+        const int n = n_w + c16 * 16;
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const int row = lrow + 8 * t;
-        const v4i x = *reinterpret_cast<const v4i *>(cstage + row * 128 + ((c16 ^ lrow) << 4));
-        v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == t & 3
-        o[0] = x[(0 + t) & 3];
-        o[1] = x[(1 + t) & 3];
-        o[2] = x[(2 + t) & 3];
-        o[3] = x[(3 + t) & 3];
-        const int m = m_w + row;
-        if (m < g.m && n < g.n) {
-          int8_t *dst = c + (int64_t)m * g.ldc + n;
-          if (vec16 && n + 16 <= g.n) {
-            *reinterpret_cast<v4i *>(dst) = o;
-          } else {
+        for (int tt = 0; tt < 8; ++tt) {
+          const int t = jh * 8 + tt;
+          const int row = lrow + 8 * t;
+          const v4i x = *reinterpret_cast<const v4i *>(cstage + row * 128 + ((c16 ^ lrow) << 4));
+          v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == t & 3
+          o[0] = x[(0 + t) & 3];
+          o[1] = x[(1 + t) & 3];
+          o[2] = x[(2 + t) & 3];
+          o[3] = x[(3 + t) & 3];
+          const int m = m_w + row;
+          if (m < g.m && n < g.n) {
+            int8_t *dst = c + (int64_t)m * g.ldc + n;
+            if (vec16 && n + 16 <= g.n) {
+              *reinterpret_cast<v4i *>(dst) = o;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
+              for (int e = 0; e < 4; ++e)
+                if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
+            }
           }
         }
       }
@@ -397,7 +410,7 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   const int r = lane & 31, h = lane >> 5;
   const int ktiles = (g.k + BKD - 1) / BKD;  // the zero padding of the weights past K needs no MFMAs
   const int kchunks = g.k >> 4;
-  EpiParams<TILE_N, EPI> epi;
+  EpiParams<TILE_N, EPI, FAST> epi;
   epi.fetch(rq, dq, n0, tid);
 
   // loader: a 1 KiB block holds 16 rows x 64 B.  Lane L fills slot (L & 3) of row (L >> 2) of its block, i.e. it
@@ -457,7 +470,7 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
 #pragma unroll
     for (int j = 0; j < TM; ++j)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = (int)kAccBias;  // see gemm_kblock_kernel
   int rowsum[TM];
 #pragma unroll
   for (int j = 0; j < TM; ++j) rowsum[j] = 0;
@@ -528,7 +541,7 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
-  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
                                                    lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
                                                    m0 + wm * WM, r, h);
 }
@@ -588,7 +601,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int r = lane & 31, h = lane >> 5;
   const int kblocks = (g.k + KB - 1) / KB;
   const int kchunks = g.k >> 4;
-  EpiParams<TILE, EPI> epi;
+  EpiParams<TILE, EPI, FAST> epi;
   epi.fetch(rq, dq, n0, tid);
 
   // loader: instruction i of a wave fills rows 64 * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
@@ -791,11 +804,11 @@ int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
   GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
   DequantParams dq{};
   if (rq.has_zw) {
-    return rq.fast ? launch_pick_tile<EPI_REQUANT, true, true>(g, rq, dq, stream)
-                   : launch_pick_tile<EPI_REQUANT, true, false>(g, rq, dq, stream);
+    return rq.fast2 ? launch_pick_tile<EPI_REQUANT, true, true>(g, rq, dq, stream)
+                    : launch_pick_tile<EPI_REQUANT, true, false>(g, rq, dq, stream);
   }
-  return rq.fast ? launch_pick_tile<EPI_REQUANT, false, true>(g, rq, dq, stream)
-                 : launch_pick_tile<EPI_REQUANT, false, false>(g, rq, dq, stream);
+  return rq.fast2 ? launch_pick_tile<EPI_REQUANT, false, true>(g, rq, dq, stream)
+                  : launch_pick_tile<EPI_REQUANT, false, false>(g, rq, dq, stream);
 }
 
 template <int TILE_N, int TILE_M, bool HAS_ZW, bool FAST, int NST, int OCC>
@@ -847,11 +860,11 @@ int launch_gemm_conv_requant(const int8_t *in, const ConvGeom &cg, const int8_t 
                 magic(cg.kernel_w), fill16};
   GemmArgs g{in, 0, (int)m64, (int)k64, w.w, w.ldw, w.k_pad, cg.out_c, 0, 0, out, cg.out_c};
   if (rq.has_zw) {
-    return rq.fast ? launch_conv_pick_tile<true, true>(g, cv, rq, stream)
-                   : launch_conv_pick_tile<true, false>(g, cv, rq, stream);
+    return rq.fast2 ? launch_conv_pick_tile<true, true>(g, cv, rq, stream)
+                    : launch_conv_pick_tile<true, false>(g, cv, rq, stream);
   }
-  return rq.fast ? launch_conv_pick_tile<false, true>(g, cv, rq, stream)
-                 : launch_conv_pick_tile<false, false>(g, cv, rq, stream);
+  return rq.fast2 ? launch_conv_pick_tile<false, true>(g, cv, rq, stream)
+                  : launch_conv_pick_tile<false, false>(g, cv, rq, stream);
 }
 
 int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
