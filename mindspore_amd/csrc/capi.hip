@@ -263,9 +263,13 @@ struct RequantState {
       m2[c] = (uint32_t)h_mult[c] << 1;
       const uint64_t c2 = (uint64_t)(2 * ((int64_t)h_bias2[c] - (int64_t)kAccBias)) * (uint64_t)(int64_t)h_mult[c] +
                           ((uint64_t)1 << 31);
+      if ((int64_t)c2 >= 0) {  // the epilogue reads the sign of x off the carry of a * mult2 + c2
+        fast2 = false;
+        break;
+      }
       lo[c] = (uint32_t)c2;
       hi[c] = (uint32_t)(c2 >> 32);
-      prev[c] = (int32_t)(((uint32_t)1 << e[c]) >> 1) + (int32_t)((uint32_t)zo << e[c]);
+      prev[c] = (int32_t)(((uint32_t)1 << e[c]) >> 1) + (int32_t)((uint32_t)zo << e[c]) - 1;
     }
     int rc;
     if ((rc = upload(&mult2, m2)) != MI_OK) return rc;

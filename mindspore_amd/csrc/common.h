@@ -45,12 +45,12 @@ struct RequantParams {
   // Single-multiply form of the cheap rounding, for accumulators that start from kAccBias (gemm_i8.hip).  With
   // a = accumulator register read as unsigned (true sum + kAccBias [- rowsum * zw]):
   //   x = high dword of (a * mult2 + c2)      == floor(((sum + bias2) * mult + 2^30) / 2^31), the doubling high mul
-  //   y = clamp((x + pre + (x >> 31)) >> e)   pre = 2^(e-1) + (zo << e)
-  // mult2 = 2 * mult, c2 = 2 * (bias2 - kAccBias) * mult + 2^31 (mod 2^64), split into dwords.
+  //   y = clamp((x + pre + [x >= 0]) >> e)    pre = 2^(e-1) + (zo << e) - 1; [x >= 0] is the carry of a * mult2 + c2
+  // mult2 = 2 * mult, c2 = 2 * (bias2 - kAccBias) * mult + 2^31 (mod 2^64, negative as a signed number), in dwords.
   const uint32_t *mult2;
   const uint32_t *c2lo, *c2hi;
   const int32_t *pre;
-  int fast2;   // fast, and every mult >= 0, and K * 16384 + K * 128 * |zw| <= kAccBias (a stays in [0, 2^31))
+  int fast2;   // fast, and every mult >= 0, every c2 < 0, and K * 16384 + K * 128 * |zw| <= kAccBias (a in [0, 2^31))
 };
 
 // ---- fp32 dequantising epilogue (dynamic-quant MatMul) ----

@@ -102,7 +102,7 @@ struct EpiParams {
       const int n = n0 + tid;  // arrays are padded to a multiple of 256 channels
       if (EPI == EPI_REQUANT && FAST) {
         v[0] = (int)rq.mult2[n];
-        v[1] = (int)rq.c2lo[n];
+        v[1] = (int)rq.c2lo[n];  // arrays 1 and 2 are interleaved in LDS: {lo, hi} of channel t at 2 * t
         v[2] = (int)rq.c2hi[n];
         v[3] = rq.pre[n];
         v[4] = rq.rshift[n];
@@ -124,7 +124,13 @@ struct EpiParams {
   __device__ __forceinline__ void to_lds(int *p, int tid) const {
     if (tid < TILE_N) {
 #pragma unroll
-      for (int a = 0; a < kEpiArrays; ++a) p[a * TILE_N + tid] = v[a];
+      for (int a = 0; a < kEpiArrays; ++a) {
+        if (EPI == EPI_REQUANT && FAST && (a == 1 || a == 2)) {
+          p[TILE_N + 2 * tid + (a - 1)] = v[a];
+        } else {
+          p[a * TILE_N + tid] = v[a];
+        }
+      }
     }
     __syncthreads();
   }
@@ -143,108 +149,175 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
   }
   if (EPI == EPI_REQUANT) {
     int8_t *c = static_cast<int8_t *>(g.c);
-    const int amin_v = rq.amin, amax_v = rq.amax;
+    int amin_v = rq.amin, amax_v = rq.amax;
+    asm volatile("" : "+v"(amin_v), "+v"(amax_v));  // kept in vector registers, as v_med3 wants them
     // A 128-channel-wide wave tile goes through LDS so that global memory sees whole 128-byte rows: written
     // straight from the accumulator layout, every store instruction would touch 32 rows with 8 bytes each, and the
     // L2 write path then becomes the bottleneck of the whole kernel.  Wave-private staging tile, 128 rows x 128 B:
     // 16-byte chunk c of row R sits at slot c ^ (R & 7), and inside a chunk dword d sits at (d + (R >> 3)) & 3, which
     // makes both the dword writes (32 rows, one column) and the 16-byte row reads bank-conflict free.
-    // The tile is produced and written out in two halves of 64 rows, so that the stores of the first half are under
-    // way while the second half is being requantised.
+    // The output leaves at memory-write speed (all workgroups reach this point together), and a store instruction
+    // that finds the write queue full holds up the wave: so the tile is requantised in two halves of 64 rows, and the
+    // eight store instructions of the first half are issued one at a time between the pieces of the second.  (Four
+    // passes of 32 rows would hide more of the stores, but every pass re-reads the per-channel constants from LDS,
+    // and at four passes those reads take longer than the arithmetic.)
     constexpr bool kStageC = (TN == 4 && TM == 4);
-    constexpr int kHalves = kStageC ? 2 : 1, kJ = TM / kHalves;
     const int lane = h * 32 + r;
     const bool vec16 = ((g.ldc & 15) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
+    // four outputs (consecutive channels of one row): accumulator registers -> clamped int32
+    auto requant4 = [&](const int32_t (&accv)[4], int rsum, v4i mult, v4i c2lo, v4i c2hi, v4i pre, v4i bias, v4i e4,
+                        v4i ls, v4i zw, int (&y)[4]) {
+      if (FAST) {
+        // the host proved that the accumulator register, read as unsigned, stays below 2^31, that c2 is negative and
+        // that none of the sums below leaves its type (RequantParams::fast2).  p2 = a * mult2 + c2 as unsigned 64-bit
+        // numbers carries out exactly when the true (signed) sum is >= 0, i.e. when x >= 0: the carry is the
+        // "+1 unless negative" of the rounding, so pre arrives here as pre - 1.  The four chains are written stage
+        // by stage so that no instruction waits for the one before it.
+        uint64_t p2[4], carry[4], unused;
+        int32_t t[4];
 #pragma unroll
-    for (int jh = 0; jh < kHalves; ++jh) {
+        for (int e = 0; e < 4; ++e) {
+          uint32_t a = (uint32_t)accv[e];
+          if (HAS_ZW) a -= (uint32_t)rsum * (uint32_t)zw[e];
+          const uint64_t c2 = ((uint64_t)(uint32_t)c2hi[e] << 32) | (uint32_t)c2lo[e];
+          asm("v_mad_u64_u32 %0, %1, %2, %3, %4" : "=&v"(p2[e]), "=s"(carry[e]) : "v"(a), "v"(mult[e]), "v"(c2));
+        }
 #pragma unroll
-      for (int i = 0; i < TN; ++i) {
+        for (int e = 0; e < 4; ++e)
+          asm("v_addc_co_u32_e64 %0, %1, %2, %3, %4"
+              : "=v"(t[e]), "=s"(unused)
+              : "v"((int32_t)(p2[e] >> 32)), "v"(pre[e]), "s"(carry[e]));
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int nb = n_w + i * 32 + q * 8 + h * 4;
-          if (nb >= g.n) continue;
-          const int *pl = p + (nb - n_tile);
-          v4i mult4, bias4 = {0, 0, 0, 0}, e4, zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0}, pre4 = {0, 0, 0, 0};
-          v4i c2lo4 = {0, 0, 0, 0}, c2hi4 = {0, 0, 0, 0};
-          mult4 = *reinterpret_cast<const v4i *>(pl);
-          if (FAST) {
-            c2lo4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
-            c2hi4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
-            pre4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
-            e4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
-            if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 5 * TILE_N);
+        for (int e = 0; e < 4; ++e) t[e] >>= e4[e];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) y[e] = med3_i32(t[e], amin_v, amax_v);
+        return;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t v = (uint32_t)accv[e];
+        if (HAS_ZW) v -= (uint32_t)rsum * (uint32_t)zw[e];
+        v += (uint32_t)bias[e];
+        int32_t t = rdiv_pot(srdhm((int32_t)(v << ls[e]), mult[e]), e4[e]);
+        t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
+        t = t < rq.amax ? t : rq.amax;
+        y[e] = t > rq.amin ? t : rq.amin;
+      }
+    };
+    // whole wave tile inside the matrix and 16-byte stores possible: the stores need no bounds checks
+    const bool full_tile = vec16 && m_w + 32 * TM <= g.m && n_w + 32 * TN <= g.n;
+    // The body is compiled twice: for wave tiles that lie wholly inside the matrix with 16-byte stores possible
+    // (no bounds checks, no divergent branches around the stores) and for the ragged rest.
+    auto body = [&](auto full_c) {
+      constexpr bool FULL = decltype(full_c)::value;
+      // rows lrow + 8 * t of the staging tile -> global memory (t: 0..15, one store instruction)
+      auto store_rows = [&](int t) {
+        const int c16 = lane & 7, lrow = lane >> 3;
+        const int n = n_w + c16 * 16;
+        const int row = lrow + 8 * t;
+        const v4i x = *reinterpret_cast<const v4i *>(cstage + row * 128 + ((c16 ^ lrow) << 4));
+        v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == t & 3
+        o[0] = x[(0 + t) & 3];
+        o[1] = x[(1 + t) & 3];
+        o[2] = x[(2 + t) & 3];
+        o[3] = x[(3 + t) & 3];
+        const int m = m_w + row;
+        if (FULL) {
+          *reinterpret_cast<v4i *>(c + (int64_t)m * g.ldc + n) = o;
+        } else if (m < g.m && n < g.n) {
+          int8_t *dst = c + (int64_t)m * g.ldc + n;
+          if (vec16 && n + 16 <= g.n) {
+            *reinterpret_cast<v4i *>(dst) = o;
           } else {
-            bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
-            e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
-            if (HAS_ZW) zw4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
-            ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) bias4[e] = (int32_t)((uint32_t)bias4[e] - ACC0);
+  #pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
           }
-#pragma unroll
-          for (int jj = 0; jj < kJ; ++jj) {
-            const int j = jh * kJ + jj;
-            const int m = m_w + j * 32 + r;
-            int y[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (FAST) {
-                // the host proved that the accumulator register, read as unsigned, stays below 2^31 and that none
-                // of the sums below leaves its type (RequantParams::fast2)
-                uint32_t a = (uint32_t)acc[i][j][q * 4 + e];
-                if (HAS_ZW) a -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
-                const uint64_t c2 = ((uint64_t)(uint32_t)c2hi4[e] << 32) | (uint32_t)c2lo4[e];
-                const uint64_t p2 = (uint64_t)a * (uint64_t)(uint32_t)mult4[e] + c2;
-                const int32_t x = (int32_t)(p2 >> 32);
-                const int32_t t = (x + pre4[e] + (x >> 31)) >> e4[e];
-                y[e] = med3_i32(t, amin_v, amax_v);
+        }
+      };
+      constexpr int kPhases = kStageC ? 2 : 1, kJ = TM / kPhases;  // row blocks per pass over the channels
+      // where this lane's dword of piece (i, q) goes in its staging row (see the layout above)
+      int stage_off[kStageC ? TN * 4 : 1];
+      if (kStageC) {
+  #pragma unroll
+        for (int i = 0; i < TN; ++i)
+  #pragma unroll
+          for (int q = 0; q < 4; ++q)
+            stage_off[i * 4 + q] = r * 128 + (((2 * i + (q >> 1)) ^ (r & 7)) << 4) + (((2 * q + h + (r >> 3)) & 3) << 2);
+      }
+      // per-channel constants of one piece (4 channels); the next piece's are requested before this piece's
+      // arithmetic starts, so that the LDS latency is not paid once per piece
+      struct Piece {
+        v4i mult4, bias4, e4, zw4, ls4, pre4, c01, c23;
+      };
+      auto load_piece = [&](int blk) {
+        Piece pc;
+        const int i = (blk >> 2) % TN, q = blk & 3;
+        int nb = n_w + i * 32 + q * 8 + h * 4;
+        const int *pl = p + (nb - n_tile);
+        pc.mult4 = *reinterpret_cast<const v4i *>(pl);
+        pc.bias4 = pc.zw4 = pc.ls4 = pc.pre4 = pc.c01 = pc.c23 = v4i{0, 0, 0, 0};
+        if (FAST) {
+          pc.c01 = *reinterpret_cast<const v4i *>(p + TILE_N + 2 * (nb - n_tile));  // {lo, hi} x 2
+          pc.c23 = *reinterpret_cast<const v4i *>(p + TILE_N + 2 * (nb - n_tile) + 4);
+          pc.pre4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
+          pc.e4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+          if (HAS_ZW) pc.zw4 = *reinterpret_cast<const v4i *>(pl + 5 * TILE_N);
+        } else {
+          pc.bias4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+          pc.e4 = *reinterpret_cast<const v4i *>(pl + 2 * TILE_N);
+          if (HAS_ZW) pc.zw4 = *reinterpret_cast<const v4i *>(pl + 3 * TILE_N);
+          pc.ls4 = *reinterpret_cast<const v4i *>(pl + 4 * TILE_N);
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) pc.bias4[e] = (int32_t)((uint32_t)pc.bias4[e] - ACC0);
+        }
+        return pc;
+      };
+      Piece next = load_piece(0);
+  #pragma unroll
+      for (int ph = 0; ph < kPhases; ++ph) {
+  #pragma unroll
+        for (int i = 0; i < TN; ++i) {
+  #pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int nb = n_w + i * 32 + q * 8 + h * 4;
+            const Piece pc = next;
+            next = load_piece(i * 4 + q + 1);  // (wraps to piece 0 for the next pass; the arrays are padded)
+            // (the staged form computes every channel of the padded tile and lets the stores check the bounds)
+            if (!kStageC && nb >= g.n) continue;
+            const v4i c2lo4 = v4i{pc.c01[0], pc.c01[2], pc.c23[0], pc.c23[2]};
+            const v4i c2hi4 = v4i{pc.c01[1], pc.c01[3], pc.c23[1], pc.c23[3]};
+  #pragma unroll
+            for (int jj = 0; jj < kJ; ++jj) {
+              const int j = ph * kJ + jj;
+              int y[4];
+              const int32_t a4[4] = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+              requant4(a4, rowsum[j], pc.mult4, c2lo4, c2hi4, pc.pre4, pc.bias4, pc.e4, pc.ls4, pc.zw4, y);
+              const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
+              if (kStageC) {
+                *reinterpret_cast<uint32_t *>(cstage + j * 32 * 128 + stage_off[i * 4 + q]) = packed;
               } else {
-                uint32_t v = (uint32_t)acc[i][j][q * 4 + e];
-                if (HAS_ZW) v -= (uint32_t)rowsum[j] * (uint32_t)zw4[e];
-                v += (uint32_t)bias4[e];
-                int32_t t = rdiv_pot(srdhm((int32_t)(v << ls4[e]), mult4[e]), e4[e]);
-                t = (int32_t)((uint32_t)t + (uint32_t)rq.zo);
-                t = t < rq.amax ? t : rq.amax;
-                y[e] = t > rq.amin ? t : rq.amin;
+                const int m = m_w + j * 32 + r;
+                if (m < g.m) *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
               }
             }
-            const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
-            if (kStageC) {
-              const int row = j * 32 + r;
-              const int slot = (2 * i + (q >> 1)) ^ (r & 7), d = (2 * q + h + (r >> 3)) & 3;
-              *reinterpret_cast<uint32_t *>(cstage + row * 128 + slot * 16 + d * 4) = packed;
-            } else if (m < g.m) {
-              *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
+            if (kStageC && ph == 1 && (q & 1)) {  // the first half's eight store instructions, one per two pieces
+              __builtin_amdgcn_sched_barrier(0);
+              store_rows(i * 2 + (q >> 1));
+              __builtin_amdgcn_sched_barrier(0);
             }
           }
         }
       }
       if (kStageC) {
-        const int c16 = lane & 7, lrow = lane >> 3;
-        const int n = n_w + c16 * 16;
-#pragma unroll
-        for (int tt = 0; tt < 8; ++tt) {
-          const int t = jh * 8 + tt;
-          const int row = lrow + 8 * t;
-          const v4i x = *reinterpret_cast<const v4i *>(cstage + row * 128 + ((c16 ^ lrow) << 4));
-          v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == t & 3
-          o[0] = x[(0 + t) & 3];
-          o[1] = x[(1 + t) & 3];
-          o[2] = x[(2 + t) & 3];
-          o[3] = x[(3 + t) & 3];
-          const int m = m_w + row;
-          if (m < g.m && n < g.n) {
-            int8_t *dst = c + (int64_t)m * g.ldc + n;
-            if (vec16 && n + 16 <= g.n) {
-              *reinterpret_cast<v4i *>(dst) = o;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
-            }
-          }
-        }
+  #pragma unroll
+        for (int t = 8; t < 16; ++t) store_rows(t);
       }
+    };
+    if (full_tile) {
+      body(std::true_type());
+    } else {
+      body(std::false_type());
     }
   } else {
     float *c = static_cast<float *>(g.c);
@@ -571,9 +644,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
 //   Q3  MFMAs on chunks 4-5 | reads chunks 6-7, then waits for its own LDS reads and loads and meets the other
 //       waves: block b+1 is complete in LDS and nobody reads block b any more
 //   Q4  MFMAs on chunks 6-7 | reads chunks 0-1 of block b+1 | issues the loads of W block b+2 into block b's slot
-// One barrier per 128 bytes of K.  In a slot, 16-byte chunk c of row R sits at position c ^ (R & 7): the loader's
-// 1 KiB writes (8 rows x 8 chunks) and the fragment reads (8 consecutive rows, one logical chunk) both cover all
-// 32 banks.
+// One barrier per 128 bytes of K.  In a slot, 16-byte chunk c of row R sits at position c ^ ((R >> 1) & 7): the LDS
+// has 64 banks (256 bytes per clock), so 16 consecutive rows of one logical chunk -- what 16 lanes of a fragment
+// read ask for -- must land on 16 different 16-byte positions of a 256-byte period, and two rows of 128 bytes make
+// one period.
 //
 // kAccBias: the accumulators start from this constant instead of 0 and the epilogue's per-channel constants take it
 // out again (exact: wrap-around arithmetic).  Partial sums of signed products hover around zero, where every sign
@@ -586,6 +660,7 @@ template <int EPI, bool HAS_ZW, bool FAST>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kblock_kernel(GemmArgs g,
                                                                                                       RequantParams rq,
                                                                                                       DequantParams dq) {
+#if defined(__HIP_DEVICE_COMPILE__)  // the buffer-resource type exists in the device pass only; the host pass needs just the stub
   constexpr int TILE = 256, KB = 128, T = 4;  // wave tile 128 x 128 = T x T MFMA tiles
   constexpr int SLOT = TILE * KB;             // one operand, one K block
   constexpr int LPW = 8;                      // loader instructions per wave, operand and block (64 rows)
@@ -605,29 +680,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   epi.fetch(rq, dq, n0, tid);
 
   // loader: instruction i of a wave fills rows 64 * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
-  // L & 7 of its row, i.e. fetches logical chunk (L & 7) ^ (row & 7)
+  // L & 7 of its row, i.e. fetches logical chunk (L & 7) ^ ((row >> 1) & 7).  The loads are buffer loads: the address
+  // is descriptor base + per-lane byte offset (a loop constant) + a scalar offset (row group and K block), so
+  // issuing one costs scalar instructions only.
   const int drow = lane >> 3;
-  const int dchunk = (lane & 7) ^ drow;
-  const int8_t *wsrc = g.w + (int64_t)(n0 + wave * 64 + drow) * g.ldw + dchunk * 16;
-  const int8_t *asrc[LPW];
+  const int dchunk = (lane & 7) ^ (drow >> 1);  // for even i; odd i: ^ 4
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<int8_t *>(g.w) + (int64_t)(n0 + wave * 64) * g.ldw, (short)0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(g.a) + (int64_t)m0 * g.lda, (short)0, -1, 0x00020000);
+  const int w_voff = drow * g.ldw + dchunk * 16;  // ldw is a multiple of 256: odd i is w_voff ^ 64
+  int a_voff[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
-    int m = m0 + wave * 64 + 8 * i + drow;
-    m = m < g.m ? m : g.m - 1;
-    asrc[i] = g.a + (int64_t)m * g.lda;
+    int m = wave * 64 + 8 * i + drow;
+    m = m0 + m < g.m ? m : g.m - 1 - m0;
+    a_voff[i] = m * (int)g.lda + ((dchunk ^ ((i & 1) << 2)) << 4);
   }
-  const int a_last = (kchunks - 1) * 16;
+  // A has exactly K valid bytes per row (the weights are zero padded, A is the caller's): in the last K block a
+  // 16-byte chunk past K is fetched from the row's last chunk instead.  The offsets are moved there once, before
+  // that block is first requested (the re-fetches after it ask for the same block).
+  const int a_last = (kchunks - 1) * 16 - (kblocks - 1) * KB;  // offset of the last valid chunk in the last block
+  auto a_offsets_for_last_block = [&]() {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int c16 = (dchunk ^ ((i & 1) << 2)) << 4;
+      a_voff[i] += (c16 < a_last ? c16 : a_last) - c16;
+    }
+  };
+  auto lds_ptr = [](char *p) { return (__attribute__((address_space(3))) void *)p; };
   auto dma_w = [&](int slot, int kb) {
     char *dst = lds + slot * SLOT + wave * 64 * KB;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) async_copy16(wsrc + (int64_t)(8 * i) * g.ldw + kb * KB, dst + i * 1024);
+    for (int i = 0; i < LPW; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, lds_ptr(dst + i * 1024), 16, w_voff ^ ((i & 1) << 6),
+                                               8 * i * g.ldw + kb * KB, 0, 0);
   };
   auto dma_a = [&](int slot, int kb) {
     char *dst = lds + (2 + slot) * SLOT + wave * 64 * KB;
-    int koff = kb * KB + dchunk * 16;
-    koff = koff < a_last ? koff : a_last;  // past K: any valid read will do, the weights are zero there
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) async_copy16(asrc[i] + koff, dst + i * 1024);
+    for (int i = 0; i < LPW; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, lds_ptr(dst + i * 1024), 16, a_voff[i], kb * KB, 0, 0);
   };
 
   v16i acc[T][T];
@@ -641,7 +734,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
   for (int j = 0; j < T; ++j) rowsum[j] = 0;
 
-  const int swz = r & 7;
+  const int swz = (r >> 1) & 7;
   const int w_off = (wn * 128 + r) * KB, a_off = 2 * SLOT + (wm * 128 + r) * KB;
   Frag<T, T> f0, f1;
   auto read_frag = [&](Frag<T, T> &f, int slot, int q) {  // q: 32-byte sub-step inside the block
@@ -690,6 +783,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  if (kblocks == 1) a_offsets_for_last_block();
   dma_w(0, 0);
   dma_a(0, 0);
   dma_w(1, kblocks > 1 ? 1 : 0);
@@ -699,6 +793,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int slot = b & 1;
     const int kb_a = b + 1 < kblocks ? b + 1 : kblocks - 1;  // past the end: re-fetch the last block into a slot
     const int kb_w = b + 2 < kblocks ? b + 2 : kblocks - 1;  // nobody reads again
+    if (b + 2 == kblocks) a_offsets_for_last_block();
     read_frag(f1, slot, 1);
     dma_a(slot ^ 1, kb_a);
     mma(f0, b * 8 + h);
@@ -722,6 +817,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
                                                          lds + kEpiArrays * TILE * 4 + wave * epi_stage_bytes<EPI, T>(),
                                                          n0, n0 + wn * 128, m0 + wm * 128, r, h);
+#endif
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
@@ -756,7 +852,9 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
   // the fp32 epilogue writes four times the bytes: below one 256 x 256 tile per CU it is worth more to overlap it
   // with another workgroup's main loop (two 128 x 128 tiles per CU) than to save operand traffic
-  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192)) return launch_kblock<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  // (its loader addresses activation rows with 32-bit offsets from the tile's first row)
+  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192) && g.lda < (1 << 23))
+    return launch_kblock<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // a few hundred activation rows against many channels: 256-channel x 128-row tiles keep the weight re-reads of
   // the square 128 tile away while still giving every CU a tile
   if (g.m <= 512 && (int64_t)((g.m + 127) / 128) * ((g.n + 255) / 256) >= 128)
