@@ -636,14 +636,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
 // What the compute-bound GEMM pays for is operand delivery: the L2 -> L1 path moves whole 128-byte lines, so a loader
 // that asks for 64 bytes of a row per K step has every line sent twice, one K step apart.  Here K advances in blocks of 128 bytes
 // -- whole cache lines -- so that each line leaves the L2 once: one wave instruction fetches 8 rows x 128 bytes.
-// LDS holds two slots per operand (slot = 256 rows x 128 B = 32 KiB; 128 KiB in all).  A loop iteration is one K
-// block = four 32-byte MFMA sub-steps (quarters) on double-buffered fragments:
-//   Q1  MFMAs on chunks 0-1 | reads chunks 2-3 | issues the loads of A block b+1 (its slot was released by the
-//                                               previous iteration's barrier)
-//   Q2  MFMAs on chunks 2-3 | reads chunks 4-5
-//   Q3  MFMAs on chunks 4-5 | reads chunks 6-7, then waits for its own LDS reads and loads and meets the other
-//       waves: block b+1 is complete in LDS and nobody reads block b any more
-//   Q4  MFMAs on chunks 6-7 | reads chunks 0-1 of block b+1 | issues the loads of W block b+2 into block b's slot
+// LDS holds three slots for W and two for A (slot = 256 rows x 128 B = 32 KiB; all 160 KiB of the CU).  The path from
+// the L1 into LDS moves 64 bytes per clock and CU: four waves issuing eight 1 KiB loads each within one quarter of a
+// block saturate it, and a wave whose load does not fit the queue cannot issue its next MFMA either.  So every quarter
+// issues four loads per wave, which takes a load window of a whole block per operand, hence the third W slot.  A loop
+// iteration is one K block = four 32-byte MFMA sub-steps (quarters) on double-buffered fragments:
+//   Q1  MFMAs on chunks 0-1 | reads chunks 2-3 | loads the second half of A block b+1
+//   Q2  MFMAs on chunks 2-3 | reads chunks 4-5 | loads the first half of W block b+2 (into block b-1's slot)
+//   Q3  MFMAs on chunks 4-5 | reads chunks 6-7 | loads the second half of W block b+2, then waits until all but
+//       these eight W loads have landed (loads complete in order) and meets the other waves: block b+1 is complete
+//       in LDS and nobody reads block b any more
+//   Q4  MFMAs on chunks 6-7 | reads chunks 0-1 of block b+1 | loads the first half of A block b+2 into block b's slot
 // One barrier per 128 bytes of K.  In a slot, 16-byte chunk c of row R sits at position c ^ ((R >> 1) & 7): the LDS
 // has 64 banks (256 bytes per clock), so 16 consecutive rows of one logical chunk -- what 16 lanes of a fragment
 // read ask for -- must land on 16 different 16-byte positions of a 256-byte period, and two rows of 128 bytes make
@@ -664,8 +667,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   constexpr int TILE = 256, KB = 128, T = 4;  // wave tile 128 x 128 = T x T MFMA tiles
   constexpr int SLOT = TILE * KB;             // one operand, one K block
   constexpr int LPW = 8;                      // loader instructions per wave, operand and block (64 rows)
-  static_assert(4 * SLOT >= kEpiArrays * TILE * 4 + 4 * epi_stage_bytes<EPI, T>(), "the epilogue staging must fit");
-  __shared__ __attribute__((aligned(1024))) char lds[4 * SLOT];  // W slot 0, W slot 1, A slot 0, A slot 1
+  static_assert(5 * SLOT >= kEpiArrays * TILE * 4 + 4 * epi_stage_bytes<EPI, T>(), "the epilogue staging must fit");
+  __shared__ __attribute__((aligned(1024))) char lds[5 * SLOT];  // W slots 0-2, A slots 0-1
 
   int tile_m, tile_n;
   tile_coords(g, &tile_m, &tile_n);
@@ -709,18 +712,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
   };
   auto lds_ptr = [](char *p) { return (__attribute__((address_space(3))) void *)p; };
-  auto dma_w = [&](int slot, int kb) {
+  // half: 0 = the wave's first four loader instructions (rows 0-31 of its 64), 1 = the other four
+  auto dma_w = [&](int slot, int kb, int half) {
     char *dst = lds + slot * SLOT + wave * 64 * KB;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i)
+    for (int ii = 0; ii < LPW / 2; ++ii) {
+      const int i = half * (LPW / 2) + ii;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, lds_ptr(dst + i * 1024), 16, w_voff ^ ((i & 1) << 6),
                                                8 * i * g.ldw + kb * KB, 0, 0);
+    }
   };
-  auto dma_a = [&](int slot, int kb) {
-    char *dst = lds + (2 + slot) * SLOT + wave * 64 * KB;
+  auto dma_a = [&](int slot, int kb, int half) {
+    char *dst = lds + (3 + slot) * SLOT + wave * 64 * KB;
 #pragma unroll
-    for (int i = 0; i < LPW; ++i)
+    for (int ii = 0; ii < LPW / 2; ++ii) {
+      const int i = half * (LPW / 2) + ii;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, lds_ptr(dst + i * 1024), 16, a_voff[i], kb * KB, 0, 0);
+    }
   };
 
   v16i acc[T][T];
@@ -735,14 +743,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int j = 0; j < T; ++j) rowsum[j] = 0;
 
   const int swz = (r >> 1) & 7;
-  const int w_off = (wn * 128 + r) * KB, a_off = 2 * SLOT + (wm * 128 + r) * KB;
+  const int w_off = (wn * 128 + r) * KB, a_off = 3 * SLOT + (wm * 128 + r) * KB;
   Frag<T, T> f0, f1;
-  auto read_frag = [&](Frag<T, T> &f, int slot, int q) {  // q: 32-byte sub-step inside the block
-    const char *base = lds + slot * SLOT + (((2 * q + h) ^ swz) << 4);
+  auto read_frag = [&](Frag<T, T> &f, int wslot, int aslot, int q) {  // q: 32-byte sub-step inside the block
+    const int c = ((2 * q + h) ^ swz) << 4;
+    const char *wb = lds + wslot * SLOT + w_off + c, *ab = lds + aslot * SLOT + a_off + c;
 #pragma unroll
-    for (int i = 0; i < T; ++i) f.w[i] = *reinterpret_cast<const v4i *>(base + w_off + i * 32 * KB);
+    for (int i = 0; i < T; ++i) f.w[i] = *reinterpret_cast<const v4i *>(wb + i * 32 * KB);
 #pragma unroll
-    for (int j = 0; j < T; ++j) f.a[j] = *reinterpret_cast<const v4i *>(base + a_off + j * 32 * KB);
+    for (int j = 0; j < T; ++j) f.a[j] = *reinterpret_cast<const v4i *>(ab + j * 32 * KB);
   };
   auto mma = [&](const Frag<T, T> &f, int chunk) {
     if (HAS_ZW) {
@@ -765,51 +774,62 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.a[j], acc[i][j], 0, 0, 0);
       }
   };
-  // one LDS read behind each of the first 8 MFMAs of a quarter, then (when the quarter issues loads) one load
-  // behind each of the other 8
-  auto hints = [&](auto with_loads) {
+  // one LDS read behind each of the first 8 MFMAs of a quarter, then one load behind every other one of the rest
+  auto hints = [&]() {
 #pragma unroll
     for (int i = 0; i < 2 * T; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
     }
-    if constexpr (decltype(with_loads)::value) {
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
-      }
+    for (int i = 0; i < LPW / 2; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  const int last = kblocks - 1;
   if (kblocks == 1) a_offsets_for_last_block();
-  dma_w(0, 0);
-  dma_a(0, 0);
-  dma_w(1, kblocks > 1 ? 1 : 0);
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LPW) : "memory");
-  read_frag(f0, 0, 0);
+  dma_w(0, 0, 0);
+  dma_w(0, 0, 1);
+  dma_a(0, 0, 0);
+  dma_a(0, 0, 1);
+  if (kblocks == 2) a_offsets_for_last_block();
+  dma_w(1, last < 1 ? last : 1, 0);
+  dma_w(1, last < 1 ? last : 1, 1);
+  dma_a(1, last < 1 ? last : 1, 0);
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LPW + LPW / 2) : "memory");  // W(0) and A(0) are in
+  read_frag(f0, 0, 0, 0);
+  int ws = 0, ws1 = 1, ws2 = 2;  // W slots of blocks b, b+1, b+2
   for (int b = 0; b < kblocks; ++b) {
-    const int slot = b & 1;
-    const int kb_a = b + 1 < kblocks ? b + 1 : kblocks - 1;  // past the end: re-fetch the last block into a slot
-    const int kb_w = b + 2 < kblocks ? b + 2 : kblocks - 1;  // nobody reads again
-    if (b + 2 == kblocks) a_offsets_for_last_block();
-    read_frag(f1, slot, 1);
-    dma_a(slot ^ 1, kb_a);
+    const int as = b & 1;
+    const int kb1 = b + 1 < last ? b + 1 : last;  // past the end: the last block again, into a slot nobody reads
+    const int kb2 = b + 2 < last ? b + 2 : last;
+    read_frag(f1, ws, as, 1);
+    dma_a(as ^ 1, kb1, 1);
     mma(f0, b * 8 + h);
-    hints(std::true_type());
-    read_frag(f0, slot, 2);
+    hints();
+    read_frag(f0, ws, as, 2);
+    dma_w(ws2, kb2, 0);
     mma(f1, b * 8 + 2 + h);
-    hints(std::false_type());
-    read_frag(f1, slot, 3);
+    hints();
+    read_frag(f1, ws, as, 3);
+    dma_w(ws2, kb2, 1);
     mma(f0, b * 8 + 4 + h);
-    hints(std::false_type());
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    hints();
+    // everything but the eight loads of W block b+2 has landed: that includes all of block b+1
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LPW) : "memory");
     __builtin_amdgcn_sched_barrier(0);
-    read_frag(f0, slot ^ 1, 0);
-    dma_w(slot, kb_w);
+    if (b + 3 == kblocks) a_offsets_for_last_block();
+    read_frag(f0, ws1, as ^ 1, 0);
+    dma_a(as, kb2, 0);
     mma(f1, b * 8 + 6 + h);
-    hints(std::true_type());
+    hints();
+    const int t = ws;
+    ws = ws1;
+    ws1 = ws2;
+    ws2 = t;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing re-fetches land before the LDS is reused
   __syncthreads();

@@ -82,10 +82,11 @@ def test_decode_rows_every_stream_shape(orc, n, k):
         assert np.array_equal(got, want), (m, n, k, int((got != want).sum()))
 
 
-@pytest.mark.parametrize("m,n,k", [(2100, 6144, 1008), (3073, 4100, 144), (4096, 3072, 64), (2049, 6148, 400)])
+@pytest.mark.parametrize("m,n,k", [(2100, 6144, 1008), (3073, 4100, 144), (4096, 3072, 64), (2049, 6148, 400),
+                                   (3072, 4096, 336)])
 def test_matmul_whole_cu_tile_ragged(orc, m, n, k):
     """The 256 x 256 tile (128-byte K blocks, biased accumulators) with ragged rows, channels and K: K below one
-    block, K that ends inside a block, inside its first half, per-tensor / per-channel, zero and non-zero weight zero
+    block, two, three and more blocks, K that ends inside a block, inside its first half, per-tensor / per-channel, zero and non-zero weight zero
     points, the generic rounding path."""
     rng = np.random.default_rng(m + n + k)
     orc.set_threads(16)
