@@ -223,7 +223,9 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
         o[3] = x[(3 + t) & 3];
         const int m = m_w + row;
         if (FULL) {
-          *reinterpret_cast<v4i *>(c + (int64_t)m * g.ldc + n) = o;
+          // (the staged form only runs on outputs of a dozen megabytes and more: streamed past the L2, they leave no
+          //  dirty lines for the end-of-kernel write-back, which otherwise adds ~1.5 us before the next kernel starts)
+          __builtin_nontemporal_store(o, reinterpret_cast<v4i *>(c + (int64_t)m * g.ldc + n));
         } else if (m < g.m && n < g.n) {
           int8_t *dst = c + (int64_t)m * g.ldc + n;
           if (vec16 && n + 16 <= g.n) {
@@ -732,15 +734,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
 
   v16i acc[T][T];
-#pragma unroll
-  for (int i = 0; i < T; ++i)
-#pragma unroll
-    for (int j = 0; j < T; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = (int)kAccBias;
   int rowsum[T];
 #pragma unroll
   for (int j = 0; j < T; ++j) rowsum[j] = 0;
+  // the 256 accumulator registers are set while the first tiles are on their way (see below)
+  auto init_accumulators = [&]() {
+    const int bias = (int)kAccBias;
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+      for (int j = 0; j < T; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e)  // volatile: stays ahead of the wait for the first tiles
+          asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(acc[i][j][e]) : "v"(bias));
+  };
 
   const int swz = (r >> 1) & 7;
   const int w_off = (wn * 128 + r) * KB, a_off = 3 * SLOT + (wm * 128 + r) * KB;
@@ -799,6 +806,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   dma_w(1, last < 1 ? last : 1, 0);
   dma_w(1, last < 1 ? last : 1, 1);
   dma_a(1, last < 1 ? last : 1, 0);
+  init_accumulators();
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LPW + LPW / 2) : "memory");  // W(0) and A(0) are in
   read_frag(f0, 0, 0, 0);
   int ws = 0, ws1 = 1, ws2 = 2;  // W slots of blocks b, b+1, b+2
