@@ -131,6 +131,15 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
 int mi_matmul_run_noalloc(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
 /* Same with host tensors: copies in, runs, copies out, synchronises. */
 int mi_matmul_run_host(mi_matmul *h, const int8_t *a_host, int32_t rows, int8_t *c_host);
+/* Several MatMul / FullConnection kernels that read the same input tensor (same `deep`), e.g. the gate and up
+ * projections of a decoder layer or separate Q, K, V projections: equal to mi_matmul_run(handles[i], a_dev, rows,
+ * c_dev[i], stream) for i = 0 .. count-1.  With at most 32 rows and two to four members the weight-streaming kernels
+ * run them as ONE launch (one grid, the members' channel ranges side by side), which saves the start-up and drain of
+ * the memory stream once per merged member; other cases run member by member.  The reference executes such sibling
+ * kernels one after the other (mindspore/lite/src/executor/sub_graph_kernel.cc:456-466; each is a
+ * MatmulBaseInt8CPUKernel::Run, LK/int8/matmul_base_int8.cc:530-570). */
+int mi_matmul_run_group(mi_matmul *const *handles, int32_t count, const int8_t *a_dev, int32_t rows,
+                        int8_t *const *c_dev, void *stream);
 /* Derived per-channel parameters (arrays of `col` entries, any may be NULL): multiplier / shifts, the folded bias
  * K*zx*zw - zx*sum(w) + bias, and the clamp bounds. */
 int mi_matmul_get_params(const mi_matmul *h, int32_t *multiplier, int32_t *left_shift, int32_t *right_shift,

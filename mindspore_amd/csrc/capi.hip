@@ -645,6 +645,58 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
   return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, Workspace::growable(&h->c_ws), s);
 }
 
+int mi_matmul_run_group(mi_matmul *const *handles, int32_t count, const int8_t *a_dev, int32_t rows,
+                        int8_t *const *c_dev, void *stream) {
+  if (handles == nullptr || a_dev == nullptr || c_dev == nullptr) {
+    set_error("mi_matmul_run_group: null argument");
+    return MI_NULL_PTR;
+  }
+  if (count < 1 || rows < 0) {
+    set_error("mi_matmul_run_group: count=%d rows=%d", count, rows);
+    return MI_PARAM_INVALID;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (handles[i] == nullptr || c_dev[i] == nullptr) {
+      set_error("mi_matmul_run_group: member %d is null", i);
+      return MI_NULL_PTR;
+    }
+    if (handles[i]->st.k != handles[0]->st.k) {
+      set_error("mi_matmul_run_group: member %d has deep %d, member 0 has %d", i, handles[i]->st.k, handles[0]->st.k);
+      return MI_PARAM_INVALID;
+    }
+  }
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  // the activation rows are brought into the kernels' form once, for all members
+  if ((rc = prepare_rows(a_dev, rows, handles[0]->st.k, Workspace::growable(&handles[0]->a_ws), s, &a, &lda, &k16)) != MI_OK)
+    return rc;
+  // decode-sized runs of up to four members go out as one launch; anything else runs member by member
+  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvMaxRows;
+  for (int i = 0; i < count && one_launch; ++i)
+    one_launch = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024 : handles[i]->st.w_blocked.p != nullptr;
+  if (one_launch) {
+    WeightView wv[4];
+    RequantParams rq[4];
+    int n[4];
+    for (int i = 0; i < count; ++i) {
+      const RequantState &st = handles[i]->st;
+      wv[i] = WeightView{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, static_cast<const int8_t *>(st.w_blocked.p)};
+      rq[i] = st.params();
+      n[i] = st.n;
+    }
+    return launch_gemv_group(a, lda, rows, k16, count, wv, n, rq, c_dev, s);
+  }
+  for (int i = 0; i < count; ++i)
+    if ((rc = run_requant_gemm(handles[i]->st, a, lda, rows, k16, c_dev[i], Workspace::growable(&handles[i]->c_ws), s)) != MI_OK)
+      return rc;
+  return MI_OK;
+}
+
 int mi_matmul_run_noalloc(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream) {
   if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
     set_error("mi_matmul_run_noalloc: null argument");

@@ -96,6 +96,11 @@ constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel (activations st
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
 
+// Up to four weight matrices with the same K against the same activation rows, as one launch (the grid is the
+// concatenation of the members' grids); member i writes c[i] with row stride n[i].
+int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *w, const int *n,
+                      const RequantParams *rq, int8_t *const *c, hipStream_t stream);
+
 // Per-device set-up of the skinny-M kernels (function attributes); called by mi_init with the device current.
 int gemv_prepare_device();
 

@@ -11,6 +11,7 @@
 #include "common.h"
 #include "quant_math.h"
 
+#include <algorithm>
 #include <type_traits>
 
 namespace mi {
@@ -56,12 +57,12 @@ struct GemvArgs {
 // ones): lanes past the end of a row re-read its last 16 bytes and chunks past the end of the stream re-read the
 // last chunk; both meet a zero activation fragment or are not accumulated.
 template <int M, int R, int D, bool DIRECT>
-__global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
+__device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantParams &rq, int block) {
   static_assert(D % R == 0, "the slot -> row mapping must be static");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   v4i *sa = reinterpret_cast<v4i *>(smem);  // [M][nseg * 64], zero past K
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_base = (blockIdx.x * 4 + wave) * R;
+  const int n_base = (block * 4 + wave) * R;
   const int nseg = (g.kchunks + 63) >> 6;
   const int kc_pad = nseg * 64;
   const int total = nseg * R;
@@ -193,6 +194,51 @@ __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams 
 }
 
 template <int M, int R, int D, bool DIRECT>
+__global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
+  gemv_i8_body<M, R, D, DIRECT>(g, rq, (int)blockIdx.x);
+}
+
+// Several weight matrices against the same activation rows in one launch (MatMuls that share their input, e.g. the
+// gate and up projections of a decoder layer): the grid is the concatenation of the members' grids, and a workgroup
+// first finds the member it belongs to.  Every field is picked with selects over constant indices, which keeps the
+// table in scalar registers (a dynamically indexed kernel argument would be copied to scratch memory).
+constexpr int kGemvGroupMax = 4;
+struct GemvGroup {
+  int count;
+  int block_end[kGemvGroupMax];  // exclusive prefix sums of the members' workgroup counts
+  GemvArgs g[kGemvGroupMax];
+  RequantParams rq[kGemvGroupMax];
+};
+
+__device__ __forceinline__ void pick_member(const GemvGroup &grp, int block, GemvArgs *g, RequantParams *rq,
+                                            int *local_block) {
+  int member = 0;
+#pragma unroll
+  for (int i = 1; i < kGemvGroupMax; ++i)
+    if (i < grp.count && block >= grp.block_end[i - 1]) member = i;
+  *g = grp.g[0];
+  *rq = grp.rq[0];
+  *local_block = block;
+#pragma unroll
+  for (int i = 1; i < kGemvGroupMax; ++i) {
+    if (member == i) {
+      *g = grp.g[i];
+      *rq = grp.rq[i];
+      *local_block = block - grp.block_end[i - 1];
+    }
+  }
+}
+
+template <int M, int R, int D, bool DIRECT>
+__global__ __launch_bounds__(256) void gemv_i8_group_kernel(GemvGroup grp) {
+  GemvArgs g;
+  RequantParams rq;
+  int block;
+  pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
+  gemv_i8_body<M, R, D, DIRECT>(g, rq, block);
+}
+
+template <int M, int R, int D, bool DIRECT>
 static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
   auto kern = gemv_i8_kernel<M, R, D, DIRECT>;
   // (more than 64 KiB of dynamic LDS needs the attribute that gemv_prepare_device set when the library was initialised)
@@ -204,9 +250,24 @@ static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t s
   return MI_OK;
 }
 
+template <int M, int R, int D, bool DIRECT>
+static int launch_group_mrdx(GemvGroup &grp, hipStream_t stream) {
+  const int lds_bytes = DIRECT ? 0 : M * ((grp.g[0].kchunks + 63) / 64) * 1024;
+  int blocks = 0;
+  for (int i = 0; i < grp.count; ++i) {
+    blocks += (grp.g[i].n + 4 * R - 1) / (4 * R);
+    grp.block_end[i] = blocks;
+  }
+  hipLaunchKernelGGL((gemv_i8_group_kernel<M, R, D, DIRECT>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 template <int M, int R, int D>
 static int allow_big_lds() {
   MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_kernel<M, R, D, false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_kernel<M, R, D, false>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   return MI_OK;
 }
@@ -226,6 +287,21 @@ template <int M, int R, int D>
 static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
   const int total = ((g.kchunks + 63) >> 6) * R;
   return total <= D ? launch_mrdx<M, R, D, true>(g, rq, stream) : launch_mrdx<M, R, D, false>(g, rq, stream);
+}
+
+template <int M, int R, int D>
+static int launch_group_mrd(GemvGroup &grp, hipStream_t stream) {
+  const int total = ((grp.g[0].kchunks + 63) >> 6) * R;
+  return total <= D ? launch_group_mrdx<M, R, D, true>(grp, stream) : launch_group_mrdx<M, R, D, false>(grp, stream);
+}
+
+template <int M>
+static int launch_group_m(GemvGroup &grp, hipStream_t stream) {  // same choice as launch_m: it depends on K only
+  const int nseg = (grp.g[0].kchunks + 63) >> 6;
+  if (nseg == 1) return launch_group_mrd<M, 4, 4>(grp, stream);
+  if (nseg == 2) return launch_group_mrd<M, 4, 8>(grp, stream);
+  if (nseg <= 4) return launch_group_mrd<M, 2, 8>(grp, stream);
+  return launch_group_mrd<M, 1, 12>(grp, stream);
 }
 
 template <int M>
@@ -254,12 +330,12 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 // (D x RG KiB of weights) in flight, and the partial sums meet in LDS.
 // =====================================================================================================================
 template <int RG, int D, int MG>
-__global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, RequantParams rq) {
+__device__ __forceinline__ void gemv_mfma_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
   constexpr int WAVES = 8;
   __shared__ v4i red[WAVES][(RG + 1) * MG][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane >> 4, idx = lane & 15;
-  const int n0 = blockIdx.x * (RG * 16);
+  const int n0 = block * (RG * 16);
   const int k_bytes = g.kchunks * 16;
   const int total = g.k_pad >> 6;  // 64-byte steps in a (zero padded) weight row
   const int spw = (total + WAVES - 1) / WAVES;
@@ -399,6 +475,32 @@ __global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, 
   }
 }
 
+template <int RG, int D, int MG>
+__global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, RequantParams rq) {
+  gemv_mfma_body<RG, D, MG>(g, m_rows, rq, (int)blockIdx.x);
+}
+
+template <int RG, int D, int MG>
+__global__ __launch_bounds__(512) void gemv_mfma_group_kernel(GemvGroup grp, int m_rows) {
+  GemvArgs g;
+  RequantParams rq;
+  int block;
+  pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
+  gemv_mfma_body<RG, D, MG>(g, m_rows, rq, block);
+}
+
+template <int RG, int D, int MG = 1>
+static int launch_group_mfma(GemvGroup &grp, int m, hipStream_t stream) {
+  int blocks = 0;
+  for (int i = 0; i < grp.count; ++i) {
+    blocks += (grp.g[i].n + RG * 16 - 1) / (RG * 16);
+    grp.block_end[i] = blocks;
+  }
+  hipLaunchKernelGGL((gemv_mfma_group_kernel<RG, D, MG>), dim3(blocks), dim3(512), 0, stream, grp, m);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 template <int RG, int D, int MG = 1>
 static int launch_mfma(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
   const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
@@ -428,27 +530,58 @@ int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t 
   return MI_OK;
 }
 
-int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n,
-                        const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
-  const int8_t *w = wv.w;
-  const int k_pad = wv.k_pad;
-  if (a == nullptr || w == nullptr || c == nullptr) {
+static int check_gemv_operands(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n, const int8_t *c) {
+  if (a == nullptr || wv.w == nullptr || c == nullptr) {
     set_error("gemv: null pointer");
     return MI_NULL_PTR;
   }
   if (m < 1 || m > kGemvMaxRows || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
-      k_pad % kKPad != 0 || k_pad < k || wv.ldw < k_pad || (wv.ldw & 15) != 0 ||
+      wv.k_pad % kKPad != 0 || wv.k_pad < k || wv.ldw < wv.k_pad || (wv.ldw & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
       (m <= kGemvDotRows && (int64_t)m * round_up(k, 1024) > 160 * 1024 - 1024)) {
     set_error("gemv: unsupported operand geometry m=%d n=%d k=%d lda=%lld", m, n, k, (long long)lda);
     return MI_PARAM_INVALID;
   }
+  if (m > kGemvDotRows && wv.blocked == nullptr) {
+    set_error("gemv: the blocked weight copy is missing");
+    return MI_NULL_PTR;
+  }
+  return MI_OK;
+}
+
+int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *wv, const int *n,
+                      const RequantParams *rq, int8_t *const *c, hipStream_t stream) {
+  if (count < 1 || count > kGemvGroupMax) {
+    set_error("gemv group: %d members (1..%d)", count, kGemvGroupMax);
+    return MI_PARAM_INVALID;
+  }
+  GemvGroup grp{};
+  grp.count = count;
+  int n_max = 0, k_pad_max = 0;
+  for (int i = 0; i < count; ++i) {
+    const int rc = check_gemv_operands(a, lda, m, k, wv[i], n[i], c[i]);
+    if (rc != MI_OK) return rc;
+    grp.g[i] = GemvArgs{a, lda, k / 16, m > kGemvDotRows ? wv[i].blocked : wv[i].w, wv[i].ldw, wv[i].k_pad, n[i], c[i], n[i]};
+    grp.rq[i] = rq[i];
+    n_max = std::max(n_max, n[i]);
+    k_pad_max = std::max(k_pad_max, wv[i].k_pad);
+  }
+  if (m > kGemvDotRows) {  // the same choices as for a single matrix, made for the group's largest member
+    const bool wide = n_max >= 8192 && k_pad_max <= 4096;
+    if (m > 16) return wide ? launch_group_mfma<2, 4, 2>(grp, m, stream) : launch_group_mfma<1, 8, 2>(grp, m, stream);
+    return wide ? launch_group_mfma<2, 4>(grp, m, stream) : launch_group_mfma<1, 8>(grp, m, stream);
+  }
+  return m == 1 ? launch_group_m<1>(grp, stream) : launch_group_m<2>(grp, stream);
+}
+
+int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n,
+                        const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
+  const int8_t *w = wv.w;
+  const int k_pad = wv.k_pad;
+  const int rc = check_gemv_operands(a, lda, m, k, wv, n, c);
+  if (rc != MI_OK) return rc;
   GemvArgs g{a, lda, k / 16, w, wv.ldw, k_pad, n, c, ldc};
   if (m > kGemvDotRows) {
-    if (wv.blocked == nullptr) {
-      set_error("gemv: the blocked weight copy is missing");
-      return MI_NULL_PTR;
-    }
     g.w = wv.blocked;
     // two 16-channel groups per workgroup (half the activation traffic) once there are enough channels to fill the
     // device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once

@@ -156,10 +156,25 @@ static int run_decode(int rows, int layers, int steps, int warmup) {
   hipEvent_t e0, e1;
   CHECK_HIP(hipEventCreate(&e0));
   CHECK_HIP(hipEventCreate(&e1));
+  // gate and up read the same activation: they go out through mi_matmul_run_group (one launch), as a provider
+  // would run sibling FullConnection nodes; NATIVE_BENCH_NO_GROUP=1 runs them one by one
+  const bool group = getenv("NATIVE_BENCH_NO_GROUP") == nullptr;
+  size_t launches = 0;
   auto step = [&]() -> int {
-    for (size_t i = 0; i < handles.size(); ++i) CHECK_MI(mi_matmul_run(handles[i], acts[i], rows, outs[i], st));
+    launches = 0;
+    for (size_t i = 0; i < handles.size(); ++i, ++launches) {
+      if (group && i % 5 == 2) {
+        mi_matmul *pair[2] = {handles[i], handles[i + 1]};
+        int8_t *out[2] = {outs[i], outs[i + 1]};
+        CHECK_MI(mi_matmul_run_group(pair, 2, acts[i], rows, out, st));
+        ++i;
+      } else {
+        CHECK_MI(mi_matmul_run(handles[i], acts[i], rows, outs[i], st));
+      }
+    }
     return 0;
   };
+  if (group) bytes -= (double)layers * rows * kDecode[3].k;  // the pair reads its activation rows once
   for (int i = 0; i < warmup; ++i)
     if (step()) return 1;
   CHECK_HIP(hipStreamSynchronize(st));
@@ -173,7 +188,7 @@ static int run_decode(int rows, int layers, int steps, int warmup) {
   const double ms_step = ms / steps;
   printf("{\"mode\": \"decode\", \"m\": %d, \"launches_per_step\": %zu, \"ms_per_step\": %.6f, \"us_per_launch\": %.3f, "
          "\"bytes_per_step\": %.0f, \"gbps\": %.1f}\n",
-         rows, handles.size(), ms_step, ms_step * 1e3 / handles.size(), bytes, bytes / (ms_step * 1e-3) / 1e9);
+         rows, launches, ms_step, ms_step * 1e3 / launches, bytes, bytes / (ms_step * 1e-3) / 1e9);
   for (auto *h : handles) mi_matmul_destroy(h);
   return 0;
 }

@@ -138,6 +138,23 @@ class FullconnectionInt8Kernel(MatmulInt8Kernel):
         super().__init__(weight, bias, in_quant, weight_quant, out_quant, True, act, device)
 
 
+def matmul_run_group(kernels, a, outs=None):
+    """Runs several MatmulInt8Kernel objects that share the input `a` (a contiguous CUDA int8 tensor [..., K]) as
+    mi_matmul_run_group does: decode-sized inputs go out as one launch.  Returns the list of outputs."""
+    import torch
+    L = _lib.load()
+    k = kernels[0].k
+    if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.shape[-1] != k:
+        raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % k)
+    rows = a.numel() // k
+    if outs is None:
+        outs = [torch.empty(a.shape[:-1] + (kn.n,), dtype=torch.int8, device=a.device) for kn in kernels]
+    hs = (C.c_void_p * len(kernels))(*[kn._h.value for kn in kernels])
+    cs = (C.c_void_p * len(kernels))(*[o.data_ptr() for o in outs])
+    _lib.check(L.mi_matmul_run_group(hs, len(kernels), a.data_ptr(), rows, cs, _stream()), "mi_matmul_run_group")
+    return outs
+
+
 class ConvolutionInt8Kernel(_Handle):
     """Conv2DFusion int8, NHWC.  weight [OC, KH, KW, IC] (group 1) or [C, KH, KW] (depthwise, group == C).
     pad = (up, down, left, right).  Raises MiError with code MI_NOT_SUPPORT for the cases a provider must decline.

@@ -14,7 +14,7 @@ ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
 EXPORTS = [
     "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_quantize_multiplier_single", "mi_activation_range", "mi_requant_params",
     "mi_multiply_by_quantized_multiplier",
-    "mi_matmul_create", "mi_matmul_reserve", "mi_matmul_run", "mi_matmul_run_noalloc", "mi_matmul_run_host", "mi_matmul_get_params", "mi_matmul_destroy",
+    "mi_matmul_create", "mi_matmul_reserve", "mi_matmul_run", "mi_matmul_run_noalloc", "mi_matmul_run_host", "mi_matmul_run_group", "mi_matmul_get_params", "mi_matmul_destroy",
     "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_reserve", "mi_conv_destroy",
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
     "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
@@ -108,6 +108,7 @@ def load():
     L.mi_matmul_reserve.argtypes = [vp, i32]
     L.mi_matmul_run.argtypes = [vp, vp, i32, vp, vp]
     L.mi_matmul_run_noalloc.argtypes = [vp, vp, i32, vp, vp]
+    L.mi_matmul_run_group.argtypes = [C.POINTER(vp), i32, vp, i32, C.POINTER(vp), vp]
     L.mi_matmul_run_host.argtypes = [vp, vp, i32, vp]
     L.mi_matmul_get_params.argtypes = [vp, vp, vp, vp, vp, pi32, pi32]
     L.mi_matmul_destroy.argtypes = [vp]

@@ -100,6 +100,33 @@ def test_matmul_whole_cu_tile_ragged(orc, m, n, k):
         assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("rows,k,ns", [(1, 4096, (1100, 900)), (2, 1040, (64, 260, 36)), (1, 144, (8, 4, 12, 20)),
+                                       (1, 11008, (300, 301)), (5, 4096, (256, 8200)), (8, 1040, (48, 16, 100)),
+                                       (17, 2048, (40, 520)), (32, 400, (33, 31, 64, 5)),
+                                       (40, 528, (96, 100)), (3, 64, (8, 8, 8, 8, 8))])
+def test_matmul_group_equals_member_by_member(orc, rows, k, ns):
+    """mi_matmul_run_group: members that share the input run as one launch (up to 32 rows, two to four members) or
+    one after the other (more rows, five members); every member's output is compared with the oracle.  Members differ
+    in width, quantisation granularity, weight zero points and activation."""
+    import torch
+    rng = np.random.default_rng(rows * 131 + k + sum(ns))
+    a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    sx, zx = float(rng.uniform(0.01, 0.05)), int(rng.integers(-20, 21))
+    cases, kerns = [], []
+    for i, n in enumerate(ns):
+        c = _mm_case(rng, rows, n, k, bool(i & 1), i % 3 == 2, i != 1, [0, 1, 3, 0][i % 4])
+        c.update(a=a, sx=sx, zx=zx)
+        cases.append(c)
+        kerns.append(K.MatmulInt8Kernel(c["w"], c["bias"], QP(sx, zx), _qps(c["sw"], c["zw"]), QP(c["so"], c["zo"]),
+                                        c["b_transpose"], c["act"]))
+    outs = K.matmul_run_group(kerns, torch.from_numpy(a).cuda())
+    torch.cuda.synchronize()
+    for i, c in enumerate(cases):
+        want = orc.matmul_int8(**c)
+        got = outs[i].cpu().numpy()
+        assert np.array_equal(got, want), (rows, k, ns, i, int((got != want).sum()))
+
+
 def test_matmul_generic_rounding_paths(orc):
     """Cases the fast epilogue must not take: real multiplier >= 1 (left shift), shift 0, huge bias (wrap)."""
     rng = np.random.default_rng(5)
