@@ -56,25 +56,35 @@ struct GemvArgs {
 // No weight load is predicated (a predicated load makes the compiler wait for earlier loads before issuing later
 // ones): lanes past the end of a row re-read its last 16 bytes and chunks past the end of the stream re-read the
 // last chunk; both meet a zero activation fragment or are not accumulated.
-template <int M, int R, int D, bool DIRECT>
+// KS = 2: two neighbouring waves share their R rows, each walks one half of K (long rows: twice the waves, each with
+// half the registers, so that more of them are resident), and the even wave adds the odd wave's sums through LDS.
+template <int M, int R, int D, bool DIRECT, int KS>
 __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantParams &rq, int block) {
   static_assert(D % R == 0, "the slot -> row mapping must be static");
+  static_assert(KS == 1 || KS == 2, "one or two waves per row group");
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  v4i *sa = reinterpret_cast<v4i *>(smem);  // [M][nseg * 64], zero past K
+  v4i *sa = reinterpret_cast<v4i *>(smem);  // [M][nseg_all * 64], zero past K
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n_base = (block * 4 + wave) * R;
-  const int nseg = (g.kchunks + 63) >> 6;
-  const int kc_pad = nseg * 64;
+  const int n_base = (block * (4 / KS) + wave / KS) * R;
+  const int nseg_all = (g.kchunks + 63) >> 6;
+  const int kc_pad = nseg_all * 64;
+  const int seg_per = (nseg_all + KS - 1) / KS;
+  const int seg0 = (wave % KS) * seg_per;                                   // this wave's K segments: seg0 ..
+  const int nseg = seg0 < nseg_all ? (seg_per < nseg_all - seg0 ? seg_per : nseg_all - seg0) : 0;  // .. seg0 + nseg
   const int total = nseg * R;
   const int last_off = (g.kchunks - 1) * 16;
   const int8_t *wrow = g.w + (int64_t)n_base * g.ldw;
 
+  // (a slot past the end of the stream -- only the looping form has such -- asks for the first 16 bytes of the
+  //  activation row, which are in the nearest cache, instead of pulling weight bytes through the memory system again)
   auto load_chunk = [&](int c) -> v4i {
-    c = c < total ? c : total - 1;
-    const int seg = c / R, rr = c % R;
+    const bool live = c < total;
+    c = live ? c : 0;
+    const int seg = seg0 + c / R, rr = c % R;
     int off = seg * 1024 + lane * 16;
     off = off < last_off ? off : last_off;
-    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wrow + (int64_t)rr * g.ldw + off));
+    const int8_t *p = live ? wrow + (int64_t)rr * g.ldw + off : g.a;
+    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p));
   };
   v4i buf[D];
 #pragma unroll
@@ -95,10 +105,10 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
     for (int sgi = 0; sgi < D / R; ++sgi)
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        const int chunk = sgi * 64 + lane;
+        const int chunk = (seg0 + sgi) * 64 + lane;
         const int cc = chunk < g.kchunks ? chunk : g.kchunks - 1;
         const v4i v = reinterpret_cast<const v4i *>(g.a + (int64_t)m * g.lda)[cc];
-        const bool live = chunk < g.kchunks;
+        const bool live = chunk < g.kchunks && sgi < nseg;
         apre[sgi][m].x = live ? v.x : 0;
         apre[sgi][m].y = live ? v.y : 0;
         apre[sgi][m].z = live ? v.z : 0;
@@ -141,7 +151,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
           if (DIRECT) {
             af[m] = apre[i / R][m];
           } else {
-            af[m] = seg < nseg ? sa[m * kc_pad + seg * 64 + lane] : z;
+            af[m] = seg < nseg ? sa[m * kc_pad + (seg0 + seg) * 64 + lane] : z;
           }
           if (rq.has_zw) {
             v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
@@ -172,6 +182,17 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
       }
     }
   }
+  if (KS == 2) {
+    __shared__ int halves[2][2][64];  // [row group of the workgroup][sum, activation sum][lane]
+    if (wave & 1) {
+      halves[wave >> 1][0][lane] = mine;
+      halves[wave >> 1][1][lane] = my_asum;
+    }
+    __syncthreads();
+    if (wave & 1) return;
+    mine += halves[wave >> 1][0][lane];
+    my_asum += halves[wave >> 1][1][lane];
+  }
   if (lane < R * M) {
     const int m = my_m, n = my_n;
     if (n < g.n) {
@@ -193,9 +214,9 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
   }
 }
 
-template <int M, int R, int D, bool DIRECT>
+template <int M, int R, int D, bool DIRECT, int KS>
 __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
-  gemv_i8_body<M, R, D, DIRECT>(g, rq, (int)blockIdx.x);
+  gemv_i8_body<M, R, D, DIRECT, KS>(g, rq, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activation rows in one launch (MatMuls that share their input, e.g. the
@@ -229,91 +250,99 @@ __device__ __forceinline__ void pick_member(const GemvGroup &grp, int block, Gem
   }
 }
 
-template <int M, int R, int D, bool DIRECT>
+template <int M, int R, int D, bool DIRECT, int KS>
 __global__ __launch_bounds__(256) void gemv_i8_group_kernel(GemvGroup grp) {
   GemvArgs g;
   RequantParams rq;
   int block;
   pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
-  gemv_i8_body<M, R, D, DIRECT>(g, rq, block);
+  gemv_i8_body<M, R, D, DIRECT, KS>(g, rq, block);
 }
 
-template <int M, int R, int D, bool DIRECT>
+template <int M, int R, int D, bool DIRECT, int KS>
 static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  auto kern = gemv_i8_kernel<M, R, D, DIRECT>;
+  auto kern = gemv_i8_kernel<M, R, D, DIRECT, KS>;
   // (more than 64 KiB of dynamic LDS needs the attribute that gemv_prepare_device set when the library was initialised)
   const int lds_bytes = DIRECT ? 0 : M * ((g.kchunks + 63) / 64) * 1024;
-  const int rows_per_block = 4 * R;
+  const int rows_per_block = 4 / KS * R;
   const int blocks = (g.n + rows_per_block - 1) / rows_per_block;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds_bytes, stream, g, rq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
 
-template <int M, int R, int D, bool DIRECT>
+template <int M, int R, int D, bool DIRECT, int KS>
 static int launch_group_mrdx(GemvGroup &grp, hipStream_t stream) {
   const int lds_bytes = DIRECT ? 0 : M * ((grp.g[0].kchunks + 63) / 64) * 1024;
   int blocks = 0;
   for (int i = 0; i < grp.count; ++i) {
-    blocks += (grp.g[i].n + 4 * R - 1) / (4 * R);
+    blocks += (grp.g[i].n + 4 / KS * R - 1) / (4 / KS * R);
     grp.block_end[i] = blocks;
   }
-  hipLaunchKernelGGL((gemv_i8_group_kernel<M, R, D, DIRECT>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
+  hipLaunchKernelGGL((gemv_i8_group_kernel<M, R, D, DIRECT, KS>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
 
-template <int M, int R, int D>
+template <int M>
 static int allow_big_lds() {
-  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_kernel<M, R, D, false>),
+  // the looping form stages the activation rows in dynamic LDS: up to 160 KiB
+  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_kernel<M, 1, 12, false, 1>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_kernel<M, R, D, false>),
+  MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_kernel<M, 1, 12, false, 1>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   return MI_OK;
 }
 
-// Once per device, from mi_init: the kernels that stage long activation rows in LDS may ask for up to 160 KiB.
+// Once per device, from mi_init.
 int gemv_prepare_device() {
   int rc;
-  if ((rc = allow_big_lds<1, 4, 4>()) != MI_OK || (rc = allow_big_lds<1, 4, 8>()) != MI_OK ||
-      (rc = allow_big_lds<1, 2, 8>()) != MI_OK || (rc = allow_big_lds<1, 1, 12>()) != MI_OK ||
-      (rc = allow_big_lds<2, 4, 4>()) != MI_OK || (rc = allow_big_lds<2, 4, 8>()) != MI_OK ||
-      (rc = allow_big_lds<2, 2, 8>()) != MI_OK || (rc = allow_big_lds<2, 1, 12>()) != MI_OK)
-    return rc;
+  if ((rc = allow_big_lds<1>()) != MI_OK || (rc = allow_big_lds<2>()) != MI_OK) return rc;
   return MI_OK;
 }
 
-template <int M, int R, int D>
-static int launch_mrd(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  const int total = ((g.kchunks + 63) >> 6) * R;
-  return total <= D ? launch_mrdx<M, R, D, true>(g, rq, stream) : launch_mrdx<M, R, D, false>(g, rq, stream);
-}
-
-template <int M, int R, int D>
-static int launch_group_mrd(GemvGroup &grp, hipStream_t stream) {
-  const int total = ((grp.g[0].kchunks + 63) >> 6) * R;
-  return total <= D ? launch_group_mrdx<M, R, D, true>(grp, stream) : launch_group_mrdx<M, R, D, false>(grp, stream);
+// Measured on MI355X: HBM streams fastest with many light waves that each have their whole share in flight at once
+// (a wave that loops needs >= 8-16 resident waves per CU to keep up), and a load slot that has no chunk of its own
+// still costs a request.  So rows per wave R and slots D are picked so that R x ceil(K / 1 KiB) == D exactly for
+// every K up to 12 KiB; longer rows loop over 12 slots with the activation rows staged in LDS.
+template <int M, typename F>
+static int with_config(int nseg, F &&f) {
+  using std::integral_constant;
+  typedef integral_constant<int, 1> one;
+  typedef integral_constant<int, 2> two;
+  switch (nseg) {  // f(R, D, DIRECT, KS)
+    case 1: return f(integral_constant<int, 4>(), integral_constant<int, 4>(), std::true_type(), one());
+    case 2: return f(integral_constant<int, 4>(), integral_constant<int, 8>(), std::true_type(), one());
+    case 3: return f(two(), integral_constant<int, 6>(), std::true_type(), one());
+    case 4: return f(two(), integral_constant<int, 8>(), std::true_type(), one());
+    case 5: return f(two(), integral_constant<int, 10>(), std::true_type(), one());
+    case 6: return f(two(), integral_constant<int, 12>(), std::true_type(), one());
+    // from here on the rows are long enough that one per wave would need 7+ KiB of slots plus as many activation
+    // registers: two waves per row, each with half of K
+    case 7:
+    case 8: return f(one(), integral_constant<int, 4>(), std::true_type(), two());
+    case 9:
+    case 10: return f(one(), integral_constant<int, 5>(), std::true_type(), two());
+    case 11:
+    case 12: return f(one(), integral_constant<int, 6>(), std::true_type(), two());
+    default: return f(one(), integral_constant<int, 12>(), std::false_type(), one());
+  }
 }
 
 template <int M>
-static int launch_group_m(GemvGroup &grp, hipStream_t stream) {  // same choice as launch_m: it depends on K only
-  const int nseg = (grp.g[0].kchunks + 63) >> 6;
-  if (nseg == 1) return launch_group_mrd<M, 4, 4>(grp, stream);
-  if (nseg == 2) return launch_group_mrd<M, 4, 8>(grp, stream);
-  if (nseg <= 4) return launch_group_mrd<M, 2, 8>(grp, stream);
-  return launch_group_mrd<M, 1, 12>(grp, stream);
+static int launch_group_m(GemvGroup &grp, hipStream_t stream) {  // the choice depends on K only
+  return with_config<M>((grp.g[0].kchunks + 63) >> 6, [&](auto r, auto d, auto direct, auto ks) {
+    return launch_group_mrdx<M, decltype(r)::value, decltype(d)::value, decltype(direct)::value, decltype(ks)::value>(
+        grp, stream);
+  });
 }
 
 template <int M>
 static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
-  // Measured on MI355X: HBM streams fastest with many light waves that each have their whole share in flight at
-  // once (a wave that loops needs >= 8-16 resident waves per CU to keep up).  So pick the rows per wave so that a
-  // wave's R x ceil(K / 1 KiB) chunks fit the in-flight budget, and fall back to looping for very long rows.
-  const int nseg = (g.kchunks + 63) >> 6;
-  if (nseg == 1) return launch_mrd<M, 4, 4>(g, rq, stream);
-  if (nseg == 2) return launch_mrd<M, 4, 8>(g, rq, stream);
-  if (nseg <= 4) return launch_mrd<M, 2, 8>(g, rq, stream);
-  return launch_mrd<M, 1, 12>(g, rq, stream);
+  return with_config<M>((g.kchunks + 63) >> 6, [&](auto r, auto d, auto direct, auto ks) {
+    return launch_mrdx<M, decltype(r)::value, decltype(d)::value, decltype(direct)::value, decltype(ks)::value>(
+        g, rq, stream);
+  });
 }
 
 // =====================================================================================================================
@@ -365,10 +394,13 @@ __device__ __forceinline__ void gemv_mfma_body(const GemvArgs &g, int m_rows, co
     }
   }
 
+  // (a step past this wave's slice or past the row asks for the first 16 bytes of an activation row, which are in
+  //  the nearest cache, instead of weight bytes that another wave streams or that do not exist)
   auto load_w = [&](int j, int rg) -> v4i {
-    int s = s0 + j;
-    s = s < total ? s : total - 1;
-    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wbase + ((int64_t)rg * total + s) * 1024));
+    const int s = s0 + j;
+    const bool live = j < spw && s < total;
+    const int8_t *p = live ? wbase + ((int64_t)rg * total + s) * 1024 : abase[0];
+    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p));
   };
   auto load_x = [&](int j, int mg) -> v4i {
     int off = (s0 + j) * 64 + grp * 16;

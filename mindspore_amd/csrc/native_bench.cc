@@ -193,6 +193,34 @@ static int run_decode(int rows, int layers, int steps, int warmup) {
   return 0;
 }
 
+// one shape, enough distinct copies that the memory-side cache cannot hold them, launched round robin
+static int run_shape(int n, int k, int rows, int steps, int warmup) {
+  const Shape sh{"shape", n, k};
+  const int copies = (int)(700e6 / ((double)n * k)) + 1;
+  std::vector<Matrix> ms(copies);
+  Rng rng{4242};
+  for (auto &m : ms)
+    if (make_matrix(sh, rows, &rng, &m)) return 1;
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  for (int i = 0; i < warmup * copies; ++i) CHECK_MI(mi_matmul_run(ms[i % copies].h, ms[i % copies].act, rows, ms[i % copies].out, st));
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps * copies; ++i) CHECK_MI(mi_matmul_run(ms[i % copies].h, ms[i % copies].act, rows, ms[i % copies].out, st));
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms_total = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms_total, e0, e1));
+  const double us = ms_total * 1e3 / (steps * copies);
+  printf("{\"mode\": \"shape\", \"n\": %d, \"k\": %d, \"m\": %d, \"copies\": %d, \"us\": %.3f, \"gbps\": %.1f}\n", n, k, rows, copies, us,
+         ms[0].bytes / (us * 1e-6) / 1e9);
+  for (auto &m : ms) mi_matmul_destroy(m.h);
+  return 0;
+}
+
 static int run_read(int mib, int steps, int warmup) {
   const size_t total = (size_t)3 << 30, slice = (size_t)mib << 20;
   const int nslices = (int)(total / slice);
@@ -220,10 +248,11 @@ static int run_read(int mib, int steps, int warmup) {
 
 int main(int argc, char **argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup>\n");
+    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup> | shape <n> <k> <rows> <steps> <warmup>\n");
     return 2;
   }
   CHECK_MI(mi_init(0));
+  if (strcmp(argv[1], "shape") == 0 && argc >= 7) return run_shape(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
   if (strcmp(argv[1], "decode") == 0 && argc >= 6) return run_decode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
   if (strcmp(argv[1], "warm") == 0 && argc >= 5) return run_warm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
   if (strcmp(argv[1], "read") == 0 && argc >= 5) return run_read(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));

@@ -67,12 +67,14 @@ def test_matmul_shapes(orc, m, n, k):
         assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
 
 
-@pytest.mark.parametrize("n,k", [(40, 2048), (24, 4000), (16, 5008), (9, 13008), (8200, 1040), (8196, 208)])
+@pytest.mark.parametrize("n,k", [(40, 2048), (24, 4000), (16, 5008), (9, 13008), (8200, 1040), (8196, 208),
+                                 (21, 2800), (18, 6144), (13, 7008), (11, 8192), (7, 9232), (10, 10240), (6, 11008),
+                                 (5, 12288)])
 def test_decode_rows_every_stream_shape(orc, n, k):
     """1..32 activation rows (v_dot4 kernel up to 2, matrix-core kernel above: one group of 16 rows up to 16, two
     groups up to 32) and the first row counts of the GEMM path, against every weight-stream shape the
-    skinny path distinguishes: rows of one, two, up to four and more 1 KiB segments, a stream longer than the
-    in-flight queue, few and many output channels."""
+    skinny path distinguishes: rows of one to six 1 KiB segments (whole rows per wave), seven to twelve (two waves
+    per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels."""
     rng = np.random.default_rng(n * 131 + k)
     orc.set_threads(16)
     for m in list(range(1, 19)) + [23, 31, 32, 33, 40]:
