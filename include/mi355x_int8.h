@@ -325,6 +325,13 @@ int mi_device_free(void *dev); /* NULL is allowed */
 int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream);
 int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream);
 int mi_stream_synchronize(void *stream);
+/* A HIP stream of the library's device (default priority, not ordered against the null stream) and its release.  A
+ * provider gives every session (every mindspore::Context it is handed) a stream of its own and passes it to all run
+ * and copy calls of that session, so that sessions running on different threads do not wait for one another: the
+ * part of the reference this stands for is the per-kernel thread-pool context each kernel executes under
+ * (mindspore/lite/src/executor/sub_graph_kernel.cc:456-466, InnerContext::thread_pool_). */
+int mi_stream_create(void **out_stream);
+int mi_stream_destroy(void *stream); /* NULL is allowed */
 
 #ifdef __cplusplus
 }

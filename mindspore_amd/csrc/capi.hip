@@ -526,6 +526,23 @@ int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *str
   return MI_OK;
 }
 
+int mi_stream_create(void **out_stream) {
+  if (out_stream == nullptr) return MI_NULL_PTR;
+  *out_stream = nullptr;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  hipStream_t s = nullptr;
+  MI_HIP_CHECK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority; independent of the null stream
+  *out_stream = s;
+  return MI_OK;
+}
+
+int mi_stream_destroy(void *stream) {
+  if (stream == nullptr) return MI_OK;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  MI_HIP_CHECK(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return MI_OK;
+}
+
 int mi_stream_synchronize(void *stream) {
   if (ensure_device() != MI_OK) return MI_ERROR;
   MI_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));

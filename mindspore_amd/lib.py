@@ -21,7 +21,7 @@ EXPORTS = [
     "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
     "mi_dynmm_destroy",
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
-    "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize",
+    "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize", "mi_stream_create", "mi_stream_destroy",
     "mi_host_malloc", "mi_host_free",
 ]
 # libmi355x_diag.so (include/mi355x_diag.h): the benchmark's measurement aids, not part of the product library
@@ -150,6 +150,8 @@ def load():
     L.mi_copy_to_device.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_copy_to_host.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_stream_synchronize.argtypes = [vp]
+    L.mi_stream_create.argtypes = [C.POINTER(vp)]
+    L.mi_stream_destroy.argtypes = [vp]
     _lib = L
     return L
 

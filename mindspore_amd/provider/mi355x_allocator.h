@@ -12,10 +12,14 @@
 // to a size-ordered free list and is reused for requests it fits without being more than 2^6 times too large
 // (shiftFactor_, inner_allocator.h), reference counts start at 0 and are -1 for pointers the allocator does not
 // know.  Blocks return to the system when the allocator is destroyed.  Thread safe.
+// The allocator initialises the library itself (a session may allocate tensors before any creator of the provider
+// has run, or run a model that has none of its operators); where page-locked memory cannot be had -- no GPU, no
+// gfx950 -- it hands out ordinary 64-byte-aligned memory, so that a CPU-only session keeps working.
 #ifndef MINDSPORE_AMD_PROVIDER_MI355X_ALLOCATOR_H_
 #define MINDSPORE_AMD_PROVIDER_MI355X_ALLOCATOR_H_
 #include <stddef.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include <map>
 #include <memory>
@@ -33,8 +37,8 @@ class PinnedAllocator : public Allocator {
   PinnedAllocator(const PinnedAllocator &) = delete;
   PinnedAllocator &operator=(const PinnedAllocator &) = delete;
   ~PinnedAllocator() override {
-    for (auto &it : allocated_) mi_host_free(it.first);
-    for (auto &it : free_) mi_host_free(it.second);
+    for (auto &it : allocated_) Release(it.first, it.second.pinned);
+    for (auto &it : free_) Release(it.second.ptr, it.second.pinned);
   }
 
   void *Malloc(size_t size) override {
@@ -42,14 +46,19 @@ class PinnedAllocator : public Allocator {
     std::lock_guard<std::mutex> lock(mutex_);
     auto it = free_.lower_bound(size);
     if (it != free_.end() && it->first <= (size >= (SIZE_MAX >> kReuseShift) ? SIZE_MAX : size << kReuseShift)) {
-      void *p = it->second;
-      allocated_[p] = Block{it->first, 0};
+      void *p = it->second.ptr;
+      allocated_[p] = Block{it->first, 0, it->second.pinned};
       free_.erase(it);
       return p;
     }
     void *p = nullptr;
-    if (mi_host_malloc(size, &p) != MI_OK) return nullptr;
-    allocated_[p] = Block{size, 0};
+    bool pinned = false;
+    if (LibraryUp() && mi_host_malloc(size, &p) == MI_OK) {
+      pinned = true;
+    } else if (posix_memalign(&p, 64, (size + 63) & ~size_t{63}) != 0) {
+      return nullptr;
+    }
+    allocated_[p] = Block{size, 0, pinned};
     return p;
   }
 
@@ -58,7 +67,7 @@ class PinnedAllocator : public Allocator {
     std::lock_guard<std::mutex> lock(mutex_);
     auto it = allocated_.find(ptr);
     if (it == allocated_.end()) return;  // not ours: nothing this allocator may release
-    free_.emplace(it->second.size, ptr);
+    free_.emplace(it->second.size, FreeBlock{ptr, it->second.pinned});
     allocated_.erase(it);
   }
 
@@ -71,8 +80,29 @@ class PinnedAllocator : public Allocator {
   struct Block {
     size_t size;
     int ref_count;
+    bool pinned;  // from mi_host_malloc (else from posix_memalign)
+  };
+  struct FreeBlock {
+    void *ptr;
+    bool pinned;
   };
   static constexpr int kReuseShift = 6;
+
+  // the same device choice as the provider's kernels make (MI355X_DEVICE, else device 0)
+  static bool LibraryUp() {
+    static const bool ok = [] {
+      const char *device = getenv("MI355X_DEVICE");
+      return mi_init(device != nullptr ? atoi(device) : 0) == MI_OK;
+    }();
+    return ok;
+  }
+  static void Release(void *p, bool pinned) {
+    if (pinned) {
+      mi_host_free(p);
+    } else {
+      free(p);
+    }
+  }
 
   template <typename F>
   int Update(void *ptr, F f) {
@@ -86,7 +116,7 @@ class PinnedAllocator : public Allocator {
 
   std::mutex mutex_;
   std::unordered_map<void *, Block> allocated_;
-  std::multimap<size_t, void *> free_;
+  std::multimap<size_t, FreeBlock> free_;
 };
 
 inline std::shared_ptr<Allocator> MakePinnedAllocator() { return std::make_shared<PinnedAllocator>(); }

@@ -3,9 +3,14 @@
 // This translation unit is the reference-side half of the drop-in boundary: it subclasses mindspore::kernel::Kernel
 // (include/api/kernel.h:29-55) and registers creators through registry::RegisterKernel
 // (mindspore/lite/include/registry/register_kernel.h:57-74) for MatMulFusion, FullConnection, Conv2DFusion (int8) and
-// DynamicQuant (float32), plus a kernel::KernelInterface (include/kernel_interface.h:29-59) for their shape inference
-// through registry::RegisterKernelInterface (include/registry/register_kernel_interface.h:36-75).  Everything below
-// the Kernel objects is the C ABI of include/mi355x_int8.h.
+// DynamicQuant (float32).  Everything below the Kernel objects is the C ABI of include/mi355x_int8.h.
+//
+// No kernel::KernelInterface is registered for these operator types, on purpose.  They are builtin types: when a
+// provider's interface answers, Scheduler::InferNodeShape returns before it creates the node's OpParameter
+// (mindspore/lite/src/litert/scheduler.cc:652-698), and a node that a creator below then declines can no longer fall
+// back to the builtin kernel (FindBackendKernel finds no OpParameter, :1178-1183) -- Model::Build would fail for
+// every fp32 convolution of the graph.  The builtin inference produces the same shapes (and the data types), and
+// ConvKernel::ReSize derives SAME-mode padding from the tensor shapes itself.
 //
 // It needs a MindSpore Lite SDK to compile (register_kernel.h includes the flatc-generated schema/model_generated.h)
 // and is therefore not part of the library build:
@@ -42,9 +47,7 @@
 #include "include/api/kernel.h"
 #include "include/api/status.h"
 #include "include/api/types.h"
-#include "include/kernel_interface.h"
 #include "include/registry/register_kernel.h"
-#include "include/registry/register_kernel_interface.h"
 #include "mi355x_int8.h"
 #include "schema/model_generated.h"
 
@@ -81,13 +84,32 @@ void FilterQuant(const MSTensor &w, std::vector<double> *scales, std::vector<int
 
 int ToStatus(int mi_code) { return mi_code == MI_OK ? static_cast<int>(kSuccess) : static_cast<int>(kLiteError); }
 
-int64_t RowsOf(const MSTensor &t) {
-  const auto shape = t.Shape();
+}  // namespace
+
+// One HIP stream per session: every kernel of a session is handed the same mindspore::Context, and everything it
+// launches or copies goes to that session's stream, so that sessions running on different threads neither share a
+// queue nor wait for each other's copies.  Streams live as long as the process (a provider is never told that a
+// session ended).
+void *SessionStream(const Context *ctx) {
+  static std::mutex *mutex = new std::mutex;
+  static std::map<const Context *, void *> *streams = new std::map<const Context *, void *>;
+  std::lock_guard<std::mutex> lock(*mutex);
+  auto it = streams->find(ctx);
+  if (it != streams->end()) return it->second;
+  void *stream = nullptr;
+  if (mi_stream_create(&stream) != MI_OK) stream = nullptr;  // the null stream still works, only without overlap
+  (*streams)[ctx] = stream;
+  return stream;
+}
+
+// Rows of a MatMul / FullConnection: the product of the output's leading dimensions, as the reference kernels take
+// it (fullconnection_int8.cc:49-58, which also covers use_axis; matmul_int8.cc InitParameter).
+int64_t RowsOfOutput(const MSTensor &out) {
+  const auto shape = out.Shape();
   int64_t rows = 1;
   for (size_t i = 0; i + 1 < shape.size(); ++i) rows *= shape[i];
   return rows;
 }
-}  // namespace
 
 // Device addresses this provider has published on tensors.  GetDeviceData() of an input is trusted only when it is
 // one of them: an application may have attached memory of some other device to a graph input.
@@ -152,8 +174,9 @@ class DeviceBuffer {
 // this provider left it there, uploaded otherwise) and hand the output on.
 class DeviceIo {
  public:
-  // reads [mi355x] device_only_outputs for the given output tensor
-  void Configure(const std::map<std::string, std::string> &section, const std::string &output_name) {
+  // the session's stream, and [mi355x] device_only_outputs for the given output tensor
+  void Configure(void *stream, const std::map<std::string, std::string> &section, const std::string &output_name) {
+    stream_ = stream;
     const auto it = section.find("device_only_outputs");
     if (it == section.end()) return;
     const std::string &list = it->second;
@@ -177,7 +200,8 @@ class DeviceIo {
     const size_t bytes = t->DataSize();
     if (host == nullptr || bytes == 0) return nullptr;
     void *staged = in_.Reserve(bytes);
-    if (staged == nullptr || mi_copy_to_device(staged, host.get(), bytes, nullptr) != MI_OK) return nullptr;
+    // (returns once the bytes have left the host buffer: the runtime may recycle it as soon as Execute returns)
+    if (staged == nullptr || mi_copy_to_device(staged, host.get(), bytes, stream_) != MI_OK) return nullptr;
     return staged;
   }
 
@@ -187,15 +211,17 @@ class DeviceIo {
     return p;
   }
 
-  // after the launch: publish the device address; copy to the host unless the output was declared device-only
+  // after the launch: publish the device address; copy to the host unless the output was declared device-only (the
+  // copy waits for this session's stream only; a device-only output is ordered by the stream itself)
   int Deliver(MSTensor *t) {
     t->SetDeviceData(out_.get());
     if (!host_copy_) return kSuccess;
     void *host = t->MutableData();
     if (host == nullptr) return kLiteNullptr;
-    return mi_copy_to_host(host, out_.get(), t->DataSize(), nullptr) == MI_OK ? static_cast<int>(kSuccess)
-                                                                              : static_cast<int>(kLiteError);
+    return mi_copy_to_host(host, out_.get(), t->DataSize(), stream_) == MI_OK ? static_cast<int>(kSuccess)
+                                                                               : static_cast<int>(kLiteError);
   }
+  void *stream() const { return stream_; }
 
   void Withdraw(MSTensor *t) {
     if (t->GetDeviceData() == out_.get()) t->SetDeviceData(nullptr);
@@ -204,6 +230,7 @@ class DeviceIo {
  private:
   DeviceBuffer in_, out_;
   bool host_copy_ = true;
+  void *stream_ = nullptr;
 };
 
 // ---- MatMulFusion / FullConnection, int8 in -> int8 out (full quant) or fp32 out (dynamic quant) ----------------
@@ -219,12 +246,13 @@ class MatmulKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
     const MSTensor &w = inputs_[kWeightIndex];
     const auto wshape = w.Shape();
     if (wshape.size() != 2 || w.Data() == nullptr) return kLiteError;
     const int32_t n = static_cast<int32_t>(b_transpose_ ? wshape[0] : wshape[1]);
     const int32_t k = static_cast<int32_t>(b_transpose_ ? wshape[1] : wshape[0]);
+    k_ = k;
     std::vector<double> scales;
     std::vector<int32_t> zps;
     FilterQuant(w, &scales, &zps);
@@ -245,20 +273,21 @@ class MatmulKernel : public kernel::Kernel {
   int ReSize() override { return kSuccess; }  // the row count is read from the input tensor at every Execute
 
   int Execute() override {
-    const int32_t rows = static_cast<int32_t>(RowsOf(inputs_[0]));
+    const int32_t rows = static_cast<int32_t>(RowsOfOutput(outputs_[0]));
     if (rows == 0) return kSuccess;
+    if (inputs_[0].ElementNum() != static_cast<int64_t>(rows) * k_) return kLiteError;
     const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
     void *c = io_.Output(outputs_[0].DataSize());
     if (a == nullptr || c == nullptr) return kLiteNullptr;
     int rc = MI_ERROR;
     if (full_ != nullptr) {
-      rc = mi_matmul_run(full_, a, rows, static_cast<int8_t *>(c), nullptr);
+      rc = mi_matmul_run(full_, a, rows, static_cast<int8_t *>(c), io_.stream());
     } else {
       // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
       // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
       const auto iqs = inputs_[0].QuantParams();
       if (iqs.size() == 1) {
-        rc = mi_dynmm_run(dyn_, a, rows, iqs[0].scale, iqs[0].zero_point, static_cast<float *>(c), nullptr);
+        rc = mi_dynmm_run(dyn_, a, rows, iqs[0].scale, iqs[0].zero_point, static_cast<float *>(c), io_.stream());
       } else {
         // one scale per row (input_per_channel_, :152-171), narrowed to float (:168-171); the zero point used is
         // the first one (matmul_dynamic_int8.cc:61)
@@ -269,8 +298,9 @@ class MatmulKernel : public kernel::Kernel {
         }
         const size_t bytes = ps.size() * sizeof(mi_dq_params);
         void *dev = row_params_.Reserve(bytes);
-        if (dev == nullptr || mi_copy_to_device(dev, ps.data(), bytes, nullptr) != MI_OK) return kLiteError;
-        rc = mi_dynmm_run_rows(dyn_, a, rows, static_cast<const mi_dq_params *>(dev), static_cast<float *>(c), nullptr);
+        if (dev == nullptr || mi_copy_to_device(dev, ps.data(), bytes, io_.stream()) != MI_OK) return kLiteError;
+        rc = mi_dynmm_run_rows(dyn_, a, rows, static_cast<const mi_dq_params *>(dev), static_cast<float *>(c),
+                               io_.stream());
       }
     }
     return rc == MI_OK ? io_.Deliver(&outputs_[0]) : static_cast<int>(kLiteError);
@@ -279,6 +309,7 @@ class MatmulKernel : public kernel::Kernel {
  private:
   bool b_transpose_;
   int act_;
+  int32_t k_ = 0;
   mi_matmul *full_ = nullptr;
   mi_dynmm *dyn_ = nullptr;
   DeviceIo io_;
@@ -291,7 +322,8 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
   bool b_transpose = true;
   int act = 0;
   if (const auto *fc = prim->value_as_FullConnection()) {  // weight is always [N, K] (fullconnection_int8.cc:33-34)
-    if (fc->use_axis()) return nullptr;
+    // use_axis only changes how the input's dimensions fold into rows x K, which the kernel takes from the output
+    // shape and the weight exactly as the reference does (fullconnection_int8.cc:49-58)
     act = fc->activation_type();
   } else if (const auto *mm = prim->value_as_MatMulFusion()) {
     if (mm->transpose_a()) return nullptr;
@@ -311,6 +343,24 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
     const auto want = out_i8 ? DataType::kNumberTypeInt32 : DataType::kNumberTypeFloat32;
     if (!in[kBiasIndex].IsConst() || in[kBiasIndex].DataType() != want) return nullptr;
   }
+  // everything Prepare / Execute would otherwise fail on is screened here, where declining still lets the scheduler
+  // fall back: the activation type, quant parameters present and of a usable count, the contraction length
+  // (a dynamic-quant MatMul finds its input's scale on the tensor only at run time: DynamicQuant writes it there)
+  if (in[0].DataType() != DataType::kNumberTypeInt8) return nullptr;
+  const auto wshape = w.Shape();
+  const int64_t n = b_transpose ? wshape[0] : wshape[1], k = b_transpose ? wshape[1] : wshape[0];
+  const size_t nfilter = w.QuantParams().size();
+  if (n <= 0 || k <= 0 || (nfilter != 1 && nfilter != static_cast<size_t>(n))) return nullptr;
+  const auto ashape = in[0].Shape();
+  bool known = !ashape.empty();
+  int64_t elements = 1;
+  for (int64_t d : ashape) {
+    known = known && d >= 0;
+    elements *= d;
+  }
+  if (known) {
+    if (prim->value_as_MatMulFusion() != nullptr ? ashape.back() != k : elements % k != 0) return nullptr;
+  }
   return std::make_shared<MatmulKernel>(in, out, prim, ctx, b_transpose, act);
 }
 
@@ -324,7 +374,7 @@ class ConvKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
     return Build();
   }
 
@@ -348,7 +398,7 @@ class ConvKernel : public kernel::Kernel {
     auto *y = static_cast<int8_t *>(io_.Output(outputs_[0].DataSize()));
     if (x == nullptr || y == nullptr) return kLiteNullptr;
     if (mi_conv_run(conv_, x, static_cast<int32_t>(s[0]), static_cast<int32_t>(s[1]), static_cast<int32_t>(s[2]), y,
-                    nullptr) != MI_OK) {
+                    io_.stream()) != MI_OK) {
       return kLiteError;
     }
     return io_.Deliver(&outputs_[0]);
@@ -423,11 +473,13 @@ std::shared_ptr<kernel::Kernel> ConvCreator(const std::vector<MSTensor> &in, con
   if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || out[0].DataType() != DataType::kNumberTypeInt8) {
     return nullptr;
   }
-  if (!PerTensor(in[0]) || !PerTensor(out[0])) return nullptr;
+  if (in[0].DataType() != DataType::kNumberTypeInt8 || !PerTensor(in[0]) || !PerTensor(out[0])) return nullptr;
   if (in.size() > kBiasIndex &&
       (!in[kBiasIndex].IsConst() || in[kBiasIndex].DataType() != DataType::kNumberTypeInt32)) {
     return nullptr;
   }
+  const size_t nfilter = w.QuantParams().size();  // per tensor or one per output channel (convolution_base.cc:377-397)
+  if (cv->out_channel() <= 0 || (nfilter != 1 && nfilter != static_cast<size_t>(cv->out_channel()))) return nullptr;
   const int64_t kh = cv->kernel_size()->Get(0), kw = cv->kernel_size()->Get(1);
   const bool depthwise = cv->group() > 1 && cv->group() == cv->in_channel() && cv->group() == cv->out_channel();
   if (cv->group() != 1 && !depthwise) return nullptr;
@@ -451,7 +503,7 @@ class DynamicQuantKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
     const auto *p = primitive_->value_as_DynamicQuant();
     per_row_ = p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0;
     return ToStatus(mi_dynquant_create(p->symmetric() ? 1 : 0, &dq_));
@@ -470,8 +522,8 @@ class DynamicQuantKernel : public kernel::Kernel {
       std::vector<mi_dq_params> ps(static_cast<size_t>(segments));
       const size_t bytes = ps.size() * sizeof(mi_dq_params);
       auto *dev = static_cast<mi_dq_params *>(row_params_.Reserve(bytes));
-      if (dev == nullptr || mi_dynquant_run_segments(dq_, x, segments, unit, q, dev, nullptr) != MI_OK ||
-          mi_copy_to_host(ps.data(), dev, bytes, nullptr) != MI_OK) {
+      if (dev == nullptr || mi_dynquant_run_segments(dq_, x, segments, unit, q, dev, io_.stream()) != MI_OK ||
+          mi_copy_to_host(ps.data(), dev, bytes, io_.stream()) != MI_OK) {
         return kLiteError;
       }
       std::vector<QuantParam> qps(ps.size());
@@ -486,7 +538,8 @@ class DynamicQuantKernel : public kernel::Kernel {
       return io_.Deliver(&outputs_[0]);
     }
     mi_dq_params p{};
-    if (mi_dynquant_run(dq_, x, n, q, nullptr) != MI_OK || mi_dynquant_get_params(dq_, nullptr, &p) != MI_OK) {
+    if (mi_dynquant_run(dq_, x, n, q, io_.stream()) != MI_OK ||
+        mi_dynquant_get_params(dq_, io_.stream(), &p) != MI_OK) {
       return kLiteError;
     }
     // what DynamicQuantCPUKernel::CalculatePerlayerScaleZp publishes on the output tensor (dynamic_quant.cc:156-186)
@@ -530,96 +583,6 @@ std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> 
   return std::make_shared<DynamicQuantKernel>(in, out, prim, ctx);
 }
 
-// ---- shape inference -----------------------------------------------------------------------------------------------
-// Lite asks a provider's KernelInterface before its builtin inference (infer_manager.cc:90-145).  Output shapes come
-// from the library's mi_infer_* functions, which reproduce nnacl's results; data types stay as the model file has
-// them (a provider cannot see CNode.quantType, which is what makes the builtin MatMul inference switch a
-// dynamic-quant output to float32, matmul_infer.c:137-139).
-class ShapeInference : public kernel::KernelInterface {
- public:
-  Status Infer(std::vector<MSTensor> *inputs, std::vector<MSTensor> *outputs,
-               const schema::Primitive *primitive) override {
-    if (inputs == nullptr || outputs == nullptr || primitive == nullptr || inputs->empty() || outputs->size() != 1) {
-      return kLiteInferError;
-    }
-    const auto dims = [](const MSTensor &t) {
-      std::vector<int32_t> v;
-      for (int64_t d : t.Shape()) v.push_back(static_cast<int32_t>(d));
-      return v;
-    };
-    int32_t out[MI_MAX_DIMS] = {0};
-    int32_t out_dims = 0;
-    int ret = MI_INFER_ERR;
-    const size_t n = inputs->size();
-    const std::vector<int32_t> a = dims((*inputs)[0]);
-    const std::vector<int32_t> b = n > 1 ? dims((*inputs)[1]) : std::vector<int32_t>();
-    const std::vector<int32_t> bias = n > 2 ? dims((*inputs)[2]) : std::vector<int32_t>();
-    if (a.size() > MI_MAX_DIMS || b.size() > MI_MAX_DIMS || bias.size() > MI_MAX_DIMS) return kLiteInferError;
-    switch (primitive->value_type()) {
-      case schema::PrimitiveType_MatMulFusion: {
-        const auto *mm = primitive->value_as_MatMulFusion();
-        if (mm == nullptr || (n != 2 && n != 3)) return kLiteInferError;
-        ret = mi_infer_matmul(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()),
-                              bias.data(), static_cast<int32_t>(bias.size()), mm->transpose_a(), mm->transpose_b(), out,
-                              &out_dims);
-        break;
-      }
-      case schema::PrimitiveType_FullConnection: {
-        const auto *fc = primitive->value_as_FullConnection();
-        if (fc == nullptr || n < 2) return kLiteInferError;
-        ret = mi_infer_fullconnection(a.data(), static_cast<int32_t>(a.size()), b.data(),
-                                      static_cast<int32_t>(b.size()), bias.data(), static_cast<int32_t>(bias.size()),
-                                      fc->has_bias(), fc->use_axis(), static_cast<int32_t>(fc->axis()), out, &out_dims);
-        break;
-      }
-      case schema::PrimitiveType_Conv2DFusion: {
-        const auto *cv = primitive->value_as_Conv2DFusion();
-        if (cv == nullptr || (n != 2 && n != 3)) return kLiteInferError;
-        // attribute defaults as the builtin populate step fills them (ops/populate/conv2d_populate.cc)
-        mi_conv_infer p{};
-        const auto at = [](const flatbuffers::Vector<int64_t> *v, uint32_t i, int32_t dflt) {
-          return v != nullptr && v->size() > i ? static_cast<int32_t>(v->Get(i)) : dflt;
-        };
-        p.kernel_h = at(cv->kernel_size(), 0, -1);
-        p.kernel_w = at(cv->kernel_size(), 1, -1);
-        p.stride_h = at(cv->stride(), 0, 1);
-        p.stride_w = at(cv->stride(), 1, 1);
-        p.dilation_h = at(cv->dilation(), 0, 1);
-        p.dilation_w = at(cv->dilation(), 1, 1);
-        p.pad_mode = cv->pad_mode() == schema::PadMode_SAME    ? MI_PAD_SAME
-                     : cv->pad_mode() == schema::PadMode_VALID ? MI_PAD_VALID
-                                                               : MI_PAD_EXPLICIT;
-        const bool has_pads = cv->pad_list() != nullptr && cv->pad_list()->size() >= 4;
-        p.pad_u = has_pads ? at(cv->pad_list(), 0, 0) : 0;
-        p.pad_d = has_pads ? at(cv->pad_list(), 1, 0) : 0;
-        p.pad_l = has_pads ? at(cv->pad_list(), 2, 0) : 0;
-        p.pad_r = has_pads ? at(cv->pad_list(), 3, 0) : 0;
-        p.group = static_cast<int32_t>(cv->group());
-        ret = mi_infer_conv2d(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()), &p,
-                              out, &out_dims);
-        break;
-      }
-      case schema::PrimitiveType_DynamicQuant: {  // same shape as the input (dynamic_quant_infer.c:21-40)
-        for (int32_t d : a) {
-          if (d < 0) return kLiteInferInvalid;
-        }
-        (*outputs)[0].SetFormat((*inputs)[0].format());
-        (*outputs)[0].SetShape((*inputs)[0].Shape());
-        return kSuccess;
-      }
-      default:
-        return kLiteInferError;
-    }
-    (*outputs)[0].SetFormat((*inputs)[0].format());
-    if (ret == MI_INFER_INVALID) return kLiteInferInvalid;
-    if (ret != MI_OK) return kLiteInferError;
-    (*outputs)[0].SetShape(std::vector<int64_t>(out, out + out_dims));
-    return kSuccess;
-  }
-};
-
-std::shared_ptr<kernel::KernelInterface> ShapeInferenceCreator() { return std::make_shared<ShapeInference>(); }
-
 // ---- registration: arch "CPU" for applications, arch "" for the stock benchmark tool --------------------------------
 namespace {
 struct Registrar {
@@ -633,10 +596,6 @@ struct Registrar {
                                           ConvCreator);
       registry::RegisterKernel::RegKernel(arch, "mi355x", DataType::kNumberTypeFloat32,
                                           schema::PrimitiveType_DynamicQuant, DynamicQuantCreator);
-    }
-    for (int op : {schema::PrimitiveType_MatMulFusion, schema::PrimitiveType_FullConnection,
-                   schema::PrimitiveType_Conv2DFusion, schema::PrimitiveType_DynamicQuant}) {
-      registry::RegisterKernelInterface::Reg("mi355x", op, ShapeInferenceCreator);
     }
   }
 } g_registrar;

@@ -13,7 +13,7 @@ REFERENCE = "/root/reference"
 def build_harness():
     os.makedirs(os.path.dirname(OUT), exist_ok=True)
     subprocess.check_call([
-        "g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-Wall", "-I" + HERE, "-I" + os.path.join(ROOT, "include"),
+        "g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-pthread", "-Wall", "-I" + HERE, "-I" + os.path.join(ROOT, "include"),
         os.path.join(HERE, "harness.cc"), "-L" + os.path.join(ROOT, "mindspore_amd"), "-lmi355x_int8",
         "-Wl,-rpath,$ORIGIN/../../../mindspore_amd", "-o", OUT])
     return OUT

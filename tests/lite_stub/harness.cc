@@ -1,8 +1,10 @@
 // TEST INFRASTRUCTURE.  Plays the part of the Lite scheduler for mindspore_amd/provider/mi355x_provider.cc, compiled
-// against the stand-in API of this directory: looks the creator up by (arch, provider, data type, op type) as
-// scheduler.cc:1131-1177 does, runs the provider's shape inference, Prepare / ReSize / Execute, and hands tensors in
-// and out through a C interface for the Python tests.  The provider source is included, so its static registrar
-// runs when this library is loaded.
+// against the stand-in API of this directory: infers the node's shape (through a provider's KernelInterface when one
+// is registered for the operator, else through the stand-in for the builtin inference below -- and, as
+// Scheduler::InferNodeShape does, only the builtin path leaves the node an OpParameter, scheduler.cc:652-698), looks
+// the creator up by (arch, provider, data type, op type) as scheduler.cc:1131-1177 does, runs Prepare / ReSize /
+// Execute, and hands tensors in and out through a C interface for the Python tests.  The provider source is
+// included, so its static registrar runs when this library is loaded.
 #include <string.h>
 
 #include <map>
@@ -10,8 +12,12 @@
 #include <string>
 #include <vector>
 
+#include <thread>
+
 #include "../../mindspore_amd/provider/mi355x_allocator.h"
 #include "../../mindspore_amd/provider/mi355x_provider.cc"
+#include "include/kernel_interface.h"
+#include "include/registry/register_kernel_interface.h"
 
 using mindspore::MSTensor;
 namespace schema = mindspore::schema;
@@ -44,14 +50,108 @@ typedef struct ph_op {
 }
 
 namespace {
-enum Stage { kOk = 0, kNoCreator = 1, kDeclined = 2, kInferFailed = 3, kPrepareFailed = 4, kResizeFailed = 5, kExecuteFailed = 6 };
+// kDeclined: the creator returned nullptr and the node has an OpParameter, i.e. the scheduler now takes the builtin CPU
+// kernel.  kDeclinedNoFallback: it returned nullptr after a provider's KernelInterface had inferred the node, so that
+// there is no OpParameter and FindBackendKernel gives up (scheduler.cc:1178-1183): Model::Build fails.
+enum Stage { kOk = 0, kNoCreator = 1, kDeclined = 2, kInferFailed = 3, kPrepareFailed = 4, kResizeFailed = 5, kExecuteFailed = 6,
+             kDeclinedNoFallback = 7 };
+
+// Stand-in for the builtin (nnacl) shape inference of the four operator types: output shapes from the library's
+// mi_infer_* functions, which tests/test_infer_shape.py checks against the compiled nnacl functions.
+class BuiltinInference : public mindspore::kernel::KernelInterface {
+ public:
+  mindspore::Status Infer(std::vector<MSTensor> *inputs, std::vector<MSTensor> *outputs,
+               const schema::Primitive *primitive) override {
+    if (inputs == nullptr || outputs == nullptr || primitive == nullptr || inputs->empty() || outputs->size() != 1) {
+      return mindspore::kLiteInferError;
+    }
+    const auto dims = [](const MSTensor &t) {
+      std::vector<int32_t> v;
+      for (int64_t d : t.Shape()) v.push_back(static_cast<int32_t>(d));
+      return v;
+    };
+    int32_t out[MI_MAX_DIMS] = {0};
+    int32_t out_dims = 0;
+    int ret = MI_INFER_ERR;
+    const size_t n = inputs->size();
+    const std::vector<int32_t> a = dims((*inputs)[0]);
+    const std::vector<int32_t> b = n > 1 ? dims((*inputs)[1]) : std::vector<int32_t>();
+    const std::vector<int32_t> bias = n > 2 ? dims((*inputs)[2]) : std::vector<int32_t>();
+    if (a.size() > MI_MAX_DIMS || b.size() > MI_MAX_DIMS || bias.size() > MI_MAX_DIMS) return mindspore::kLiteInferError;
+    switch (primitive->value_type()) {
+      case schema::PrimitiveType_MatMulFusion: {
+        const auto *mm = primitive->value_as_MatMulFusion();
+        if (mm == nullptr || (n != 2 && n != 3)) return mindspore::kLiteInferError;
+        ret = mi_infer_matmul(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()),
+                              bias.data(), static_cast<int32_t>(bias.size()), mm->transpose_a(), mm->transpose_b(), out,
+                              &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_FullConnection: {
+        const auto *fc = primitive->value_as_FullConnection();
+        if (fc == nullptr || n < 2) return mindspore::kLiteInferError;
+        ret = mi_infer_fullconnection(a.data(), static_cast<int32_t>(a.size()), b.data(),
+                                      static_cast<int32_t>(b.size()), bias.data(), static_cast<int32_t>(bias.size()),
+                                      fc->has_bias(), fc->use_axis(), static_cast<int32_t>(fc->axis()), out, &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_Conv2DFusion: {
+        const auto *cv = primitive->value_as_Conv2DFusion();
+        if (cv == nullptr || (n != 2 && n != 3)) return mindspore::kLiteInferError;
+        // attribute defaults as the builtin populate step fills them (ops/populate/conv2d_populate.cc)
+        mi_conv_infer p{};
+        const auto at = [](const flatbuffers::Vector<int64_t> *v, uint32_t i, int32_t dflt) {
+          return v != nullptr && v->size() > i ? static_cast<int32_t>(v->Get(i)) : dflt;
+        };
+        p.kernel_h = at(cv->kernel_size(), 0, -1);
+        p.kernel_w = at(cv->kernel_size(), 1, -1);
+        p.stride_h = at(cv->stride(), 0, 1);
+        p.stride_w = at(cv->stride(), 1, 1);
+        p.dilation_h = at(cv->dilation(), 0, 1);
+        p.dilation_w = at(cv->dilation(), 1, 1);
+        p.pad_mode = cv->pad_mode() == schema::PadMode_SAME    ? MI_PAD_SAME
+                     : cv->pad_mode() == schema::PadMode_VALID ? MI_PAD_VALID
+                                                               : MI_PAD_EXPLICIT;
+        const bool has_pads = cv->pad_list() != nullptr && cv->pad_list()->size() >= 4;
+        p.pad_u = has_pads ? at(cv->pad_list(), 0, 0) : 0;
+        p.pad_d = has_pads ? at(cv->pad_list(), 1, 0) : 0;
+        p.pad_l = has_pads ? at(cv->pad_list(), 2, 0) : 0;
+        p.pad_r = has_pads ? at(cv->pad_list(), 3, 0) : 0;
+        p.group = static_cast<int32_t>(cv->group());
+        ret = mi_infer_conv2d(a.data(), static_cast<int32_t>(a.size()), b.data(), static_cast<int32_t>(b.size()), &p,
+                              out, &out_dims);
+        break;
+      }
+      case schema::PrimitiveType_DynamicQuant: {  // same shape as the input (dynamic_quant_infer.c:21-40)
+        for (int32_t d : a) {
+          if (d < 0) return mindspore::kLiteInferInvalid;
+        }
+        (*outputs)[0].SetFormat((*inputs)[0].format());
+        (*outputs)[0].SetShape((*inputs)[0].Shape());
+        return mindspore::kSuccess;
+      }
+      default:
+        return mindspore::kLiteInferError;
+    }
+    (*outputs)[0].SetFormat((*inputs)[0].format());
+    if (ret == MI_INFER_INVALID) return mindspore::kLiteInferInvalid;
+    if (ret != MI_OK) return mindspore::kLiteInferError;
+    (*outputs)[0].SetShape(std::vector<int64_t>(out, out + out_dims));
+    return mindspore::kSuccess;
+  }
+};
+
+
+
 
 struct Session {
   schema::Primitive prim;
   std::vector<MSTensor> inputs, outputs;
   std::shared_ptr<mindspore::kernel::Kernel> kernel;
-  std::shared_ptr<mindspore::kernel::KernelInterface> infer;
+  std::shared_ptr<mindspore::kernel::KernelInterface> infer;  // a provider's, or nullptr: builtin inference
+  bool has_op_parameter = false;
   mindspore::Context ctx;
+  const mindspore::Context *session_ctx = &ctx;  // nodes linked to a producer belong to the producer's session
   std::map<std::string, std::map<std::string, std::string>> config;  // the session's config file sections
 };
 
@@ -95,10 +195,18 @@ void Fill(const ph_op &op, schema::Primitive *p) {
 }
 
 int Infer(Session *s) {
-  if (s->infer == nullptr) return kOk;  // the builtin inference would run; the tests always register one
-  const mindspore::Status st = s->infer->Infer(&s->inputs, &s->outputs, &s->prim);
-  return st.IsOk() ? kOk : kInferFailed;
+  if (s->infer != nullptr) {  // a provider answered: InferNodeShape returns before it makes the OpParameter
+    s->has_op_parameter = false;
+    return s->infer->Infer(&s->inputs, &s->outputs, &s->prim).IsOk() ? kOk : kInferFailed;
+  }
+  s->has_op_parameter = true;
+  BuiltinInference builtin;
+  return builtin.Infer(&s->inputs, &s->outputs, &s->prim).IsOk() ? kOk : kInferFailed;
 }
+
+// A KernelInterface that a test may register under the provider name to see what registering one for a builtin
+// operator does to the fallback (the provider itself registers none).
+std::shared_ptr<mindspore::kernel::KernelInterface> TestInterfaceCreator() { return std::make_shared<BuiltinInference>(); }
 }  // namespace
 
 extern "C" {
@@ -120,6 +228,7 @@ void *ph_create_node(const ph_op *op, const char *arch, const char *provider, co
   for (int i = 0; i < n_in; ++i) {
     if (i == 0 && producer != nullptr) {
       s->inputs.push_back(static_cast<Session *>(producer)->outputs[0]);
+      s->session_ctx = static_cast<Session *>(producer)->session_ctx;
     } else {
       s->inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
     }
@@ -136,9 +245,9 @@ void *ph_create_node(const ph_op *op, const char *arch, const char *provider, co
     *stage = kNoCreator;
     return nullptr;
   }
-  s->kernel = creator(s->inputs, s->outputs, &s->prim, &s->ctx);
+  s->kernel = creator(s->inputs, s->outputs, &s->prim, s->session_ctx);
   if (s->kernel == nullptr) {
-    *stage = kDeclined;  // the scheduler would now take the builtin CPU kernel
+    *stage = s->has_op_parameter ? kDeclined : kDeclinedNoFallback;
     return nullptr;
   }
   s->kernel->SetConfig(&s->config);  // scheduler.cc:1455-1457
@@ -222,8 +331,9 @@ int32_t ph_infer(const ph_op *op, const char *provider, const ph_tensor *inputs,
   Fill(*op, &s.prim);
   for (int i = 0; i < n_in; ++i) s.inputs.push_back(Tensor(inputs[i], "in" + std::to_string(i)));
   s.outputs.push_back(MSTensor("out", mindspore::DataType::kNumberTypeInt8, {}, nullptr, 0, false));
-  auto iface = mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &s.prim);
-  if (iface == nullptr) return -3;
+  std::shared_ptr<mindspore::kernel::KernelInterface> iface =
+    mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &s.prim);
+  if (iface == nullptr) iface = std::make_shared<BuiltinInference>();
   const mindspore::Status st = iface->Infer(&s.inputs, &s.outputs, &s.prim);
   if (st == mindspore::kLiteInferInvalid) return -2;
   if (!st.IsOk()) return -1;
@@ -233,6 +343,53 @@ int32_t ph_infer(const ph_op *op, const char *provider, const ph_tensor *inputs,
 }
 
 void ph_destroy(void *h) { delete static_cast<Session *>(h); }
+
+// 1 when a KernelInterface is registered under `provider` for the operator type, else 0.
+int32_t ph_has_provider_interface(const char *provider, int32_t op_type) {
+  schema::Primitive prim;
+  prim.type_ = static_cast<schema::PrimitiveType>(op_type);
+  return mindspore::registry::RegisterKernelInterface::GetKernelInterface(provider, &prim) != nullptr ? 1 : 0;
+}
+
+// Registers the harness's own inference class under `provider` for one operator type (see TestInterfaceCreator).
+void ph_register_test_interface(const char *provider, int32_t op_type) {
+  mindspore::registry::RegisterKernelInterface::Reg(provider, op_type, TestInterfaceCreator);
+}
+
+// Two sessions at once: each node is executed `repeats` times on a thread of its own with its own input (the same
+// shape it was last run with).  Returns 0, or the first failing stage (of node a in the low byte, node b above it).
+int32_t ph_execute_concurrently(void *a, const void *in_a, void *b, const void *in_b, int32_t repeats) {
+  int32_t result[2] = {0, 0};
+  auto run = [&](void *h, const void *in, int32_t *out) {
+    auto *s = static_cast<Session *>(h);
+    for (int i = 0; i < repeats && *out == 0; ++i) {
+      memcpy(s->inputs[0].MutableData(), in, s->inputs[0].DataSize());
+      if (s->kernel->Execute() != 0) *out = kExecuteFailed;
+    }
+  };
+  std::thread ta(run, a, in_a, &result[0]), tb(run, b, in_b, &result[1]);
+  ta.join();
+  tb.join();
+  return result[0] | (result[1] << 8);
+}
+
+// The allocator where no page-locked memory can be had (no GPU): Malloc still returns usable, 64-byte-aligned memory
+// and the bookkeeping behaves the same.  Returns 0, or the number of the first check that failed.
+int32_t ph_allocator_fallback_selftest(void) {
+  std::shared_ptr<mindspore::Allocator> a = mindspore::mi355x::MakePinnedAllocator();
+  void *p = a->Malloc(1000);
+  if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 63) != 0) return 1;
+  memset(p, 0x11, 1000);
+  if (a->RefCount(p) != 0 || a->SetRefCount(p, 3) != 3 || a->DecRefCount(p, 1) != 2) return 2;
+  a->Free(p);
+  if (a->RefCount(p) != -1) return 3;
+  void *q = a->Malloc(800);
+  if (q != p) return 4;  // the freed block is reused
+  void *big = a->Malloc(size_t{1} << 20);
+  if (big == nullptr) return 5;
+  memset(big, 0x22, size_t{1} << 20);
+  return 0;  // the destructor releases both
+}
 
 // The pinned allocator as the runtime would use it for tensor data (lite::Tensor::MallocData / FreeData with the
 // reference counting of the executor).  Returns 0, or the number of the first check that failed.
