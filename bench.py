@@ -8,7 +8,7 @@ requantising epilogue); the decode GEMV (configuration 4, batch 1), DynamicQuant
 timed region.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm4096|gemm8192] [--no-cpu] [--no-extra]
-                    [--calibrate] [--conv3x3]
+                    [--calibrate] [--conv3x3] [--dynquant]
 """
 import argparse
 import json
@@ -210,7 +210,7 @@ def bench_vendor_int_mm(size, steps):
     return dict(ms=ms, tops=2.0 * size ** 3 / (ms * 1e-3) / 1e12, what="torch._int_mm, int32 output, uniform int8")
 
 
-def native_bench(*args):
+def native_bench(*args, env=None):
     """Runs mindspore_amd/native_bench (C++ host over the C ABI) as a child process and returns its JSON, or None when
     the binary is not built."""
     import subprocess
@@ -218,7 +218,8 @@ def native_bench(*args):
     if not os.path.exists(exe):
         return None
     try:
-        out = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=300, check=True)
+        out = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=300, check=True,
+                             env=dict(os.environ, **(env or {})))
         return json.loads(out.stdout.strip().splitlines()[-1])
     except Exception as ex:  # noqa: BLE001
         return dict(error=str(ex)[:200])
@@ -455,6 +456,9 @@ def main():
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--conv3x3", action="store_true",
                     help="also launch the batch-32 3x3 convolution of the extras 20 times (for profiling that kernel)")
+    ap.add_argument("--dynquant", action="store_true",
+                    help="also run DynamicQuant on the 4096 x 768 activation of configuration 3 a hundred times (for "
+                         "profiling its two kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this hot path is a single-GPU path; only --gpus 1 is supported (got %d)" % args.gpus,
@@ -511,6 +515,12 @@ def main():
             best["frac_of_hbm_peak"] = best["gbps"] / PEAK_HBM_GBPS
             if py:
                 best["python_host"] = dict(ms_per_step=py["ms_per_step"], gbps=py["gbps"])
+            if "host" in best and best["host"].startswith("native"):
+                best["note"] = "gate and up, which share their input, go out as one launch (mi_matmul_run_group)"
+                solo = native_bench("decode", m, 3, max(10, args.steps // 2), 3, env={"NATIVE_BENCH_NO_GROUP": "1"})
+                if solo and "gbps" in solo:
+                    best["one_launch_per_matrix"] = dict(ms_per_step=solo["ms_per_step"], gbps=solo["gbps"],
+                                                         launches_per_step=solo["launches_per_step"])
             extra["gemv_decode_m%d" % m] = best
         warm = native_bench("warm", 1, 200, 20)
         if warm and "qkv" in warm:
@@ -544,6 +554,14 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             lib.check(L.mi_diag_copy(dst.data_ptr(), src.data_ptr(), 256 << 20, _stream()), "mi_diag_copy")
+        torch.cuda.synchronize()
+    if args.dynquant:
+        from mindspore_amd import kernels as K
+        from mindspore_amd import workloads as wl
+        xq = torch.from_numpy(wl.bert_c3_activation(768)).cuda()
+        dq = K.DynamicQuantKernel(False)
+        for _ in range(100):
+            dq.run(xq, fetch_params=False)
         torch.cuda.synchronize()
     if args.conv3x3:
         kern, xin, yout, _ = make_conv3x3()
