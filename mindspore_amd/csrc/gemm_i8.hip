@@ -661,14 +661,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) v
 // benchmark's, sustains 7-9 % more (power-limited shader clock) with it.  For the same reason consecutive MFMAs
 // share one operand (serpentine order over the 4 x 4 sub-tiles): +5 %.
 // =====================================================================================================================
-template <int EPI, bool HAS_ZW, bool FAST>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kblock_kernel(GemmArgs g,
-                                                                                                      RequantParams rq,
-                                                                                                      DequantParams dq) {
+// T: the wave's sub-tile is T x T MFMA tiles, the workgroup's tile 64 T x 64 T.  T = 4 is the 256 x 256 tile described
+// above.  T = 2 (128 x 128, slots of 16 KiB, 80 KiB of LDS, a quarter of the registers) lets two workgroups share a
+// CU: for shapes with fewer than one 256 x 256 tile per CU, or short K, where one tile's prologue and epilogue have
+// to overlap another tile's main loop.  Per quarter a wave then has 4 MFMAs, 4 fragment reads and 2 loads.
+template <int T, int EPI, bool HAS_ZW, bool FAST>
+__device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const RequantParams &rq, const DequantParams &dq) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the buffer-resource type exists in the device pass only; the host pass needs just the stub
-  constexpr int TILE = 256, KB = 128, T = 4;  // wave tile 128 x 128 = T x T MFMA tiles
-  constexpr int SLOT = TILE * KB;             // one operand, one K block
-  constexpr int LPW = 8;                      // loader instructions per wave, operand and block (64 rows)
+  constexpr int TILE = 64 * T, KB = 128;  // wave tile 32 T x 32 T = T x T MFMA tiles
+  constexpr int SLOT = TILE * KB;         // one operand, one K block
+  constexpr int WROWS = TILE / 4;         // rows of each operand that a wave loads per block
+  constexpr int LPW = WROWS / 8;          // loader instructions per wave, operand and block (8 rows each)
+  static_assert(T == 2 || T == 4, "wave tiles of 64 x 64 or 128 x 128");
   static_assert(5 * SLOT >= kEpiArrays * TILE * 4 + 4 * epi_stage_bytes<EPI, T>(), "the epilogue staging must fit");
   __shared__ __attribute__((aligned(1024))) char lds[5 * SLOT];  // W slots 0-2, A slots 0-1
 
@@ -684,21 +688,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   EpiParams<TILE, EPI, FAST> epi;
   epi.fetch(rq, dq, n0, tid);
 
-  // loader: instruction i of a wave fills rows 64 * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
+  // loader: instruction i of a wave fills rows WROWS * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
   // L & 7 of its row, i.e. fetches logical chunk (L & 7) ^ ((row >> 1) & 7).  The loads are buffer loads: the address
   // is descriptor base + per-lane byte offset (a loop constant) + a scalar offset (row group and K block), so
   // issuing one costs scalar instructions only.
   const int drow = lane >> 3;
   const int dchunk = (lane & 7) ^ (drow >> 1);  // for even i; odd i: ^ 4
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<int8_t *>(g.w) + (int64_t)(n0 + wave * 64) * g.ldw, (short)0, -1, 0x00020000);
+      const_cast<int8_t *>(g.w) + (int64_t)(n0 + wave * WROWS) * g.ldw, (short)0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t a_rsrc =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(g.a) + (int64_t)m0 * g.lda, (short)0, -1, 0x00020000);
   const int w_voff = drow * g.ldw + dchunk * 16;  // ldw is a multiple of 256: odd i is w_voff ^ 64
   int a_voff[LPW];
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
-    int m = wave * 64 + 8 * i + drow;
+    int m = wave * WROWS + 8 * i + drow;
     m = m0 + m < g.m ? m : g.m - 1 - m0;
     a_voff[i] = m * (int)g.lda + ((dchunk ^ ((i & 1) << 2)) << 4);
   }
@@ -714,9 +718,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
   };
   auto lds_ptr = [](char *p) { return (__attribute__((address_space(3))) void *)p; };
-  // half: 0 = the wave's first four loader instructions (rows 0-31 of its 64), 1 = the other four
+  // half: 0 = the first half of the wave's loader instructions (the upper half of its rows), 1 = the other half
   auto dma_w = [&](int slot, int kb, int half) {
-    char *dst = lds + slot * SLOT + wave * 64 * KB;
+    char *dst = lds + slot * SLOT + wave * WROWS * KB;
 #pragma unroll
     for (int ii = 0; ii < LPW / 2; ++ii) {
       const int i = half * (LPW / 2) + ii;
@@ -725,7 +729,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
   };
   auto dma_a = [&](int slot, int kb, int half) {
-    char *dst = lds + (3 + slot) * SLOT + wave * 64 * KB;
+    char *dst = lds + (3 + slot) * SLOT + wave * WROWS * KB;
 #pragma unroll
     for (int ii = 0; ii < LPW / 2; ++ii) {
       const int i = half * (LPW / 2) + ii;
@@ -737,7 +741,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   int rowsum[T];
 #pragma unroll
   for (int j = 0; j < T; ++j) rowsum[j] = 0;
-  // the 256 accumulator registers are set while the first tiles are on their way (see below)
+  // the accumulator registers are set while the first tiles are on their way (see below)
   auto init_accumulators = [&]() {
     const int bias = (int)kAccBias;
 #pragma unroll
@@ -750,7 +754,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
 
   const int swz = (r >> 1) & 7;
-  const int w_off = (wn * 128 + r) * KB, a_off = 3 * SLOT + (wm * 128 + r) * KB;
+  const int w_off = (wn * 32 * T + r) * KB, a_off = 3 * SLOT + (wm * 32 * T + r) * KB;
   Frag<T, T> f0, f1;
   auto read_frag = [&](Frag<T, T> &f, int wslot, int aslot, int q) {  // q: 32-byte sub-step inside the block
     const int c = ((2 * q + h) ^ swz) << 4;
@@ -781,17 +785,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w[i], f.a[j], acc[i][j], 0, 0, 0);
       }
   };
-  // one LDS read behind each of the first 8 MFMAs of a quarter, then one load behind every other one of the rest
+  // T = 4: one LDS read behind each of the first 8 MFMAs of a quarter, then one load behind every other one of the
+  // rest.  T = 2: a read behind each of the 4 MFMAs, a load behind every other one.
   auto hints = [&]() {
+    if constexpr (T == 4) {
 #pragma unroll
-    for (int i = 0; i < 2 * T; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-    }
+      for (int i = 0; i < 2 * T; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+      }
 #pragma unroll
-    for (int i = 0; i < LPW / 2; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
+      for (int i = 0; i < LPW / 2; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global -> LDS load issue
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < LPW / 2; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -844,8 +860,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
                                                          lds + kEpiArrays * TILE * 4 + wave * epi_stage_bytes<EPI, T>(),
-                                                         n0, n0 + wn * 128, m0 + wm * 128, r, h);
+                                                         n0, n0 + wn * 32 * T, m0 + wm * 32 * T, r, h);
 #endif
+}
+
+template <int EPI, bool HAS_ZW, bool FAST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_kblock_kernel(GemmArgs g,
+                                                                                                      RequantParams rq,
+                                                                                                      DequantParams dq) {
+  gemm_kblock_body<4, EPI, HAS_ZW, FAST>(g, rq, dq);
+}
+
+// The 128 x 128 form, two workgroups per CU.
+template <int EPI, bool HAS_ZW, bool FAST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kblock128_kernel(
+    GemmArgs g, RequantParams rq, DequantParams dq) {
+  gemm_kblock_body<2, EPI, HAS_ZW, FAST>(g, rq, dq);
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
@@ -871,6 +901,16 @@ static int launch_kblock(GemmArgs g, const RequantParams &rq, const DequantParam
 }
 
 template <int EPI, bool HAS_ZW, bool FAST>
+static int launch_kblock128(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
+  g.tiles_m = (g.m + 127) / 128;
+  g.tiles_n = (g.n + 127) / 128;
+  hipLaunchKernelGGL((gemm_kblock128_kernel<EPI, HAS_ZW, FAST>), dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g,
+                     rq, dq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <int EPI, bool HAS_ZW, bool FAST>
 static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const DequantParams &dq,
                             hipStream_t stream) {
   const int64_t tiles_l = (int64_t)((g.m + 255) / 256) * ((g.n + 255) / 256);
@@ -883,6 +923,17 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // (its loader addresses activation rows with 32-bit offsets from the tile's first row)
   if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192) && g.lda < (1 << 23))
     return launch_kblock<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
+  // From one 128 x 128 tile per two CUs on: the K-block loop on 128 x 128 tiles, two workgroups per CU.  Whole
+  // cache lines per load and one barrier per 128 bytes of K make its main loop about a third shorter than the
+  // 64-byte-step loop below; two workgroups per CU instead of three make a round of tiles more expensive.  Measured on
+  // 21 int8-output shapes from 768 x 3072 x 768 to 1536 x 1536 x 6144: 0-25 % faster (2048^3 15.3 -> 13.8 us,
+  // 512 x 8192 x 1024 13.8 -> 10.5 us), 2 % slower only at K = 32.  With fp32 output the epilogue weighs more: it wins
+  // where the loop dominates (K >= 2048: 4096 x 768 x 3072 21.0 -> 19.0 us) and where the three-per-CU form below
+  // has all its tiles store in the same moment (>= 768 tiles: 4096 x 3072 x 768 25.9 -> 24.4 us), and loses on
+  // 576 tiles at K = 768 (18.4 against 22.2 us).
+  if (tiles_m >= 128 && g.k >= 128 && g.lda < (1 << 23) &&
+      (EPI == EPI_REQUANT || g.k >= 2048 || tiles_m >= 768))
+    return launch_kblock128<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // a few hundred activation rows against many channels: 256-channel x 128-row tiles keep the weight re-reads of
   // the square 128 tile away while still giving every CU a tile
   if (g.m <= 512 && (int64_t)((g.m + 127) / 128) * ((g.n + 255) / 256) >= 128)
