@@ -136,12 +136,38 @@ struct EpiParams {
   }
 };
 
+// What the fp32 epilogue needs of the input's quantisation.  With DynamicQuant upstream the values live in device
+// memory; they are fetched before the main loop, which hides a dependent load of a microsecond that would otherwise
+// sit between the last MFMA and the first store of every tile.
+template <int TM>
+struct DeqInput {
+  float sx;
+  int32_t zx;
+  float sxr[TM];  // per_row: the scale of the rows this lane holds
+  __device__ __forceinline__ void fetch(const DequantParams &dq, int m_w, int r, int m_total) {
+    sx = dq.sx;
+    zx = dq.zx;
+    if (dq.qp_dev != nullptr) {
+      sx = dq.qp_dev->scale_f;
+      zx = dq.qp_dev->zero_point;
+    }
+    // input_per_channel_: one input scale per row (NN/int8/dynamic_matmul_int8.c:126-128)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      int m = m_w + j * 32 + r;
+      m = m < m_total ? m : m_total - 1;
+      sxr[j] = dq.per_row ? dq.qp_dev[m].scale_f : sx;
+    }
+  }
+};
+
 // ACC0: the value the accumulators started from (see kAccBias); it leaves through the per-channel constants, so it
 // costs nothing here.
 template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST, uint32_t ACC0 = 0>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)[TM], const GemmArgs &g,
-                                              const RequantParams &rq, const DequantParams &dq, const int *p,
-                                              char *cstage, int n_tile, int n_w, int m_w, int r, int h) {
+                                              const RequantParams &rq, const DequantParams &dq,
+                                              const DeqInput<TM> din, const int *p, char *cstage, int n_tile, int n_w,
+                                              int m_w, int r, int h) {
   static_assert(!(EPI == EPI_REQUANT && FAST) || ACC0 == kAccBias, "the host folds kAccBias into c2");
   if (HAS_ZW) {
 #pragma unroll
@@ -323,21 +349,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
     }
   } else {
     float *c = static_cast<float *>(g.c);
-    float sx = dq.sx;
-    int32_t zx = dq.zx;
-    if (dq.qp_dev != nullptr) {
-      sx = dq.qp_dev->scale_f;
-      zx = dq.qp_dev->zero_point;
-    }
+    const int32_t zx = din.zx;
     const uint32_t kzz = (uint32_t)dq.deep * (uint32_t)zx * (uint32_t)dq.zw0;
-    // input_per_channel_: one input scale per row (NN/int8/dynamic_matmul_int8.c:126-128)
-    float sxr[TM];
-#pragma unroll
-    for (int j = 0; j < TM; ++j) {
-      int m = m_w + j * 32 + r;
-      m = m < g.m ? m : g.m - 1;
-      sxr[j] = dq.per_row ? dq.qp_dev[m].scale_f : sx;
-    }
     // As for the int8 output, the accumulator layout (a lane holds 4 consecutive columns of 32 different rows) is
     // turned into whole 128-byte row segments before it meets global memory: per 32-column block the wave's
     // TM x 32 rows go through a wave-private LDS tile (row stride 144 bytes: the 16-byte writes of 8 consecutive
@@ -345,52 +358,74 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
     constexpr int kRowB = kDeqStageRowBytes;
     const int lane = h * 32 + r;
     const int lr = lane >> 3, lc = lane & 7;
+    const bool has_bias = dq.bias != nullptr;
+    // The body exists four times: with and without an activation (decided once per tile instead of with branches
+    // around every output) and for full and ragged tiles (no bounds compares around the stores of a full one).
+    // ReLU and ReLU6 share one form: the upper bound of ReLU is +inf, and (inf < d) is false for every d, NaN
+    // included, exactly like the comparison the reference does not make.
+    const float act_hi = dq.act == MI_ACT_RELU6 ? 6.0f : __builtin_inff();
+    auto body = [&](auto full_c, auto act_c) {
+      constexpr bool FULL = decltype(full_c)::value, ACT = decltype(act_c)::value;
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
+      for (int i = 0; i < TN; ++i) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int nb = n_w + i * 32 + q * 8 + h * 4;
-        const int *pl = p + (nb - n_tile);
-        const v4f ws4 = *reinterpret_cast<const v4f *>(pl);
-        const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
-        const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
-        uint32_t corr[4];
+        for (int q = 0; q < 4; ++q) {
+          const int nb = n_w + i * 32 + q * 8 + h * 4;
+          const int *pl = p + (nb - n_tile);
+          const v4f ws4 = *reinterpret_cast<const v4f *>(pl);
+          const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
+          const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
+          uint32_t corr[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e] - ACC0;
+          for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e] - ACC0;
 #pragma unroll
-        for (int j = 0; j < TM; ++j) {
-          v4f o;
+          for (int j = 0; j < TM; ++j) {
+            v4f o;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            uint32_t v = (uint32_t)acc[i][j][q * 4 + e] + corr[e];
-            if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
-            float d = __fmul_rn(__fmul_rn(sxr[j], ws4[e]), (float)(int32_t)v);
-            if (dq.bias != nullptr) d = __fadd_rn(d, b4[e]);
-            if (dq.act == MI_ACT_RELU) {
-              d = (0.0f > d) ? 0.0f : d;
-            } else if (dq.act == MI_ACT_RELU6) {
-              d = (0.0f > d) ? 0.0f : d;
-              d = (6.0f < d) ? 6.0f : d;
+            for (int e = 0; e < 4; ++e) {
+              uint32_t v = (uint32_t)acc[i][j][q * 4 + e] + corr[e];
+              if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
+              float d = __fmul_rn(__fmul_rn(din.sxr[j], ws4[e]), (float)(int32_t)v);
+              if (has_bias) d = __fadd_rn(d, b4[e]);
+              if (ACT) {
+                d = (0.0f > d) ? 0.0f : d;
+                d = (act_hi < d) ? act_hi : d;
+              }
+              o[e] = d;
             }
-            o[e] = d;
+            *reinterpret_cast<v4f *>(cstage + (j * 32 + r) * kRowB + (q * 8 + h * 4) * 4) = o;
           }
-          *reinterpret_cast<v4f *>(cstage + (j * 32 + r) * kRowB + (q * 8 + h * 4) * 4) = o;
+        }
+        const int n = n_w + i * 32 + lc * 4;
+#pragma unroll
+        for (int t = 0; t < TM * 4; ++t) {
+          const int row = t * 8 + lr;
+          const v4f v = *reinterpret_cast<const v4f *>(cstage + row * kRowB + lc * 16);
+          const int m = m_w + row;
+          if (FULL || (m < g.m && n < g.n)) {
+            v4f *dst = reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + n);
+            if (FAST) {  // in this epilogue the parameter selects non-temporal stores (see stream_out_hint)
+              __builtin_nontemporal_store(v, dst);
+            } else {
+              *dst = v;
+            }
+          }
         }
       }
-      const int n = n_w + i * 32 + lc * 4;
-#pragma unroll
-      for (int t = 0; t < TM * 4; ++t) {
-        const int row = t * 8 + lr;
-        const v4f v = *reinterpret_cast<const v4f *>(cstage + row * kRowB + lc * 16);
-        const int m = m_w + row;
-        if (m < g.m && n < g.n) {
-          v4f *dst = reinterpret_cast<v4f *>(c + (int64_t)m * g.ldc + n);
-          if (FAST) {  // in this epilogue the parameter selects non-temporal stores (see stream_out_hint)
-            __builtin_nontemporal_store(v, dst);
-          } else {
-            *dst = v;
-          }
-        }
+    };
+    const bool full_tile = m_w + 32 * TM <= g.m && n_w + 32 * TN <= g.n;
+    const bool with_act = dq.act == MI_ACT_RELU || dq.act == MI_ACT_RELU6;
+    if (full_tile) {
+      if (with_act) {
+        body(std::true_type(), std::true_type());
+      } else {
+        body(std::true_type(), std::false_type());
+      }
+    } else {
+      if (with_act) {
+        body(std::false_type(), std::true_type());
+      } else {
+        body(std::false_type(), std::false_type());
       }
     }
   }
@@ -487,6 +522,8 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   const int kchunks = g.k >> 4;
   EpiParams<TILE_N, EPI, FAST> epi;
   epi.fetch(rq, dq, n0, tid);
+  DeqInput<TM> din;
+  if (EPI == EPI_DEQUANT) din.fetch(dq, m0 + wm * WM, r, g.m);
 
   // loader: a 1 KiB block holds 16 rows x 64 B.  Lane L fills slot (L & 3) of row (L >> 2) of its block, i.e. it
   // fetches logical chunk (L & 3) ^ swizzle(row), swizzle(row) = (row >> 1) & 3.
@@ -616,19 +653,19 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
-  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
                                                    lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
                                                    m0 + wm * WM, r, h);
 }
 
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_direct_kernel(GemmArgs g, RequantParams rq, DequantParams dq) {
   gemm_direct_body<TILE_N, TILE_M, EPI, HAS_ZW, FAST, NST, false>(g, rq, dq, ConvGather{});
 }
 
 // The same GEMM with the activation operand gathered from an NHWC image (no im2col buffer).
 template <int TILE_N, int TILE_M, bool HAS_ZW, bool FAST, int NST, int OCC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, OCC))) void gemm_conv_kernel(GemmArgs g, ConvGather cv, RequantParams rq) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_conv_kernel(GemmArgs g, ConvGather cv, RequantParams rq) {
   gemm_direct_body<TILE_N, TILE_M, EPI_REQUANT, HAS_ZW, FAST, NST, true>(g, rq, DequantParams{}, cv);
 }
 
@@ -687,6 +724,8 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   const int kchunks = g.k >> 4;
   EpiParams<TILE, EPI, FAST> epi;
   epi.fetch(rq, dq, n0, tid);
+  DeqInput<T> din;
+  if (EPI == EPI_DEQUANT) din.fetch(dq, m0 + wm * 32 * T, r, g.m);
 
   // loader: instruction i of a wave fills rows WROWS * wave + 8 * i + (lane >> 3) of a slot; lane L writes position
   // L & 7 of its row, i.e. fetches logical chunk (L & 7) ^ ((row >> 1) & 7).  The loads are buffer loads: the address
@@ -858,7 +897,7 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing re-fetches land before the LDS is reused
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
-  gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, reinterpret_cast<const int *>(lds),
+  gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
                                                          lds + kEpiArrays * TILE * 4 + wave * epi_stage_bytes<EPI, T>(),
                                                          n0, n0 + wn * 32 * T, m0 + wm * 32 * T, r, h);
 #endif
