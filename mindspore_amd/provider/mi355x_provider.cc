@@ -37,6 +37,7 @@
 // to the builtin CPU kernel (mindspore/lite/src/litert/scheduler.cc:1173-1177).
 #include <stdlib.h>
 
+#include <atomic>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -234,12 +235,78 @@ class DeviceIo {
 };
 
 // ---- MatMulFusion / FullConnection, int8 in -> int8 out (full quant) or fp32 out (dynamic quant) ----------------
+class MatmulKernel;
+
+// Full-quant MatMuls of one session that read the same input tensor with the same K (the gate and up projections of
+// a decoder layer, q / k / v when they are separate nodes).  With a few activation rows each of them is a launch of a
+// few microseconds whose fixed part is a fifth of it, so the first member that the session executes runs all of them
+// as one launch (mi_matmul_run_group) and the others find their result waiting.  This leans on what a Lite session
+// does (sub_graph_kernel.cc:456-466): the nodes of a graph are executed one after the other, each once per run, in
+// the same order every run, and a tensor has one producer, so between the first sibling's Execute and the last one's
+// nobody writes the shared input.  Sessions with Context::SetEnableParallel(true) form no groups.
+std::atomic<int64_t> g_group_launches{0};
+
+class SiblingGroup {
+ public:
+  static constexpr size_t kMaxMembers = 4;  // what mi_matmul_run_group takes as one launch
+  static std::shared_ptr<SiblingGroup> Join(const Context *ctx, const MSTensor &input, int32_t k, MatmulKernel *m) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    auto &groups = Groups();
+    for (auto it = groups.begin(); it != groups.end();) {
+      auto grp = it->lock();
+      if (grp == nullptr) {
+        it = groups.erase(it);
+        continue;
+      }
+      if (grp->ctx_ == ctx && grp->k_ == k && grp->input_ == input && grp->members_.size() < kMaxMembers) {
+        grp->members_.push_back(m);
+        return grp;
+      }
+      ++it;
+    }
+    auto grp = std::make_shared<SiblingGroup>(ctx, input, k);
+    grp->members_.push_back(m);
+    groups.push_back(grp);
+    return grp;
+  }
+  SiblingGroup(const Context *ctx, const MSTensor &input, int32_t k) : ctx_(ctx), input_(input), k_(k) {}
+  void Leave(MatmulKernel *m) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    for (auto it = members_.begin(); it != members_.end(); ++it) {
+      if (*it == m) {
+        members_.erase(it);
+        break;
+      }
+    }
+  }
+  // (members of one session run on that session's thread; the lock only guards joining and leaving)
+  std::vector<MatmulKernel *> Members() {
+    std::lock_guard<std::mutex> lock(Mutex());
+    return members_;
+  }
+
+ private:
+  static std::mutex &Mutex() {
+    static std::mutex *m = new std::mutex;
+    return *m;
+  }
+  static std::vector<std::weak_ptr<SiblingGroup>> &Groups() {
+    static auto *g = new std::vector<std::weak_ptr<SiblingGroup>>;
+    return *g;
+  }
+  const Context *ctx_;
+  MSTensor input_;  // a handle on the shared tensor object
+  int32_t k_;
+  std::vector<MatmulKernel *> members_;
+};
+
 class MatmulKernel : public kernel::Kernel {
  public:
   MatmulKernel(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out, const schema::Primitive *prim,
                const Context *ctx, bool b_transpose, int act)
       : Kernel(in, out, prim, ctx), b_transpose_(b_transpose), act_(act) {}
   ~MatmulKernel() override {
+    if (group_ != nullptr) group_->Leave(this);
     io_.Withdraw(&outputs_[0]);
     mi_matmul_destroy(full_);
     mi_dynmm_destroy(dyn_);
@@ -262,20 +329,40 @@ class MatmulKernel : public kernel::Kernel {
       const auto oq = outputs_[0].QuantParams().front();
       mi_matmul_desc d{k, n, b_transpose_ ? 1 : 0, act_, iq.scale, iq.zero_point, oq.scale, oq.zero_point,
                        static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
-      return ToStatus(mi_matmul_create(&d, static_cast<const int8_t *>(w.Data().get()),
-                                       static_cast<const int32_t *>(bias), &full_));
+      const int rc = mi_matmul_create(&d, static_cast<const int8_t *>(w.Data().get()),
+                                      static_cast<const int32_t *>(bias), &full_);
+      // (a session that runs its nodes in parallel gives no order to lean on: no groups there)
+      if (rc == MI_OK && !inputs_[0].IsConst() && context_ != nullptr && !context_->GetEnableParallel()) {
+        group_ = SiblingGroup::Join(context_, inputs_[0], k, this);
+      }
+      return ToStatus(rc);
     }
     mi_dynmm_desc d{k, n, b_transpose_ ? 1 : 0, act_, static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
     return ToStatus(
       mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_));
   }
 
-  int ReSize() override { return kSuccess; }  // the row count is read from the input tensor at every Execute
+  int ReSize() override {  // the row count is read from the input tensor at every Execute
+    computed_by_sibling_ = false;
+    return kSuccess;
+  }
 
   int Execute() override {
     const int32_t rows = static_cast<int32_t>(RowsOfOutput(outputs_[0]));
     if (rows == 0) return kSuccess;
     if (inputs_[0].ElementNum() != static_cast<int64_t>(rows) * k_) return kLiteError;
+    if (computed_by_sibling_) {
+      // a sibling's launch wrote this kernel's output buffer during this run, on the session's stream
+      computed_by_sibling_ = false;
+      if (sibling_rows_ == rows && sibling_host_ == inputs_[0].Data().get() &&
+          sibling_dev_ == inputs_[0].GetDeviceData()) {
+        return io_.Deliver(&outputs_[0]);
+      }
+    }
+    if (full_ != nullptr && group_ != nullptr && rows <= kSiblingMaxRows) {
+      const int rc = ExecuteWithSiblings(rows);
+      if (rc != kNotGrouped) return rc;
+    }
     const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
     void *c = io_.Output(outputs_[0].DataSize());
     if (a == nullptr || c == nullptr) return kLiteNullptr;
@@ -307,9 +394,53 @@ class MatmulKernel : public kernel::Kernel {
   }
 
  private:
+  static constexpr int32_t kSiblingMaxRows = 32;  // the row counts that mi_matmul_run_group runs as one launch
+  static constexpr int kNotGrouped = -1000;
+
+  // Runs this kernel and every sibling that is ready for the same rows as one launch.  kNotGrouped: nothing was
+  // launched (no sibling qualifies) and the caller goes on alone.
+  int ExecuteWithSiblings(int32_t rows) {
+    std::vector<MatmulKernel *> run;
+    run.push_back(this);
+    for (MatmulKernel *m : group_->Members()) {
+      if (m == this || m->full_ == nullptr) continue;
+      if (RowsOfOutput(m->outputs_[0]) != rows || m->inputs_[0].ElementNum() != static_cast<int64_t>(rows) * k_) continue;
+      run.push_back(m);
+    }
+    if (run.size() < 2) return kNotGrouped;
+    const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
+    if (a == nullptr) return kLiteNullptr;
+    std::vector<mi_matmul *> handles;
+    std::vector<int8_t *> outs;
+    for (MatmulKernel *m : run) {
+      void *c = m->io_.Output(m->outputs_[0].DataSize());
+      if (c == nullptr) return kLiteNullptr;
+      handles.push_back(m->full_);
+      outs.push_back(static_cast<int8_t *>(c));
+    }
+    if (mi_matmul_run_group(handles.data(), static_cast<int32_t>(handles.size()), a, rows, outs.data(),
+                            io_.stream()) != MI_OK) {
+      return kLiteError;
+    }
+    g_group_launches.fetch_add(1, std::memory_order_relaxed);
+    for (MatmulKernel *m : run) {
+      if (m == this) continue;
+      m->computed_by_sibling_ = true;
+      m->sibling_rows_ = rows;
+      m->sibling_host_ = inputs_[0].Data().get();
+      m->sibling_dev_ = inputs_[0].GetDeviceData();
+    }
+    return io_.Deliver(&outputs_[0]);
+  }
+
   bool b_transpose_;
   int act_;
   int32_t k_ = 0;
+  std::shared_ptr<SiblingGroup> group_;
+  bool computed_by_sibling_ = false;  // the output buffer already holds this run's result
+  int32_t sibling_rows_ = 0;          // ... for this row count and this input memory
+  const void *sibling_host_ = nullptr;
+  void *sibling_dev_ = nullptr;
   mi_matmul *full_ = nullptr;
   mi_dynmm *dyn_ = nullptr;
   DeviceIo io_;
@@ -600,5 +731,8 @@ struct Registrar {
   }
 } g_registrar;
 }  // namespace
+
+// How many times sibling MatMuls went out as one launch (for tests and for checking that a model's siblings were found).
+extern "C" int64_t mi355x_provider_group_launches() { return g_group_launches.load(std::memory_order_relaxed); }
 }  // namespace mi355x
 }  // namespace mindspore

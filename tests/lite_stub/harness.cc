@@ -277,6 +277,21 @@ int32_t ph_execute_linked(void *h, int32_t *code) {
   return kOk;
 }
 
+// Context::SetEnableParallel of the node's own session object; nodes created later with this node as their producer
+// see it in their Prepare.
+void ph_set_enable_parallel(void *h, int32_t on) { static_cast<Session *>(h)->ctx.SetEnableParallel(on != 0); }
+
+// What Model::Resize does for a node before anything is executed: infer the output shape from the producer's tensor and
+// call ReSize() when it changed.
+int32_t ph_resize_linked(void *h, int32_t *code) {
+  auto *s = static_cast<Session *>(h);
+  *code = 0;
+  const std::vector<int64_t> before = s->outputs[0].Shape();
+  if (Infer(s) != kOk) return kInferFailed;
+  if (before != s->outputs[0].Shape() && (*code = s->kernel->ReSize()) != 0) return kResizeFailed;
+  return kOk;
+}
+
 // Attaches an address to input 0 as an application could with MSTensor::SetDeviceData.
 void ph_set_input_device_data(void *h, void *address) { static_cast<Session *>(h)->inputs[0].SetDeviceData(address); }
 

@@ -74,6 +74,7 @@ class MSTensor {
   std::vector<QuantParam> QuantParams() const { return impl_->quant; }
   void SetQuantParams(std::vector<QuantParam> quant_params) { impl_->quant = std::move(quant_params); }
   std::string Name() const { return impl_->name; }
+  bool operator==(const MSTensor &tensor) const { return impl_ == tensor.impl_; }
   void SetDeviceData(void *data) { impl_->device_data = data; }
   void *GetDeviceData() { return impl_->device_data; }
   bool HasHostData() const { return impl_->data != nullptr; }  // harness-side

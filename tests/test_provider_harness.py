@@ -55,6 +55,10 @@ def _load_harness():
     h.ph_create_node.restype = C.c_void_p
     h.ph_create_node.argtypes = h.ph_create.argtypes[:9] + [C.c_void_p, C.c_char_p, C.c_char_p] + h.ph_create.argtypes[9:]
     h.ph_execute_linked.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    h.ph_resize_linked.argtypes = [C.c_void_p, C.POINTER(C.c_int32)]
+    h.ph_set_enable_parallel.argtypes = [C.c_void_p, C.c_int32]
+    h.ph_set_enable_parallel.restype = None
+    h.mi355x_provider_group_launches.restype = C.c_int64
     h.ph_set_input_device_data.argtypes = [C.c_void_p, C.c_void_p]
     h.ph_set_input_device_data.restype = None
     h.ph_output_state.argtypes = [C.c_void_p]
@@ -133,6 +137,12 @@ class Node:
         """Executes on the producer's output tensor as the producer left it."""
         code = C.c_int32(0)
         st = self.H.ph_execute_linked(self.h, C.byref(code))
+        assert st == OK, (st, code.value)
+
+    def resize_linked(self):
+        """Shape inference and ReSize() on the producer's current output shape, without executing."""
+        code = C.c_int32(0)
+        st = self.H.ph_resize_linked(self.h, C.byref(code))
         assert st == OK, (st, code.value)
 
     def state(self):
@@ -322,6 +332,49 @@ def test_two_sessions_on_two_threads(H, orc):
     assert np.array_equal(y2c, y2) and not np.array_equal(y2c, want2b)
     n1.close()
     n2.close()
+
+
+@pytest.mark.gpu
+def test_sibling_fullconnections_run_as_one_launch(H, orc):
+    """Three FullConnection nodes of one session read the same tensor (the output of a fourth): the first one executed
+    runs all three as one launch and the others deliver what it left; every output equals the oracle's, also after
+    resizes, and beyond 32 rows every node runs by itself.  A session that executes its nodes in parallel forms no
+    groups."""
+    rng = np.random.default_rng(21)
+    k0, k = 192, 512
+
+    def fc(n, kk, producer=None, out_name=None):
+        a, w, sw, b, ins = _fc_inputs(rng, 4, n, kk)
+        ins[0] = tensor(I8, (4, kk), None, False, [(0.05, 5)]) if producer is not None else ins[0]
+        node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], producer=producer, out_name=out_name)
+        assert node.stage == OK, (node.stage, node.code)
+        return node, w, sw, b
+
+    for parallel in (False, True):
+        head, w0, sw0, b0 = fc(k, k0, out_name=b"hidden")
+        if parallel:
+            H.ph_set_enable_parallel(head.h, 1)
+        sibs = [fc(n, k, producer=head) for n in (384, 640, 96)]
+        before = H.mi355x_provider_group_launches()
+        runs = 0
+        for rows in (4, 1, 7, 40):
+            x = rng.integers(-128, 128, (rows, k0), dtype=np.int8)
+            hidden, _ = head.run(x)
+            want_h = orc.matmul_int8(x, w0, b0, 0.02, -3, sw0, np.zeros(k, np.int32), 0.05, 5, 0, True)
+            assert np.array_equal(hidden, want_h)
+            for node, *_ in sibs:  # the runtime resizes every node of the graph before it executes any
+                node.resize_linked()
+            for node, w, sw, b in sibs:
+                node.run_linked()
+                got, _ = node.output()
+                want = orc.matmul_int8(want_h, w, b, 0.05, 5, sw, np.zeros(w.shape[0], np.int32), 0.05, 5, 0, True)
+                assert got.shape == want.shape and np.array_equal(got, want), (parallel, rows, w.shape)
+            runs += 1 if rows <= 32 else 0
+        launches = H.mi355x_provider_group_launches() - before
+        assert launches == (0 if parallel else runs), (parallel, launches)
+        for node, *_ in reversed(sibs):
+            node.close()
+        head.close()
 
 
 @pytest.mark.gpu
