@@ -72,7 +72,7 @@ def time_steps(fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall * 1e3 / steps  # ms per step by HIP events, by host clock
 
 
-def time_in_graph(fn, steps, warmup, calls=10):
+def time_in_graph(fn, steps, warmup, calls=10, settle_ms=40.0):
     """ms per call of fn with `calls` invocations captured in one HIP graph and the graph replayed: what the GPU
     needs per call once the Python host's per-call cost (about 10 us here) is out of the way, as it is for a C++
     caller of the C ABI."""
@@ -85,6 +85,15 @@ def time_in_graph(fn, steps, warmup, calls=10):
             for _ in range(calls):
                 fn()
     torch.cuda.synchronize()
+    # replayed for about 40 ms first: the timed replays start from the state the power management settles in under
+    # this load (see settle), not from the transient after an idle device
+    t0 = time.perf_counter()
+    for _ in range(200):
+        for _ in range(25):
+            graph.replay()
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 > settle_ms * 1e-3:
+            break
     ms, _ = time_steps(graph.replay, max(3, steps // calls), warmup)
     return ms / calls
 
@@ -96,20 +105,50 @@ def make_matmul(c):
                               True, c["act"])
 
 
-def bench_sustained(kern, a, out, size, launches=400):
-    """The same GEMM launched back to back for at least 20 ms: under this load the power management lowers the shader
-    clock within a few milliseconds, so the figure of a short timed region is a burst figure.  The shader clock is
-    read by a 0.3 ms matrix-pipe loop (in-kernel cycle counter against the 100 MHz counter) queued right behind the
-    last launch, on operands drawn like the GEMM's."""
+def settle(kern, a, out, min_ms=60.0, chunk=50):
+    """Launches the GEMM back to back from an idle device until at least `min_ms` of it have run, timing every chunk
+    of launches.  Under this load the power management first over-corrects -- launches 10 to ~150 after idle run
+    10-20 % slower than the first ones -- and settles after about 20 ms at a rate it then holds; a region of a few
+    dozen launches right after idle measures that transient, not the kernel.  The timed steps therefore start from
+    the settled state, and the series is reported so that the transient is visible."""
+    import torch
+    series, total, launches = [], 0.0, 0
+    while total < min_ms and len(series) < 64:
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(chunk):
+            kern.run(a, out=out)
+        stop.record()
+        torch.cuda.synchronize()  # (a wait of microseconds: the device does not leave the state it is in)
+        ms = start.elapsed_time(stop)
+        series.append(round(ms * 1e3 / chunk, 2))
+        total += ms
+        launches += chunk
+    return dict(launches=launches, ms=total, launches_per_chunk=chunk, us_per_launch_by_chunk=series,
+                note="untimed launches from an idle device before the warm-up and the timed steps: the shader clock "
+                     "needs about 20 ms under this load to settle")
+
+
+def sustained_probe():
+    """Buffers of bench_sustained, made before the device is brought to its settled state: a host pause of a few
+    milliseconds between two timed regions is enough for the power management to start over."""
     import numpy as np
     import torch
     from mindspore_amd import lib
     D = lib.load_diag()
     ops_t = torch.from_numpy(np.random.default_rng(0).integers(-128, 128, 32768, dtype=np.int8)).cuda()
     clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
-    for _ in range(5):
-        kern.run(a, out=out)
     torch.cuda.synchronize()
+    return D, ops_t, clocks
+
+
+def bench_sustained(kern, a, out, size, probe, launches=400):
+    """The same GEMM launched back to back for at least 20 ms, straight after the timed steps, i.e. from the settled
+    state (see settle).  The shader clock is read by a 0.3 ms matrix-pipe loop (in-kernel cycle counter against the
+    100 MHz counter) queued right behind the last launch, on operands drawn like the GEMM's."""
+    import torch
+    from mindspore_amd import lib
+    D, ops_t, clocks = probe
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(launches):
@@ -136,11 +175,14 @@ def bench_gemm(size, steps, warmup, host_path=False, sustained=False):
     prepare_ms = (time.perf_counter() - t0) * 1e3  # Prepare(): quant parameters, weight sums, packing, upload
     a = torch.from_numpy(c["a"]).cuda()
     out = torch.empty((size, size), dtype=torch.int8, device="cuda")
+    probe = sustained_probe() if sustained else None
+    settled = settle(kern, a, out, chunk=50 if size <= 4096 else 10)
     ev_ms, host_ms = time_steps(lambda: kern.run(a, out=out), steps, warmup)
     ops = 2.0 * size * size * size
-    res = dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c, prepare_ms=prepare_ms)
+    res = dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c, prepare_ms=prepare_ms,
+               settled=settled)
     if sustained:
-        res["sustained"] = bench_sustained(kern, a, out, size)
+        res["sustained"] = bench_sustained(kern, a, out, size, probe)
     if host_path:
         # the boundary as the provider uses it today: host tensors in and out (pinned staging + PCIe both ways)
         kern.run(c["a"])
@@ -537,7 +579,10 @@ def main():
         "ms_per_step": g["ms"], "ms_per_step_host_clock": g["host_ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "i8", "data": "synthetic",
         "config": {"workload": "config 5: int8 GEMM M=N=K=%d, per-channel requant to int8 (fused epilogue), zx=7, "
-                               "int32 bias" % size},
+                               "int32 bias" % size,
+                   "device_state": "settled: %d untimed launches (%.0f ms) from idle precede the warm-up, see "
+                                   "settled_before_timing" % (g["settled"]["launches"], g["settled"]["ms"])},
+        "settled_before_timing": g["settled"],
         "roofline": {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": None,
                      "kernel": HEADLINE_KERNEL, "ops_per_launch": g["ops"]},
