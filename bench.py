@@ -546,7 +546,7 @@ def main():
         if nread and "gbps" in nread:
             extra["hbm_read_stream_native_host"] = nread
         for m in (1, 8, 32):
-            nat = native_bench("decode", m, 3, max(10, args.steps // 2), 3)
+            nat = native_bench("decode", m, 3, 1000, 100)  # ~0.1 s of launches after ~10 ms of warm-up: the settled rate
             py = section("gemv_decode_m%d_python_host" % m, lambda: bench_gemv(max(5, args.steps // 2), 3, m))
             if nat and "gbps" in nat:
                 best = dict(nat, host="native C++ over the C ABI")
@@ -559,7 +559,7 @@ def main():
                 best["python_host"] = dict(ms_per_step=py["ms_per_step"], gbps=py["gbps"])
             if "host" in best and best["host"].startswith("native"):
                 best["note"] = "gate and up, which share their input, go out as one launch (mi_matmul_run_group)"
-                solo = native_bench("decode", m, 3, max(10, args.steps // 2), 3, env={"NATIVE_BENCH_NO_GROUP": "1"})
+                solo = native_bench("decode", m, 3, 1000, 100, env={"NATIVE_BENCH_NO_GROUP": "1"})
                 if solo and "gbps" in solo:
                     best["one_launch_per_matrix"] = dict(ms_per_step=solo["ms_per_step"], gbps=solo["gbps"],
                                                          launches_per_step=solo["launches_per_step"])
