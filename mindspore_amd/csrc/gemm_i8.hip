@@ -359,13 +359,16 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
     const int lane = h * 32 + r;
     const int lr = lane >> 3, lc = lane & 7;
     const bool has_bias = dq.bias != nullptr;
-    // The body exists four times: with and without an activation (decided once per tile instead of with branches
-    // around every output) and for full and ragged tiles (no bounds compares around the stores of a full one).
-    // ReLU and ReLU6 share one form: the upper bound of ReLU is +inf, and (inf < d) is false for every d, NaN
-    // included, exactly like the comparison the reference does not make.
+    // The body exists three times, chosen once per tile instead of with branches around every output: full tile
+    // without activation and with one input scale (no bounds compares, no clamps, the scale product hoisted), full
+    // tile in general, ragged tile in general.
+    // The general bodies clamp between bounds that are infinite where the reference makes no comparison: (-inf > d)
+    // and (inf < d) are false for every d, NaN included, so no activation, ReLU and ReLU6 share one form.
+    const bool with_act = dq.act == MI_ACT_RELU || dq.act == MI_ACT_RELU6;
+    const float act_lo = with_act ? 0.0f : -__builtin_inff();
     const float act_hi = dq.act == MI_ACT_RELU6 ? 6.0f : __builtin_inff();
-    auto body = [&](auto full_c, auto act_c) {
-      constexpr bool FULL = decltype(full_c)::value, ACT = decltype(act_c)::value;
+    auto body = [&](auto full_c, auto act_c, auto rows_c) {
+      constexpr bool FULL = decltype(full_c)::value, ACT = decltype(act_c)::value, PER_ROW = decltype(rows_c)::value;
 #pragma unroll
       for (int i = 0; i < TN; ++i) {
 #pragma unroll
@@ -376,8 +379,12 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
           const v4i wsum4 = *reinterpret_cast<const v4i *>(pl + TILE_N);
           const v4f b4 = *reinterpret_cast<const v4f *>(pl + 2 * TILE_N);
           uint32_t corr[4];
+          float s4[4];  // one input scale for the whole tensor: the scale product is the same for every row
 #pragma unroll
-          for (int e = 0; e < 4; ++e) corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e] - ACC0;
+          for (int e = 0; e < 4; ++e) {
+            corr[e] = kzz - (uint32_t)zx * (uint32_t)wsum4[e] - ACC0;
+            s4[e] = __fmul_rn(din.sx, ws4[e]);
+          }
 #pragma unroll
           for (int j = 0; j < TM; ++j) {
             v4f o;
@@ -385,10 +392,10 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
             for (int e = 0; e < 4; ++e) {
               uint32_t v = (uint32_t)acc[i][j][q * 4 + e] + corr[e];
               if (HAS_ZW) v -= (uint32_t)dq.zw0 * (uint32_t)rowsum[j];
-              float d = __fmul_rn(__fmul_rn(din.sxr[j], ws4[e]), (float)(int32_t)v);
+              float d = __fmul_rn(PER_ROW ? __fmul_rn(din.sxr[j], ws4[e]) : s4[e], (float)(int32_t)v);
               if (has_bias) d = __fadd_rn(d, b4[e]);
               if (ACT) {
-                d = (0.0f > d) ? 0.0f : d;
+                d = (act_lo > d) ? act_lo : d;
                 d = (act_hi < d) ? act_hi : d;
               }
               o[e] = d;
@@ -414,19 +421,14 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
       }
     };
     const bool full_tile = m_w + 32 * TM <= g.m && n_w + 32 * TN <= g.n;
-    const bool with_act = dq.act == MI_ACT_RELU || dq.act == MI_ACT_RELU6;
-    if (full_tile) {
-      if (with_act) {
-        body(std::true_type(), std::true_type());
-      } else {
-        body(std::true_type(), std::false_type());
-      }
+    // (the common case, a full tile of a MatMul without activation and with one input scale, has a body of its own;
+    //  per-row scales and activations share the general one)
+    if (full_tile && !with_act && !dq.per_row) {
+      body(std::true_type(), std::false_type(), std::false_type());
+    } else if (full_tile) {
+      body(std::true_type(), std::true_type(), std::true_type());
     } else {
-      if (with_act) {
-        body(std::false_type(), std::true_type());
-      } else {
-        body(std::false_type(), std::false_type());
-      }
+      body(std::false_type(), std::true_type(), std::true_type());
     }
   }
 }
@@ -968,10 +970,10 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // 21 int8-output shapes from 768 x 3072 x 768 to 1536 x 1536 x 6144: 0-25 % faster (2048^3 15.3 -> 13.8 us,
   // 512 x 8192 x 1024 13.8 -> 10.5 us), 2 % slower only at K = 32.  With fp32 output the epilogue weighs more: it wins
   // where the loop dominates (K >= 2048: 4096 x 768 x 3072 21.0 -> 19.0 us) and where the three-per-CU form below
-  // has all its tiles store in the same moment (>= 768 tiles: 4096 x 3072 x 768 25.9 -> 24.4 us), and loses on
-  // 576 tiles at K = 768 (18.4 against 22.2 us).
+  // has all its tiles store in the same moment (>= 768 tiles: 4096 x 3072 x 768 25.9 -> 24.4 us), and with at most
+  // one tile per CU (4096 x 768 x 768: 8.6 -> 8.3 us); it loses on 576 tiles at K = 768 (18.4 against 22.2 us).
   if (tiles_m >= 128 && g.k >= 128 && g.lda < (1 << 23) &&
-      (EPI == EPI_REQUANT || g.k >= 2048 || tiles_m >= 768))
+      (EPI == EPI_REQUANT || g.k >= 2048 || tiles_m >= 768 || tiles_m <= 256))
     return launch_kblock128<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // a few hundred activation rows against many channels: 256-channel x 128-row tiles keep the weight re-reads of
   // the square 128 tile away while still giving every CU a tile
