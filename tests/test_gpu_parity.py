@@ -102,6 +102,24 @@ def test_matmul_whole_cu_tile_ragged(orc, m, n, k):
         assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("m,n,k", [(1408, 1408, 144), (1500, 1420, 144), (1536, 1536, 112), (1300, 1700, 400),
+                                   (2050, 1030, 1168), (700, 5000, 128), (1664, 1280, 256)])
+def test_matmul_128_tile_k_block_loop(orc, m, n, k):
+    """The 128 x 128 tile with 128-byte K blocks (two workgroups per CU) and its neighbours: 121 tiles (below its
+    range) and 144, K below one block and exactly one, two, K that ends inside a block, ragged rows and channels,
+    whole tiles only; per-tensor / per-channel, zero and non-zero weight zero points, the generic rounding path."""
+    rng = np.random.default_rng(m * 3 + n * 5 + k)
+    orc.set_threads(16)
+    for it in range(4):
+        case = _mm_case(rng, m, n, k, bool(it & 1), bool(it & 2), it != 2, [0, 1, 3, 0][it], it != 3,
+                        1e-3 if it == 3 else 100.0)
+        if it == 3:
+            case["bias"] = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+        got, _ = _gpu_matmul(case, device_tensors=True)
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
+
+
 @pytest.mark.parametrize("rows,k,ns", [(1, 4096, (1100, 900)), (2, 1040, (64, 260, 36)), (1, 144, (8, 4, 12, 20)),
                                        (1, 11008, (300, 301)), (5, 4096, (256, 8200)), (8, 1040, (48, 16, 100)),
                                        (17, 2048, (40, 520)), (32, 400, (33, 31, 64, 5)),
@@ -360,7 +378,10 @@ def test_dynamic_matmul(orc):
     rng = np.random.default_rng(401)
     orc.set_threads(16)
     for it, (m, n, k) in enumerate([(1, 1, 1), (5, 9, 17), (33, 70, 64), (130, 65, 300), (9, 256, 1000),
-                                    (700, 300, 129), (64, 2304, 768), (4100, 4096, 400), (4097, 4100, 208)]):
+                                    (700, 300, 129), (64, 2304, 768), (4100, 4096, 400), (4097, 4100, 208),
+                                    # fp32 output on the 128-tile K-block loop: at most one tile per CU, K >= 2048,
+                                    # 768 tiles and more; and 306 tiles, which stay on the 64-byte-step loop
+                                    (1500, 1420, 144), (1300, 1290, 2064), (4100, 3000, 144), (2100, 2304, 208)]):
         a = rng.integers(-128, 128, (m, k), dtype=np.int8)
         w = rng.integers(-128, 128, (n, k), dtype=np.int8)
         nf = n if it & 1 else 1
@@ -397,8 +418,12 @@ def test_dynamic_quant_chained_into_matmul(orc):
     assert np.array_equal(y.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("rows,k", [(1, 16), (5, 7), (37, 100), (64, 768), (130, 1030), (3, 5000)])
-def test_dynamic_quant_per_row_and_matmul(orc, rows, k):
+@pytest.mark.parametrize("rows,k,n", [(1, 16, 24), (5, 7, 24), (37, 100, 24), (64, 768, 24), (130, 1030, 24),
+                                      (3, 5000, 24),
+                                      # enough 128 x 128 tiles for the K-block loop: full and ragged tiles of the
+                                      # general fp32 epilogue with one input scale per row
+                                      (1500, 272, 1420)])
+def test_dynamic_quant_per_row_and_matmul(orc, rows, k, n):
     """Per-channel activation quantisation (one scale per row) feeding the dynamic MatMul with per-row input scales,
     host path and device-chained path, symmetric (what the converter emits) and asymmetric."""
     import torch
@@ -408,7 +433,7 @@ def test_dynamic_quant_per_row_and_matmul(orc, rows, k):
     if rows > 2:
         x[1] = 0.25          # constant row: range 0 -> the 0.01 fallback
         x[2, 0] = np.inf     # +inf dominates the row's max
-    n = 24
+    orc.set_threads(16)
     w = rng.integers(-128, 128, (n, k), dtype=np.int8)
     sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
     bias = rng.normal(0, 0.1, n).astype(np.float32)
