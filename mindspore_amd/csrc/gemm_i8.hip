@@ -11,12 +11,17 @@
 // one output row: the epilogue packs them into one 32-bit store, per-channel parameters are 16-byte loads, and
 // the input-row sum a lane needs is the one it accumulated itself (v_dot4 against 0x01010101).
 //
-// Main loop: tiles travel global -> LDS with asynchronous 16-byte-per-lane loads (global_load_lds_dwordx4), NST
-// LDS stages of 64 bytes of K, NST - 1 tiles in flight, one barrier per stage; operand fragments for K sub-step
-// s+1 are read from LDS while the MFMAs of sub-step s run.  Any K that is a multiple of 16: the weights are zero
-// padded, so an activation chunk past K only has to be a valid read (it re-reads the row's last chunk).
-// LDS rows are XOR-swizzled in units of 16 bytes so that 8 consecutive lanes of a 16-byte access always cover
-// all 32 banks.
+// Two main loops, both moving tiles global -> LDS with asynchronous 16-byte-per-lane loads and reading operand
+// fragments for the next K sub-step from LDS while the MFMAs of the current one run:
+//   * K blocks of 128 bytes (gemm_kblock_body): whole cache lines per load, five LDS slots, one barrier per block;
+//     256 x 256 tiles with one workgroup per CU for the large compute-bound shapes, 128 x 128 tiles with two
+//     workgroups per CU for the mid-sized ones;
+//   * K steps of 64 bytes through NST LDS stages (gemm_direct_body): the smaller tiles, up to four workgroups per
+//     CU, the few-rows weight stream (NST = 8 / 16) and the convolution whose activation operand is gathered from
+//     the image.
+// Any K that is a multiple of 16: the weights are zero padded, so an activation chunk past K only has to be a valid
+// read (it re-reads the row's last chunk).  LDS rows are XOR-swizzled in units of 16 bytes so that the 16-byte
+// fragment reads of a wave are bank-conflict free.
 #include "common.h"
 #include "quant_math.h"
 
