@@ -94,7 +94,7 @@ def time_in_graph(fn, steps, warmup, calls=10, settle_ms=40.0):
         torch.cuda.synchronize()
         if time.perf_counter() - t0 > settle_ms * 1e-3:
             break
-    ms, _ = time_steps(graph.replay, max(3, steps // calls), warmup)
+    ms, _ = time_steps(graph.replay, max(20, steps // calls), warmup)  # at least 200 calls: a few ms
     return ms / calls
 
 
