@@ -171,8 +171,8 @@ struct DeqInput {
 template <int TILE_N, int TN, int TM, int EPI, bool HAS_ZW, bool FAST, uint32_t ACC0 = 0>
 __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)[TM], const GemmArgs &g,
                                               const RequantParams &rq, const DequantParams &dq,
-                                              const DeqInput<TM> din, const int *p, char *cstage, int n_tile, int n_w,
-                                              int m_w, int r, int h) {
+                                              const DeqInput<TM> din, const int *p, char *cstage, char *cstage_wg,
+                                              int n_tile, int m_tile, int n_w, int m_w, int r, int h) {
   static_assert(!(EPI == EPI_REQUANT && FAST) || ACC0 == kAccBias, "the host folds kAccBias into c2");
   if (HAS_ZW) {
 #pragma unroll
@@ -193,6 +193,13 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
     // passes of 32 rows would hide more of the stores, but every pass re-reads the per-channel constants from LDS,
     // and at four passes those reads take longer than the arithmetic.)
     constexpr bool kStageC = (TN == 4 && TM == 4);
+    // The 128 x 128 tile (four wave tiles of 64 channels x 64 rows) does the same through ONE staging tile of
+    // 128 rows x 128 B shared by the workgroup (same layout), so that its rows, too, leave as whole 128-byte lines:
+    // every wave drops its quadrant, the workgroup meets, every wave stores 32 rows.  Straight from the accumulator
+    // layout the stores were a quarter to a third of the launch time of mid-sized shapes (4096 x 1024 x 1024: 2.3 of
+    // 9.0 us, 3136 x 2048 x 512: 3.3 of 10.0 us).
+    constexpr bool kStageWG = (TN == 2 && TM == 2);
+    const int wn_id = (n_w - n_tile) / (32 * TN), wm_id = (m_w - m_tile) / (32 * TM);
     const int lane = h * 32 + r;
     const bool vec16 = ((g.ldc & 15) == 0) && ((reinterpret_cast<uintptr_t>(c) & 15) == 0);
     // four outputs (consecutive channels of one row): accumulator registers -> clamped int32
@@ -236,7 +243,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
       }
     };
     // whole wave tile inside the matrix and 16-byte stores possible: the stores need no bounds checks
-    const bool full_tile = vec16 && m_w + 32 * TM <= g.m && n_w + 32 * TN <= g.n;
+    const bool full_tile = kStageWG ? vec16 && m_tile + 64 * TM <= g.m && n_tile + 64 * TN <= g.n
+                                    : vec16 && m_w + 32 * TM <= g.m && n_w + 32 * TN <= g.n;
     // The body is compiled twice: for wave tiles that lie wholly inside the matrix with 16-byte stores possible
     // (no bounds checks, no divergent branches around the stores) and for the ragged rest.
     auto body = [&](auto full_c) {
@@ -268,9 +276,42 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
           }
         }
       };
+      // the workgroup-shared form: wave w stores rows 32 w .. 32 w + 31 of the tile, 8 per instruction
+      auto store_rows_wg = [&](int tt) {
+        const int c16 = lane & 7, lrow = lane >> 3;
+        const int n = n_tile + c16 * 16;
+        const int row = lrow + 8 * (4 * (wm_id * 2 + wn_id) + tt);
+        const v4i x = *reinterpret_cast<const v4i *>(cstage_wg + row * 128 + ((c16 ^ lrow) << 4));
+        v4i o;  // undo the in-chunk rotation: (row >> 3) & 3 == tt
+        o[0] = x[(0 + tt) & 3];
+        o[1] = x[(1 + tt) & 3];
+        o[2] = x[(2 + tt) & 3];
+        o[3] = x[(3 + tt) & 3];
+        const int m = m_tile + row;
+        if (FULL) {
+          *reinterpret_cast<v4i *>(c + (int64_t)m * g.ldc + n) = o;
+        } else if (m < g.m && n < g.n) {
+          int8_t *dst = c + (int64_t)m * g.ldc + n;
+          if (vec16 && n + 16 <= g.n) {
+            *reinterpret_cast<v4i *>(dst) = o;
+          } else {
+  #pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + 4 * e < g.n) *reinterpret_cast<int *>(dst + 4 * e) = o[e];
+          }
+        }
+      };
       constexpr int kPhases = kStageC ? 2 : 1, kJ = TM / kPhases;  // row blocks per pass over the channels
       // where this lane's dword of piece (i, q) goes in its staging row (see the layout above)
-      int stage_off[kStageC ? TN * 4 : 1];
+      int stage_off[(kStageC || kStageWG) ? TN * 4 : 1];
+      if (kStageWG) {
+  #pragma unroll
+        for (int i = 0; i < TN; ++i)
+  #pragma unroll
+          for (int q = 0; q < 4; ++q)
+            stage_off[i * 4 + q] = (wm_id * 32 * TM + r) * 128 + (((wn_id * 4 + 2 * i + (q >> 1)) ^ (r & 7)) << 4) +
+                                   (((2 * q + h + (r >> 3)) & 3) << 2);
+      }
       if (kStageC) {
   #pragma unroll
         for (int i = 0; i < TN; ++i)
@@ -317,7 +358,7 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
             const Piece pc = next;
             next = load_piece(i * 4 + q + 1);  // (wraps to piece 0 for the next pass; the arrays are padded)
             // (the staged form computes every channel of the padded tile and lets the stores check the bounds)
-            if (!kStageC && nb >= g.n) continue;
+            if (!kStageC && !kStageWG && nb >= g.n) continue;
             const v4i c2lo4 = v4i{pc.c01[0], pc.c01[2], pc.c23[0], pc.c23[2]};
             const v4i c2hi4 = v4i{pc.c01[1], pc.c01[3], pc.c23[1], pc.c23[3]};
   #pragma unroll
@@ -329,6 +370,8 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
               const uint32_t packed = pack4(y[0], y[1], y[2], y[3]);
               if (kStageC) {
                 *reinterpret_cast<uint32_t *>(cstage + j * 32 * 128 + stage_off[i * 4 + q]) = packed;
+              } else if (kStageWG) {
+                *reinterpret_cast<uint32_t *>(cstage_wg + j * 32 * 128 + stage_off[i * 4 + q]) = packed;
               } else {
                 const int m = m_w + j * 32 + r;
                 if (m < g.m) *reinterpret_cast<uint32_t *>(c + (int64_t)m * g.ldc + nb) = packed;
@@ -345,6 +388,11 @@ __device__ __forceinline__ void gemm_epilogue(v16i (&acc)[TN][TM], int (&rowsum)
       if (kStageC) {
   #pragma unroll
         for (int t = 8; t < 16; ++t) store_rows(t);
+      }
+      if (kStageWG) {
+        __syncthreads();
+  #pragma unroll
+        for (int tt = 0; tt < 4; ++tt) store_rows_wg(tt);
       }
     };
     if (full_tile) {
@@ -513,6 +561,8 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   constexpr int STAGE = (TILE_N + TILE_M) * BKD;
   constexpr int WPW = TILE_N / 16 / 4, APW = TILE_M / 16 / 4, LPW = WPW + APW;  // 1 KiB blocks per wave and tile
   static_assert(WPW >= 1 && APW >= 1, "tile too small");
+  static_assert(EPI != EPI_REQUANT || TN != 2 || TM != 2 || NST * STAGE >= kEpiArrays * TILE_N * 4 + 16384,
+                "the workgroup's output staging tile must fit the main loop's LDS");
   static_assert(EPI == EPI_REQUANT ? (TN != 4 || TM != 4 || NST * STAGE >= kEpiArrays * TILE_N * 4 + 4 * 16384)
                                    : NST * STAGE >= kEpiArrays * TILE_N * 4 + 4 * epi_stage_bytes<EPI, TM>(),
                 "the epilogue staging must fit the main loop's LDS");
@@ -660,9 +710,10 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
-  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
-                                                   lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), n0, n0 + wn * WN,
-                                                   m0 + wm * WM, r, h);
+  gemm_epilogue<TILE_N, TN, TM, EPI, HAS_ZW, FAST, kAccBias>(
+      acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
+      lds + kEpiArrays * TILE_N * 4 + wave * epi_stage_bytes<EPI, TM>(), lds + kEpiArrays * TILE_N * 4, n0, m0,
+      n0 + wn * WN, m0 + wm * WM, r, h);
 }
 
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST, int OCC>
@@ -906,7 +957,8 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
                                                          lds + kEpiArrays * TILE * 4 + wave * epi_stage_bytes<EPI, T>(),
-                                                         n0, n0 + wn * 32 * T, m0 + wm * 32 * T, r, h);
+                                                         lds + kEpiArrays * TILE * 4, n0, m0, n0 + wn * 32 * T,
+                                                         m0 + wm * 32 * T, r, h);
 #endif
 }
 
