@@ -106,31 +106,41 @@ static void activation_range(int act, int32_t zp, float scale, int32_t *mn, int3
 }
 
 // ---- device memory helpers ------------------------------------------------------------------------------------------
+// A buffer that only grows.  Growing happens inside a run (a new shape, a longer im2col workspace), possibly with
+// kernels still in flight that use the old memory, so the old allocation is neither freed there -- hipFree waits for
+// the whole device -- nor reused: it is kept until the handle goes away, and the size at least doubles, which bounds
+// what is kept to the final size once more.
 struct DevBuf {
   void *p = nullptr;
   size_t bytes = 0;
+  std::vector<void *> retired;
   DevBuf() = default;
   DevBuf(const DevBuf &) = delete;
   DevBuf &operator=(const DevBuf &) = delete;
   ~DevBuf() { release(); }
   int ensure(size_t want) {
     if (want <= bytes) return MI_OK;
-    if (p != nullptr) {
-      MI_HIP_CHECK(hipFree(p));
-      p = nullptr;
-      bytes = 0;
+    size_t sz = p != nullptr && want < 2 * bytes ? 2 * bytes : want;
+    sz = (sz + 4095) & ~(size_t)4095;
+    void *q = nullptr;
+    if (hipMalloc(&q, sz) != hipSuccess) {
+      (void)hipGetLastError();
+      sz = (want + 4095) & ~(size_t)4095;  // the doubled size did not fit: exactly what is needed
+      if (hipMalloc(&q, sz) != hipSuccess) {
+        (void)hipGetLastError();
+        set_error("hipMalloc(%zu) failed", sz);
+        return MI_MEMORY_FAILED;
+      }
     }
-    const size_t sz = (want + 4095) & ~(size_t)4095;
-    if (hipMalloc(&p, sz) != hipSuccess) {
-      p = nullptr;
-      set_error("hipMalloc(%zu) failed", sz);
-      return MI_MEMORY_FAILED;
-    }
+    if (p != nullptr) retired.push_back(p);
+    p = q;
     bytes = sz;
     return MI_OK;
   }
   void release() {
     if (p != nullptr) (void)hipFree(p);
+    for (void *q : retired) (void)hipFree(q);
+    retired.clear();
     p = nullptr;
     bytes = 0;
   }
