@@ -1016,10 +1016,14 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // a few activation rows against a big weight matrix: one row of 64 x 64 tiles, deep prefetch (HBM-bound)
   if (g.m <= 64 && g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 16>(g, rq, dq, stream);
   if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
-  // the fp32 epilogue writes four times the bytes: below one 256 x 256 tile per CU it is worth more to overlap it
-  // with another workgroup's main loop (two 128 x 128 tiles per CU) than to save operand traffic
-  // (its loader addresses activation rows with 32-bit offsets from the tile's first row)
-  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 192) && g.lda < (1 << 23))
+  // The 256 x 256 tile does a unit of work in little more than half the time the 128 x 128 tiles need, so with int8
+  // output it is taken as soon as the 128 x 128 tiles would no longer fit the device in one go (more than 512 of
+  // them, i.e. more than 128 large tiles): 2304 x 4096 x 4096 51.6 -> 41.2 us, 2816 x 4096 x 1024 20.4 -> 17.8 us;
+  // at exactly 128 large tiles the 512 small ones win (2048 x 4096 x 4096: 35.5 against 39.8 us).
+  // The fp32 epilogue writes four times the bytes: below one 256 x 256 tile per CU it is worth more to overlap it
+  // with another workgroup's main loop than to save operand traffic.
+  // (the loader addresses activation rows with 32-bit offsets from the tile's first row)
+  if (tiles_l >= (EPI == EPI_DEQUANT ? 256 : 129) && g.lda < (1 << 23))
     return launch_kblock<EPI, HAS_ZW, FAST>(g, rq, dq, stream);
   // From one 128 x 128 tile per two CUs on: the K-block loop on 128 x 128 tiles, two workgroups per CU.  Whole
   // cache lines per load and one barrier per 128 bytes of K make its main loop about a third shorter than the
