@@ -380,7 +380,7 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
   const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
                                            : rows <= kGemvMaxRows && st.w_blocked.p != nullptr;
   if (skinny) {
-    if (rows > kGemvDotRows) w.blocked = static_cast<const int8_t *>(st.w_blocked.p);
+    if (rows >= 2) w.blocked = static_cast<const int8_t *>(st.w_blocked.p);  // (may be absent: two rows then take the v_dot4 kernel)
     return launch_gemv_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
   }
   if ((st.n & 3) == 0 && (reinterpret_cast<uintptr_t>(c) & 3) == 0)

@@ -68,7 +68,7 @@ class _Handle:
 
 class MatmulInt8Kernel(_Handle):
     """Full-quant int8 MatMul: C = requant(A x W^T).  weight is [N, K] when transpose_b else [K, N]; bias int32 [N].
-    decode_pack=False skips the second packed form of the weights (the one runs with 3..32 rows use); such rows then
+    decode_pack=False skips the second packed form of the weights (the one runs with 2..32 rows use); such rows then
     run on the GEMM tiles."""
     _destroy = "mi_matmul_destroy"
 

@@ -34,9 +34,9 @@ def _mm_case(rng, m, n, k, peroc, zwnz, hb, act, bt=True, so_mul=100.0):
     return dict(a=a, w=w, bias=bias, sx=sx, zx=zx, sw=sw, zw=zw, so=so, zo=zo, act=act, b_transpose=bt)
 
 
-def _gpu_matmul(case, device_tensors=False):
+def _gpu_matmul(case, device_tensors=False, decode_pack=True):
     kern = K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]), _qps(case["sw"], case["zw"]),
-                              QP(case["so"], case["zo"]), case["b_transpose"], case["act"])
+                              QP(case["so"], case["zo"]), case["b_transpose"], case["act"], decode_pack=decode_pack)
     if device_tensors:
         import torch
         out = kern.run(torch.from_numpy(case["a"]).cuda())
@@ -71,7 +71,8 @@ def test_matmul_shapes(orc, m, n, k):
                                  (21, 2800), (18, 6144), (13, 7008), (11, 8192), (7, 9232), (10, 10240), (6, 11008),
                                  (5, 12288)])
 def test_decode_rows_every_stream_shape(orc, n, k):
-    """1..32 activation rows (v_dot4 kernel up to 2, matrix-core kernel above: one group of 16 rows up to 16, two
+    """1..32 activation rows (v_dot4 kernel for one row, and for two on a handle without the blocked copy; matrix-core
+    kernel otherwise: one group of 16 rows up to 16, two
     groups up to 32) and the first row counts of the GEMM path, against every weight-stream shape the
     skinny path distinguishes: rows of one to six 1 KiB segments (whole rows per wave), seven to twelve (two waves
     per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels."""
@@ -82,6 +83,9 @@ def test_decode_rows_every_stream_shape(orc, n, k):
         got, _ = _gpu_matmul(case, device_tensors=bool(m & 4))
         want = orc.matmul_int8(**case)
         assert np.array_equal(got, want), (m, n, k, int((got != want).sum()))
+        if m == 2:  # two rows on a handle without the blocked copy: the v_dot4 kernel instead of the matrix cores
+            got, _ = _gpu_matmul(case, device_tensors=True, decode_pack=False)
+            assert np.array_equal(got, want), ("no blocked copy", m, n, k)
 
 
 @pytest.mark.parametrize("m,n,k", [(2100, 6144, 1008), (3073, 4100, 144), (4096, 3072, 64), (2049, 6148, 400),
