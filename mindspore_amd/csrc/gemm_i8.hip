@@ -805,7 +805,7 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   }
   // A has exactly K valid bytes per row (the weights are zero padded, A is the caller's): in the last K block a
   // 16-byte chunk past K is fetched from the row's last chunk instead.  The offsets are moved there once, before
-  // that block is first requested (the re-fetches after it ask for the same block).
+  // that block is first requested (in the 256 x 256 form the re-fetches after it ask for the same block).
   const int a_last = (kchunks - 1) * 16 - (kblocks - 1) * KB;  // offset of the last valid chunk in the last block
   auto a_offsets_for_last_block = [&]() {
 #pragma unroll
@@ -923,7 +923,7 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(LPW + LPW / 2) : "memory");  // W(0) and A(0) are in
   read_frag(f0, 0, 0, 0);
   int ws = 0, ws1 = 1, ws2 = 2;  // W slots of blocks b, b+1, b+2
-  for (int b = 0; b < kblocks; ++b) {
+  auto k_block_clamped = [&](int b) {
     const int as = b & 1;
     const int kb1 = b + 1 < last ? b + 1 : last;  // past the end: the last block again, into a slot nobody reads
     const int kb2 = b + 2 < last ? b + 2 : last;
@@ -951,8 +951,53 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
     ws = ws1;
     ws1 = ws2;
     ws2 = t;
+  };
+  // One K block.  NEXT1 / NEXT2: blocks b + 1 / b + 2 exist.  The last two blocks have their own copies of the body
+  // without the loads for blocks that do not exist (with 6 K blocks those would be a third of the operand traffic),
+  // and the last one also without the barrier and the read-ahead.
+  auto k_block = [&](int b, auto next1_c, auto next2_c) {
+    constexpr bool NEXT1 = decltype(next1_c)::value, NEXT2 = decltype(next2_c)::value;
+    const int as = b & 1;
+    read_frag(f1, ws, as, 1);
+    if (NEXT1) dma_a(as ^ 1, b + 1, 1);
+    mma(f0, b * 8 + h);
+    hints();
+    read_frag(f0, ws, as, 2);
+    if (NEXT2) dma_w(ws2, b + 2, 0);
+    mma(f1, b * 8 + 2 + h);
+    hints();
+    read_frag(f1, ws, as, 3);
+    if (NEXT2) dma_w(ws2, b + 2, 1);
+    mma(f0, b * 8 + 4 + h);
+    hints();
+    if (NEXT2) {
+      // everything but the loads of W block b+2 has landed: that includes all of block b+1
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LPW) : "memory");
+    } else if (NEXT1) {
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // block b+1, the last one, is in
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (NEXT2 && b + 3 == kblocks) a_offsets_for_last_block();
+    if (NEXT1) read_frag(f0, ws1, as ^ 1, 0);
+    if (NEXT2) dma_a(as, b + 2, 0);
+    mma(f1, b * 8 + 6 + h);
+    hints();
+    const int t = ws;
+    ws = ws1;
+    ws1 = ws2;
+    ws2 = t;
+  };
+  if constexpr (T == 2) {
+    for (int b = 0; b + 2 < kblocks; ++b) k_block(b, std::true_type(), std::true_type());
+    if (kblocks >= 2) k_block(last - 1, std::true_type(), std::false_type());
+    k_block(last, std::false_type(), std::false_type());
+  } else {
+    // (three copies of the 64-MFMA body push the 256 x 256 tile's register allocation into spilling, and at its
+    //  K the two blocks' worth of extra loads are a few per cent: it keeps one body and lets the loads past the
+    //  end fetch the last block again, into slots nobody reads)
+    for (int b = 0; b < kblocks; ++b) k_block_clamped(b);
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the trailing re-fetches land before the LDS is reused
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every load has landed before the LDS is reused
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
   gemm_epilogue<TILE, T, T, EPI, HAS_ZW, FAST, kAccBias>(acc, rowsum, g, rq, dq, din, reinterpret_cast<const int *>(lds),
