@@ -661,8 +661,9 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   //                order, so that is "tile kt+1 has landed, later tiles may still be in flight"), then meet the other
   //                waves: now tile kt+1 is complete in LDS and nobody reads stage st-1 (tile kt-1) any more
   //   sub-step 1 : refill that stage with tile kt+PD, f0 <- sub-step 0 of tile kt+1, MFMAs on f1
-  // Past the end of K the loads re-fetch the last tile into a stage nobody reads again, which keeps the
-  // outstanding-load count the same in every step.
+  // With more than four stages the loads past the end of K re-fetch the last tile into a stage nobody reads again,
+  // which keeps the outstanding-load count the same in every step; with up to four the last steps are separate
+  // bodies without loads (see below).
   auto step = [&](int kt, int st) {
     read_frag(f1, st, 1);
     mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0, (kt * 4 + h < kchunks) ? 0x01010101 : 0);
@@ -705,8 +706,45 @@ __device__ __forceinline__ void gemm_direct_body(const GemmArgs &g, const Requan
   for (int t = 0; t < PD; ++t) dma_tile(t, t < ktiles ? t : ktiles - 1);
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((PD - 1) * LPW) : "memory");
   read_frag(f0, 0, 0);
-  for (int kt = 0, st = 0; kt < ktiles; ++kt, st = wrap(st + 1)) step(kt, st);
-  // (also: the trailing re-fetches must have landed before the LDS is reused below or handed to another workgroup)
+  if constexpr (NST <= 4) {
+    // The last PD steps have bodies of their own that load nothing: with a dozen K steps, as in the K = 768 shapes,
+    // re-fetching the last tile PD times is a fifth of the operand traffic.  REM = tiles after this one; the tiles
+    // still in flight at its wait are kt+2 .. the last one.
+    auto tail_step = [&](int kt, int st, auto rem_c) {
+      constexpr int REM = decltype(rem_c)::value;
+      read_frag(f1, st, 1);
+      mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f0, (kt * 4 + h < kchunks) ? 0x01010101 : 0);
+      hint_interleave_reads<TN, TM>();
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (REM >= 1) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((REM - 1) * LPW) : "memory");
+        asm volatile("s_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        read_frag(f0, wrap(st + 1), 0);
+      }
+      mma_frag<TN, TM, HAS_ZW>(acc, rowsum, f1, (kt * 4 + 2 + h < kchunks) ? 0x01010101 : 0);
+      hint_interleave_reads<TN, TM>();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    int kt = 0, st = 0;
+    for (; kt + PD < ktiles; ++kt, st = wrap(st + 1)) step(kt, st);
+    if constexpr (PD >= 3) {
+      if (ktiles - 1 - kt == 2) {
+        tail_step(kt, st, std::integral_constant<int, 2>());
+        ++kt;
+        st = wrap(st + 1);
+      }
+    }
+    if (ktiles - 1 - kt == 1) {
+      tail_step(kt, st, std::integral_constant<int, 1>());
+      ++kt;
+      st = wrap(st + 1);
+    }
+    tail_step(kt, st, std::integral_constant<int, 0>());
+  } else {
+    for (int kt = 0, st = 0; kt < ktiles; ++kt, st = wrap(st + 1)) step(kt, st);
+  }
+  // (also: every load must have landed before the LDS is reused below or handed to another workgroup)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   epi.to_lds(reinterpret_cast<int *>(lds), tid);
