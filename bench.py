@@ -8,7 +8,7 @@ requantising epilogue); the decode GEMV (configuration 4, batch 1), DynamicQuant
 timed region.  Prints ONE JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm4096|gemm8192] [--no-cpu] [--no-extra]
-                    [--calibrate] [--conv3x3] [--dynquant]
+                    [--calibrate] [--conv3x3] [--dynquant] [--bert] [--c2]
 """
 import argparse
 import json
@@ -43,6 +43,18 @@ def measured_traffic(workload):
     if "traffic_bytes_per_launch" not in kv:
         return None
     return dict(bytes=int(kv["traffic_bytes_per_launch"]), kernel=kv.get("kernel"), commit=kv.get("measured_at_commit"))
+
+
+def roofline_fields(ops, nbytes, ms):
+    """Where a launch of `ops` integer operations and `nbytes` algorithmic bytes that took `ms` stands against both
+    roofs; `bound` names the roof whose floor (ops / MFMA peak, bytes / HBM peak) is the higher one for this shape and
+    `frac` is the fraction of that roof."""
+    secs = ms * 1e-3
+    f_mfma = ops / secs / 1e12 / PEAK_INT8_TOPS if ops else 0.0
+    f_hbm = nbytes / secs / 1e9 / PEAK_HBM_GBPS
+    bound = "mfma" if ops / (PEAK_INT8_TOPS * 1e12) > nbytes / (PEAK_HBM_GBPS * 1e9) else "hbm"
+    return dict(bound=bound, frac=f_mfma if bound == "mfma" else f_hbm, ops=ops, algorithmic_bytes=int(nbytes),
+                frac_of_int8_peak=f_mfma, frac_of_hbm_peak=f_hbm)
 
 
 def host_cores():
@@ -176,11 +188,19 @@ def bench_gemm(size, steps, warmup, host_path=False, sustained=False):
     a = torch.from_numpy(c["a"]).cuda()
     out = torch.empty((size, size), dtype=torch.int8, device="cuda")
     probe = sustained_probe() if sustained else None
+    ops = 2.0 * size * size * size
+    # first the region exactly as asked for, straight from the idle device (0.2 s without GPU work precede it): this
+    # is the power management's transient (see settle), reported beside the settled figure
+    torch.cuda.synchronize()
+    time.sleep(0.2)
+    idle_ms, _ = time_steps(lambda: kern.run(a, out=out), steps, warmup)
+    from_idle = dict(ms_per_step=idle_ms, tops=ops / (idle_ms * 1e-3) / 1e12,
+                     frac_of_int8_peak=ops / (idle_ms * 1e-3) / 1e12 / PEAK_INT8_TOPS, steps=steps, warmup=warmup,
+                     note="the same timed region started from an idle device, before the untimed settling launches")
     settled = settle(kern, a, out, chunk=50 if size <= 4096 else 10)
     ev_ms, host_ms = time_steps(lambda: kern.run(a, out=out), steps, warmup)
-    ops = 2.0 * size * size * size
     res = dict(ms=ev_ms, host_ms=host_ms, tops=ops / (ev_ms * 1e-3) / 1e12, ops=ops, case=c, prepare_ms=prepare_ms,
-               settled=settled)
+               settled=settled, from_idle=from_idle)
     if sustained:
         res["sustained"] = bench_sustained(kern, a, out, size, probe)
     if host_path:
@@ -298,13 +318,12 @@ def bench_bert(steps, warmup):
     dq = K.DynamicQuantKernel(False)
     ms = time_in_graph(lambda: dq.run(x, fetch_params=False), steps, warmup)
     nbytes = x.numel() * 5
-    out["dynquant_4096x768"] = dict(ms=ms, gbps=nbytes / (ms * 1e-3) / 1e9, frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS)
+    out["dynquant_4096x768"] = dict(ms=ms, gbps=nbytes / (ms * 1e-3) / 1e9, **roofline_fields(0, nbytes, ms))
     # the same two kernels on a tensor large enough to leave the launch-latency regime (16x the BERT activation)
     xl = torch.randn((65536, 768), device="cuda", dtype=torch.float32)
     ms, _ = time_steps(lambda: dq.run(xl, fetch_params=False), steps, warmup)
     nbytes = xl.numel() * 5
-    out["dynquant_65536x768"] = dict(ms=ms, gbps=nbytes / (ms * 1e-3) / 1e9,
-                                     frac_of_hbm_peak=nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+    out["dynquant_65536x768"] = dict(ms=ms, gbps=nbytes / (ms * 1e-3) / 1e9, **roofline_fields(0, nbytes, ms),
                                      note="algorithmic bytes (4 read + 1 written per element); the second pass re-reads "
                                           "201 MB, of which the Infinity Cache holds only part")
     del xl
@@ -316,10 +335,13 @@ def bench_bert(steps, warmup):
         qa = q if k == 768 else torch.randint(-128, 127, (4096, k), dtype=torch.int8, device="cuda")
         ms = time_in_graph(lambda: mm.run(qa, params_dev=dq.device_params()), steps, warmup)
         ops = 2.0 * 4096 * n * k
-        out["dynmm_" + name] = dict(ms=ms, tops=ops / (ms * 1e-3) / 1e12)
+        nbytes = 4096 * k + n * k + 4 * 4096 * n + 12 * n  # int8 activations and weights, fp32 output, per-channel scale / sum / bias
+        out["dynmm_" + name] = dict(ms=ms, tops=ops / (ms * 1e-3) / 1e12, gbps=nbytes / (ms * 1e-3) / 1e9,
+                                    **roofline_fields(ops, nbytes, ms))
         total_ops += ops
         total_ms += ms
     out["dynmm_total_tops"] = total_ops / (total_ms * 1e-3) / 1e12
+    out["dynmm_total_us"] = total_ms * 1e3
     return out
 
 
@@ -336,7 +358,8 @@ def bench_small_configs(steps, warmup):
     a = torch.from_numpy(c["a"]).cuda()
     o = torch.empty((128, 768), dtype=torch.int8, device="cuda")
     ms = time_in_graph(lambda: fc.run(a, out=o), steps, warmup)
-    out["c1_fc_128x768x768"] = dict(us=ms * 1e3, tops=2.0 * 128 * 768 * 768 / (ms * 1e-3) / 1e12)
+    out["c1_fc_128x768x768"] = dict(us=ms * 1e3, tops=2.0 * 128 * 768 * 768 / (ms * 1e-3) / 1e12,
+                                    **roofline_fields(2.0 * 128 * 768 * 768, 128 * 768 + 768 * 768 + 128 * 768 + 16 * 768, ms))
     x, layers = wl.mobilenet_c2()
     cur = torch.from_numpy(x).cuda()
     kerns, ins = [], []
@@ -349,11 +372,15 @@ def bench_small_configs(steps, warmup):
         ins.append(cur)
         cur = kern.run(cur)
     outs = [kern.run(xin) for kern, xin in zip(kerns, ins)]
+    block_bytes, block_ops = 0, 0.0
     for L, kern, xin, yout in zip(layers, kerns, ins, outs):
         ms = time_in_graph(lambda: kern.run(xin, out=yout), steps, warmup)
-        nbytes = xin.numel() + yout.numel() + L["w"].size
+        nbytes = xin.numel() + yout.numel() + L["w"].size + 16 * L["oc"]
+        kdim = L["kernel"] ** 2 * (1 if L["kind"] == "dw" else L["ic"])
         out["c2_" + L["name"]] = dict(us=ms * 1e3, in_shape=list(xin.shape), out_shape=list(yout.shape),
-                                      algorithmic_bytes=nbytes)
+                                      gbps=nbytes / (ms * 1e-3) / 1e9, **roofline_fields(2.0 * yout.numel() * kdim, nbytes, ms))
+        block_bytes += nbytes
+        block_ops += 2.0 * yout.numel() * kdim
     # the whole block as one captured HIP graph (five kernels), replayed: what the GPU needs once the host's
     # per-call cost is out of the way
     def chain():
@@ -370,11 +397,15 @@ def bench_small_configs(steps, warmup):
     ms, _ = time_steps(graph.replay, steps, warmup)
     total_us = ms * 1e3
     out["c2_block_graph_us"] = total_us
+    out["c2_block"] = dict(us=total_us, kernels=len(kerns), gbps=block_bytes / (total_us * 1e-6) / 1e9,
+                           note="stem, expand, depthwise and project replayed as one HIP graph; algorithmic bytes are "
+                                "the sum over the four layers (every intermediate tensor written once and read once)",
+                           **roofline_fields(block_ops, block_bytes, ms))
     # a mid-network 3x3 convolution: the GEMM gathers its activation operand from the image
     kern, xin, yout, nbytes = make_conv3x3()
     us = time_in_graph(lambda: kern.run(xin, out=yout), steps, 3) * 1e3
     out["conv3x3_b32_56x56x64"] = dict(us=us, tops=2.0 * yout.numel() * 9 * 64 / (us * 1e-6) / 1e12,
-                                       algorithmic_bytes=nbytes)
+                                       **roofline_fields(2.0 * yout.numel() * 9 * 64, nbytes, us * 1e-3))
     return out
 
 
@@ -419,9 +450,11 @@ def cpu_baseline(case, size):
         return 2.0 * rows * size * size / secs / 1e12, secs
 
     rows = 1024 if size <= 4096 else 256
-    tops, secs = run(rows, cores)
+    runs = sorted(run(rows, cores) for _ in range(3))  # median of three
+    tops, secs = runs[1]
     tops1, secs1 = run(64 if size <= 4096 else 16, 1)
     return dict(value=tops, unit="TOP/s", cores=cores, nproc=nproc, kind=kind, seconds=secs,
+                runs_tops=[r[0] for r in runs], statistic="median of 3 runs",
                 sample="first %d of %d activation rows of the same %d^3 GEMM (A-pack + row sums + MatmulInt8Opt "
                        "column stripes on %d threads)" % (rows, size, size, cores),
                 single_thread=dict(value=tops1, unit="TOP/s", cores=1, seconds=secs1,
@@ -498,6 +531,11 @@ def main():
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--conv3x3", action="store_true",
                     help="also launch the batch-32 3x3 convolution of the extras 20 times (for profiling that kernel)")
+    ap.add_argument("--bert", action="store_true",
+                    help="also launch each of the four BERT dynamic MatMuls of configuration 3 twenty times (for "
+                         "profiling their kernels; mindspore_amd/native_bench bert does the same without Python)")
+    ap.add_argument("--c2", action="store_true",
+                    help="also run the four layers of configuration 2 twenty times each (for profiling their kernels)")
     ap.add_argument("--dynquant", action="store_true",
                     help="also run DynamicQuant on the 4096 x 768 activation of configuration 3 a hundred times (for "
                          "profiling its two kernels)")
@@ -545,9 +583,10 @@ def main():
         nread = native_bench("read", 48, 64, 4)
         if nread and "gbps" in nread:
             extra["hbm_read_stream_native_host"] = nread
-        for m in (1, 8, 32):
+        for m in (1, 2, 4, 8, 32):
             nat = native_bench("decode", m, 3, 1000, 100)  # ~0.1 s of launches after ~10 ms of warm-up: the settled rate
-            py = section("gemv_decode_m%d_python_host" % m, lambda: bench_gemv(max(5, args.steps // 2), 3, m))
+            py = section("gemv_decode_m%d_python_host" % m, lambda: bench_gemv(max(5, args.steps // 2), 3, m)) \
+                if m in (1, 8) else None
             if nat and "gbps" in nat:
                 best = dict(nat, host="native C++ over the C ABI")
             elif py:
@@ -562,6 +601,7 @@ def main():
                 solo = native_bench("decode", m, 3, 1000, 100, env={"NATIVE_BENCH_NO_GROUP": "1"})
                 if solo and "gbps" in solo:
                     best["one_launch_per_matrix"] = dict(ms_per_step=solo["ms_per_step"], gbps=solo["gbps"],
+                                                         frac_of_hbm_peak=solo["gbps"] / PEAK_HBM_GBPS,
                                                          launches_per_step=solo["launches_per_step"])
             extra["gemv_decode_m%d" % m] = best
         warm = native_bench("warm", 1, 200, 20)
@@ -583,6 +623,7 @@ def main():
                    "device_state": "settled: %d untimed launches (%.0f ms) from idle precede the warm-up, see "
                                    "settled_before_timing" % (g["settled"]["launches"], g["settled"]["ms"])},
         "settled_before_timing": g["settled"],
+        "from_idle_before_settling": g["from_idle"],
         "roofline": {"bound": "mfma", "achieved": g["tops"], "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": g["tops"] / PEAK_INT8_TOPS, "traffic": None,
                      "kernel": HEADLINE_KERNEL, "ops_per_launch": g["ops"]},
@@ -607,6 +648,32 @@ def main():
         dq = K.DynamicQuantKernel(False)
         for _ in range(100):
             dq.run(xq, fetch_params=False)
+        torch.cuda.synchronize()
+    if args.bert:
+        from mindspore_amd import kernels as K
+        from mindspore_amd import workloads as wl
+        dq = K.DynamicQuantKernel(False)
+        q, _ = dq.run(torch.from_numpy(wl.bert_c3_activation(768)).cuda(), fetch_params=False)
+        for name, n, k in wl.BERT_SHAPES:
+            wt = wl.bert_c3_weights(name, n, k)
+            mm = K.MatmulDynamicInt8Kernel(wt["w"], wt["bias"], [K.QuantParam(float(sc), 0) for sc in wt["sw"]])
+            qa = q if k == 768 else torch.randint(-128, 127, (4096, k), dtype=torch.int8, device="cuda")
+            for _ in range(20):
+                mm.run(qa, params_dev=dq.device_params())
+        torch.cuda.synchronize()
+    if args.c2:
+        from mindspore_amd import kernels as K
+        from mindspore_amd import workloads as wl
+        x, layers = wl.mobilenet_c2()
+        cur = torch.from_numpy(x).cuda()
+        for L in layers:
+            qp = [K.QuantParam(float(sc), int(z)) for sc, z in zip(L["sw"], L["zw"])]
+            kern = K.ConvolutionInt8Kernel(L["w"], L["bias"], K.QuantParam(L["sx"], L["zx"]), qp,
+                                           K.QuantParam(L["so"], L["zo"]), (L["stride"],) * 2, (1, 1), L["pad"],
+                                           L["oc"] if L["kind"] == "dw" else 1, L["act"])
+            for _ in range(20):
+                nxt = kern.run(cur)
+            cur = nxt
         torch.cuda.synchronize()
     if args.conv3x3:
         kern, xin, yout, _ = make_conv3x3()

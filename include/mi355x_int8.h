@@ -51,6 +51,13 @@ extern "C" {
 int mi_init(int device);
 /* Message of the last failure on the calling thread ("" if none). */
 const char *mi_last_error(void);
+/* Test aid: while `bytes` is non-zero, every device allocation the library makes for a handle (packed weights,
+ * parameters, workspaces) whose size, rounded up to 4 KiB, equals `bytes` rounded up to 4 KiB fails as if the device
+ * were out of memory; 0 switches it off.  Lets a test show what a handle does when one of its allocations fails. */
+int mi_debug_fail_alloc(size_t bytes);
+/* Test aid: how many times the library has made the host wait for a stream so far (mi_copy_to_device, mi_copy_to_host,
+ * mi_stream_synchronize, mi_dynquant_get_params; the *_run_host entry points are not counted). */
+int64_t mi_debug_sync_count(void);
 const char *mi_version(void);
 
 /* ---- quant-parameter derivation (host arithmetic, no GPU needed) -------------------------------------------- */
@@ -97,6 +104,8 @@ typedef struct mi_matmul_desc {
   const double *filter_scales; /* [filter_quant_num] */
   const int32_t *filter_zps;   /* [filter_quant_num] */
   int32_t flags;               /* 0 or MI_MATMUL_NO_DECODE_PACK */
+  int32_t b_batch;             /* 0 or 1: one weight matrix; > 1: weight_host holds this many [deep x col] matrices
+                                  one after the other (a constant weight of rank > 2) */
 } mi_matmul_desc;
 
 /* All weight packing happens in mi_matmul_create (the role of TransferB, LK/int8/matmul_base_int8.cc:360-384: pack
@@ -114,10 +123,26 @@ int mi_matmul_create(const mi_matmul_desc *desc, const int8_t *weight_host, cons
  * the buffers MatmulBaseInt8CPUKernel::ReSize allocates (LK/int8/matmul_base_int8.cc:296-325).  Workspaces exist only
  * for operand shapes the kernels cannot take in place (deep % 16 != 0 or a misaligned activation base: a padded copy
  * of the activations; col % 4 != 0 or a misaligned output base: a padded output).  Without this call the first run
- * that needs a larger workspace allocates it (hipFree + hipMalloc: the device idles meanwhile). */
+ * that needs a larger workspace allocates it with hipMalloc, at least twice the previous size; the outgrown buffer
+ * may still be in use by kernels in flight, so it is kept until the handle is destroyed (a handle therefore holds at
+ * most about twice its largest workspace; the same holds for the im2col and output workspaces of mi_conv). */
 int mi_matmul_reserve(mi_matmul *h, int32_t max_rows);
 /* a_dev: int8 [rows, deep]; c_dev: int8 [rows, col].  Asynchronous on `stream`. */
 int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev, void *stream);
+/* Batched MatMul (MatmulBaseInt8CPUKernel::Run, LK/int8/matmul_base_int8.cc:549-568): output matrix i =
+ * activation matrix a_offsets[i] x weight matrix b_offsets[i], for i = 0 .. batch-1.  a_dev holds [rows, deep]
+ * matrices one after the other, c_dev receives `batch` [rows, col] matrices, the weight matrices are those given to
+ * mi_matmul_create (desc.b_batch).  The offsets are what MatmulFp32BaseCPUKernel::InitBroadcastParams
+ * (LK/fp32/matmul_fp32_base.cc:576-646) derives from the two shapes; mi_matmul_broadcast_offsets computes them. */
+int mi_matmul_run_batched(mi_matmul *h, const int8_t *a_dev, int32_t rows, int32_t batch, const int32_t *a_offsets,
+                          const int32_t *b_offsets, int8_t *c_dev, void *stream);
+/* The batch broadcast rule of MatMul (InitBroadcastParams, LK/fp32/matmul_fp32_base.cc:576-646; host arithmetic, no
+ * GPU needed): for operand shapes a_shape / b_shape (the last two extents are the matrix) the number of output
+ * matrices and, per output matrix, the index of the activation and of the weight matrix it is made of.  a_offsets /
+ * b_offsets have room for `capacity` entries; MI_PARAM_INVALID when the batch extents cannot be broadcast or the
+ * result does not fit. */
+int mi_matmul_broadcast_offsets(const int32_t *a_shape, int32_t a_dims, const int32_t *b_shape, int32_t b_dims,
+                                int32_t capacity, int32_t *batch, int32_t *a_offsets, int32_t *b_offsets);
 /* mi_matmul_run for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments, same results; instead of the
  * handle's growable workspaces it uses one scratch area of MI_NOALLOC_SCRATCH_BYTES of static device memory (held by
@@ -244,7 +269,23 @@ typedef struct mi_dynmm_desc {
   int32_t filter_quant_num; /* 1 or col; the zero point used is always filter_zps[0] (matmul_dynamic_int8.cc:52) */
   const double *filter_scales;
   const int32_t *filter_zps;
+  int32_t flags;               /* 0 or MI_DYNMM_WEIGHT_PACKED_SDOT */
+  const int32_t *weight_sums;  /* with MI_DYNMM_WEIGHT_PACKED_SDOT: the model's weight-sums tensor
+                                  [round_up(col, 16)], or NULL to have the sums computed from the weight */
 } mi_dynmm_desc;
+
+/* The weight arrives as a model converted with `cpu_option = ARM64_SIMD_DOT` stores it: packed offline for
+ * MatMulDynamicSdotInt8Kernel by RowMajor2Row4x16MajorInt8 (transpose_b) or RowMajor2Col4x16MajorInt8 (NN/int8/
+ * matmul_int8.c:143-156,770-784; LK/int8/matmul_dynamic_sdot_int8.cc:197-201) -- both produce the same bytes,
+ * [round_up(col, 16) / 16][round_up(deep, 4) / 4][16 channels][4 K-bytes], zero padded -- together with a tensor of
+ * per-channel weight sums (mindspore/lite/tools/converter/converter_packed_node.cc:47-70,129-141).  The reference
+ * takes both as they are (weight_is_packed_, LK/int8/matmul_dynamic_base_int8.cc:178-184,439-443); this library
+ * unpacks the weight once in mi_dynmm_create, on the host (the inverse that MatmulDynamicSdotInt8Unpack computes,
+ * mindspore/lite/src/litert/runtime_packed_node_pass.cc:158-192), repacks it into its own layout and uses the given
+ * sums.  b_transpose is ignored with this flag. */
+#define MI_DYNMM_WEIGHT_PACKED_SDOT 1
+/* The unpacking by itself (host arithmetic, no GPU needed): packed -> weight_nk [col][deep] row-major. */
+int mi_unpack_weight_4x16(const int8_t *packed, int32_t col, int32_t deep, int8_t *weight_nk);
 
 /* bias_host: fp32 [col] or NULL */
 int mi_dynmm_create(const mi_dynmm_desc *desc, const int8_t *weight_host, const float *bias_host, mi_dynmm **out);
@@ -324,6 +365,10 @@ int mi_host_free(void *host); /* NULL is allowed */
 int mi_device_free(void *dev); /* NULL is allowed */
 int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *stream);
 int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *stream);
+/* The same copy without the wait: it is ordered on `stream` and complete once something has waited for the stream
+ * (mi_stream_synchronize, a later mi_copy_to_host).  dst_host should be page-locked memory from mi_host_malloc;
+ * into ordinary memory the runtime may make the call wait after all. */
+int mi_copy_to_host_async(void *dst_host, const void *src_dev, size_t bytes, void *stream);
 int mi_stream_synchronize(void *stream);
 /* A HIP stream of the library's device (default priority, not ordered against the null stream) and its release.  A
  * provider gives every session (every mindspore::Context it is handed) a stream of its own and passes it to all run

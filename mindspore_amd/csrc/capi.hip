@@ -8,6 +8,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <memory>
 #include <new>
 #include <vector>
@@ -19,6 +20,13 @@ namespace mi {
 
 static thread_local char g_err[512] = "";
 static int g_device = -1;
+// how often the library made the host wait for a stream (mi_debug_sync_count): the copies with host tensors, the
+// parameter fetch of DynamicQuant, mi_stream_synchronize
+static std::atomic<int64_t> g_sync_count{0};
+static hipError_t counted_sync(hipStream_t s) {
+  g_sync_count.fetch_add(1, std::memory_order_relaxed);
+  return hipStreamSynchronize(s);
+}
 
 // Scratch memory of mi_matmul_run_noalloc: static device memory, so the entry point never allocates.  Every GPU the
 // library is initialised on holds its own copy of the array at its own address; the array's name is only a host-side
@@ -110,6 +118,16 @@ static void activation_range(int act, int32_t zp, float scale, int32_t *mn, int3
 // kernels still in flight that use the old memory, so the old allocation is neither freed there -- hipFree waits for
 // the whole device -- nor reused: it is kept until the handle goes away, and the size at least doubles, which bounds
 // what is kept to the final size once more.
+// Test aid (mi_debug_fail_alloc): while set, every DevBuf allocation of exactly this many bytes fails.
+static size_t g_fail_alloc_bytes = 0;
+static hipError_t device_alloc(void **q, size_t sz) {
+  if (g_fail_alloc_bytes != 0 && sz == g_fail_alloc_bytes) {
+    *q = nullptr;
+    return hipErrorOutOfMemory;
+  }
+  return hipMalloc(q, sz);
+}
+
 struct DevBuf {
   void *p = nullptr;
   size_t bytes = 0;
@@ -123,10 +141,10 @@ struct DevBuf {
     size_t sz = p != nullptr && want < 2 * bytes ? 2 * bytes : want;
     sz = (sz + 4095) & ~(size_t)4095;
     void *q = nullptr;
-    if (hipMalloc(&q, sz) != hipSuccess) {
+    if (device_alloc(&q, sz) != hipSuccess) {
       (void)hipGetLastError();
       sz = (want + 4095) & ~(size_t)4095;  // the doubled size did not fit: exactly what is needed
-      if (hipMalloc(&q, sz) != hipSuccess) {
+      if (device_alloc(&q, sz) != hipSuccess) {
         (void)hipGetLastError();
         set_error("hipMalloc(%zu) failed", sz);
         return MI_MEMORY_FAILED;
@@ -191,7 +209,7 @@ struct RequantState {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
   DevBuf mult2, c2lo, c2hi, pre;  // the GEMM epilogue's per-channel constants (RequantParams::fast2)
-  DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (3..32 activation rows); built in create or absent
+  DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (2..32 activation rows); built in create or absent
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
   bool has_zw = false, fast = false, fast2 = false;
@@ -255,13 +273,15 @@ struct RequantState {
       const int64_t vmax = std::min<int64_t>((int64_t)1 << 31, (int64_t)k * 16384 + llabs((long long)h_bias2[c]) +
                                                                    (int64_t)k * 128 * llabs((long long)zwv[c]));
       const int64_t xmax = ((vmax * llabs((long long)h_mult[c])) >> 31) + 1;
-      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN || vmax + kAccBias >= ((int64_t)1 << 31) ||
+      if (h_ls[c] != 0 || e[c] < 1 || e[c] > 30 || h_mult[c] == INT32_MIN || vmax >= ((int64_t)1 << 31) ||
           xmax + ((int64_t)1 << (e[c] - 1)) + (llabs((long long)zo) << e[c]) > INT32_MAX)
         fast = false;
     }
     for (int c = n; c < n_pad; ++c) e[c] = 1;
     if (amin > amax) fast = false;
-    // constants of the GEMM's single-multiply rounding form (RequantParams::fast2)
+    // constants of the GEMM's single-multiply rounding form (RequantParams::fast2).  Only that form reads the
+    // accumulator register with kAccBias still in it, so the room for kAccBias is its condition alone (the first test
+    // in the loop below: sum and row-sum term together stay within +-kAccBias, hence the register within [0, 2^31)).
     fast2 = fast;
     std::vector<uint32_t> m2(n_pad, 0), lo(n_pad, 0), hi(n_pad, 0);
     std::vector<int32_t> prev(n_pad, 0);
@@ -296,11 +316,19 @@ struct RequantState {
       for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * ldw, w_nk + (size_t)c * k, (size_t)k);
       if ((rc = upload(&w, packed)) != MI_OK) return rc;
       if (pack_decode) {
-        if ((rc = w_blocked.ensure((size_t)n_pad * k_pad)) != MI_OK) return rc;
-        rc = launch_block_weights(static_cast<const int8_t *>(w.p), n_pad, k_pad, ldw, static_cast<int8_t *>(w_blocked.p),
-                                  nullptr);
-        if (rc != MI_OK) return rc;
-        MI_HIP_CHECK(hipStreamSynchronize(nullptr));  // runs may come in on any stream
+        // The blocked copy is an optimisation for 2..32 activation rows, not a requirement: without it those row
+        // counts run on the v_dot4 kernel (two rows) or the GEMM tiles.  A device that has no room for it still gets
+        // a working handle.
+        rc = w_blocked.ensure((size_t)n_pad * k_pad);
+        if (rc == MI_OK)
+          rc = launch_block_weights(static_cast<const int8_t *>(w.p), n_pad, k_pad, ldw,
+                                    static_cast<int8_t *>(w_blocked.p), nullptr);
+        if (rc == MI_OK && hipStreamSynchronize(nullptr) != hipSuccess) rc = MI_ERROR;  // runs may come in on any stream
+        if (rc != MI_OK) {
+          (void)hipGetLastError();
+          w_blocked.release();
+          set_error("");
+        }
       }
     }
     return MI_OK;
@@ -347,6 +375,22 @@ static std::vector<int8_t> to_nk(const int8_t *w, int n, int k, int b_transpose)
   return out;
 }
 
+// The weight layout that a model converted for the ARM dot-product kernel carries (RowMajor2Row4x16MajorInt8 for
+// transpose_b, RowMajor2Col4x16MajorInt8 otherwise, nnacl/int8/matmul_int8.c:143-156,770-784; both give the same
+// bytes): blocks [n / 16][k / 4] of 16 channels x 4 K-bytes, channel-major inside a block, with the channel count
+// padded to 16 and K to 4.  Returns [n][k] row-major (the inverse that MatmulDynamicSdotInt8Unpack computes,
+// mindspore/lite/src/litert/runtime_packed_node_pass.cc:158-192).
+static std::vector<int8_t> unpack_4x16(const int8_t *packed, int n, int k) {
+  const size_t k4 = (size_t)round_up(k, 4);
+  std::vector<int8_t> out((size_t)n * k);
+  for (int c = 0; c < n; ++c) {
+    const int8_t *blk = packed + (size_t)(c / 16) * k4 * 16 + (size_t)(c % 16) * 4;
+    int8_t *row = out.data() + (size_t)c * k;
+    for (int i = 0; i < k; ++i) row[i] = blk[(size_t)(i / 4) * 64 + (i % 4)];
+  }
+  return out;
+}
+
 // Activations must reach the GEMM/GEMV kernels as 16-byte aligned rows of k16 bytes; returns the pointer/stride to
 // use, copying through `ws` when the caller's layout does not qualify.
 static int prepare_rows(const int8_t *a, int rows, int k, const Workspace &ws, hipStream_t stream,
@@ -375,8 +419,8 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
                             const Workspace &c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
-  // up to 2 rows: the dot kernel on the row-major weights; 3..32 rows: the matrix-core decode kernel on the blocked
-  // copy made at create time -- a handle created without it runs those row counts on the GEMM tiles
+  // one row: the dot kernel on the row-major weights; 2..32 rows: the matrix-core decode kernel on the blocked copy
+  // made at create time -- a handle without it runs two rows on the dot kernel and 3..32 on the GEMM tiles
   const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
                                            : rows <= kGemvMaxRows && st.w_blocked.p != nullptr;
   if (skinny) {
@@ -400,8 +444,11 @@ using namespace mi;
 
 // =====================================================================================================================
 struct mi_matmul {
-  RequantState st;
+  RequantState st;  // weight matrix 0
+  std::vector<std::unique_ptr<RequantState>> more;  // weight matrices 1 .. b_batch - 1 of a batched constant weight
   DevBuf a_ws, c_ws, h_in, h_out;
+  int b_batch() const { return 1 + (int)more.size(); }
+  RequantState &state(int b) { return b == 0 ? st : *more[(size_t)b - 1]; }
 };
 
 struct mi_conv {
@@ -522,7 +569,7 @@ int mi_copy_to_device(void *dst_dev, const void *src_host, size_t bytes, void *s
   if (ensure_device() != MI_OK) return MI_ERROR;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI_HIP_CHECK(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, s));
-  MI_HIP_CHECK(hipStreamSynchronize(s));  // the caller may reuse src_host at once (the runtime recycles tensor memory)
+  MI_HIP_CHECK(counted_sync(s));  // the caller may reuse src_host at once (the runtime recycles tensor memory)
   return MI_OK;
 }
 
@@ -532,9 +579,19 @@ int mi_copy_to_host(void *dst_host, const void *src_dev, size_t bytes, void *str
   if (ensure_device() != MI_OK) return MI_ERROR;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI_HIP_CHECK(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, s));
-  MI_HIP_CHECK(hipStreamSynchronize(s));
+  MI_HIP_CHECK(counted_sync(s));
   return MI_OK;
 }
+
+int mi_copy_to_host_async(void *dst_host, const void *src_dev, size_t bytes, void *stream) {
+  if (bytes == 0) return MI_OK;
+  if (dst_host == nullptr || src_dev == nullptr) return MI_NULL_PTR;
+  if (ensure_device() != MI_OK) return MI_ERROR;
+  MI_HIP_CHECK(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+  return MI_OK;
+}
+
+int64_t mi_debug_sync_count(void) { return g_sync_count.load(std::memory_order_relaxed); }
 
 int mi_stream_create(void **out_stream) {
   if (out_stream == nullptr) return MI_NULL_PTR;
@@ -555,7 +612,12 @@ int mi_stream_destroy(void *stream) {
 
 int mi_stream_synchronize(void *stream) {
   if (ensure_device() != MI_OK) return MI_ERROR;
-  MI_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  MI_HIP_CHECK(counted_sync(static_cast<hipStream_t>(stream)));
+  return MI_OK;
+}
+
+int mi_debug_fail_alloc(size_t bytes) {
+  g_fail_alloc_bytes = bytes == 0 ? 0 : (bytes + 4095) & ~(size_t)4095;
   return MI_OK;
 }
 
@@ -627,12 +689,23 @@ static int mi_matmul_create_impl(const mi_matmul_desc *d, const int8_t *weight_h
   std::unique_ptr<mi_matmul> owner(new (std::nothrow) mi_matmul());  // the buffers free themselves if anything below throws
   mi_matmul *h = owner.get();
   if (h == nullptr) return MI_MEMORY_FAILED;
-  const std::vector<int8_t> w_nk = to_nk(weight_host, d->col, d->deep, d->b_transpose);
-  rc = h->st.build(w_nk.data(), d->col, d->deep, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
-                   d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true,
-                   (d->flags & MI_MATMUL_NO_DECODE_PACK) == 0);
-  if (rc != MI_OK) {
-    return rc;
+  if (d->b_batch < 0 || d->b_batch > (1 << 16)) {
+    set_error("mi_matmul_create: b_batch=%d", d->b_batch);
+    return MI_PARAM_INVALID;
+  }
+  // every matrix of a batched weight gets its own packed copy and folded bias; quant parameters and bias are shared
+  // (TransferB, LK/int8/matmul_base_int8.cc:360-384)
+  const int b_batch = d->b_batch > 1 ? d->b_batch : 1;
+  for (int b = 0; b < b_batch; ++b) {
+    if (b > 0) {
+      h->more.emplace_back(new (std::nothrow) RequantState());
+      if (h->more.back() == nullptr) return MI_MEMORY_FAILED;
+    }
+    const std::vector<int8_t> w_nk = to_nk(weight_host + (size_t)b * d->col * d->deep, d->col, d->deep, d->b_transpose);
+    rc = h->state(b).build(w_nk.data(), d->col, d->deep, bias_host, d->in_scale, d->in_zp, d->out_scale, d->out_zp,
+                           d->filter_quant_num, d->filter_scales, d->filter_zps, d->act_type, true,
+                           (d->flags & MI_MATMUL_NO_DECODE_PACK) == 0);
+    if (rc != MI_OK) return rc;
   }
   *out = owner.release();
   return MI_OK;
@@ -670,6 +743,44 @@ int mi_matmul_run(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_t *c_dev
   int k16 = 0;
   if ((rc = prepare_rows(a_dev, rows, h->st.k, Workspace::growable(&h->a_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
   return run_requant_gemm(h->st, a, lda, rows, k16, c_dev, Workspace::growable(&h->c_ws), s);
+}
+
+int mi_matmul_run_batched(mi_matmul *h, const int8_t *a_dev, int32_t rows, int32_t batch, const int32_t *a_offsets,
+                          const int32_t *b_offsets, int8_t *c_dev, void *stream) {
+  if (h == nullptr || a_dev == nullptr || c_dev == nullptr || a_offsets == nullptr || b_offsets == nullptr) {
+    set_error("mi_matmul_run_batched: null argument");
+    return MI_NULL_PTR;
+  }
+  if (rows < 0 || batch < 0) {
+    set_error("mi_matmul_run_batched: rows=%d batch=%d", rows, batch);
+    return MI_PARAM_INVALID;
+  }
+  for (int i = 0; i < batch; ++i) {
+    if (a_offsets[i] < 0 || b_offsets[i] < 0 || b_offsets[i] >= h->b_batch()) {
+      set_error("mi_matmul_run_batched: output matrix %d takes activation matrix %d and weight matrix %d of %d", i,
+                a_offsets[i], b_offsets[i], h->b_batch());
+      return MI_PARAM_INVALID;
+    }
+  }
+  if (rows == 0 || batch == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const size_t a_mat = (size_t)rows * h->st.k, c_mat = (size_t)rows * h->st.n;
+  // one launch per output matrix, in order on the stream (so the shared workspaces are reused safely), as the
+  // reference runs one ParallelLaunch per batch (LK/int8/matmul_base_int8.cc:549-568)
+  for (int i = 0; i < batch; ++i) {
+    const int8_t *a = nullptr;
+    int64_t lda = 0;
+    int k16 = 0;
+    if ((rc = prepare_rows(a_dev + (size_t)a_offsets[i] * a_mat, rows, h->st.k, Workspace::growable(&h->a_ws), s, &a, &lda,
+                           &k16)) != MI_OK)
+      return rc;
+    if ((rc = run_requant_gemm(h->state(b_offsets[i]), a, lda, rows, k16, c_dev + (size_t)i * c_mat,
+                               Workspace::growable(&h->c_ws), s)) != MI_OK)
+      return rc;
+  }
+  return MI_OK;
 }
 
 int mi_matmul_run_group(mi_matmul *const *handles, int32_t count, const int8_t *a_dev, int32_t rows,
@@ -741,8 +852,9 @@ int mi_matmul_run_noalloc(mi_matmul *h, const int8_t *a_dev, int32_t rows, int8_
     set_error("mi_matmul_run_noalloc: no scratch memory on device %d", g_device);
     return MI_ERROR;
   }
-  // the padded activation rows first, the padded output behind them; a part is only used when the operand's shape
-  // or address needs it, but the size check does not depend on the pointers of this particular call
+  // the padded activation rows first, the padded output behind them; a part is only needed when the operand's shape
+  // or this call's pointer alignment asks for it, and only the needed parts count against the maximum (so a shape
+  // that passes with aligned pointers can be refused with misaligned ones)
   const size_t a_bytes = round_up64((int64_t)rows * round_up(h->st.k, 16), 256);
   const size_t c_bytes = (size_t)rows * round_up(h->st.n, 4);
   const bool a_padded = (h->st.k & 15) != 0, c_padded = (h->st.n & 3) != 0;
@@ -1050,7 +1162,7 @@ int mi_dynquant_get_params(mi_dynquant *h, void *stream, mi_dq_params *params_ho
   if (rc != MI_OK) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI_HIP_CHECK(hipMemcpyAsync(params_host, h->params.p, sizeof(mi_dq_params), hipMemcpyDeviceToHost, s));
-  MI_HIP_CHECK(hipStreamSynchronize(s));
+  MI_HIP_CHECK(counted_sync(s));
   return MI_OK;
 }
 
@@ -1127,6 +1239,10 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
     set_error("mi_dynmm_create: bad shape/activation");
     return MI_PARAM_INVALID;
   }
+  if ((d->flags & ~MI_DYNMM_WEIGHT_PACKED_SDOT) != 0) {
+    set_error("mi_dynmm_create: unknown flags 0x%x", d->flags);
+    return MI_PARAM_INVALID;
+  }
   int rc = check_filter_quant(d->filter_quant_num, d->col, d->filter_scales, d->filter_zps);
   if (rc != MI_OK) return rc;
   if ((rc = ensure_device()) != MI_OK) return rc;
@@ -1141,7 +1257,9 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
   h->act = d->act_type;
   h->zw0 = d->filter_zps[0];
   h->has_bias = bias_host != nullptr;
-  const std::vector<int8_t> w_nk = to_nk(weight_host, h->n, h->k, d->b_transpose);
+  const bool packed_sdot = (d->flags & MI_DYNMM_WEIGHT_PACKED_SDOT) != 0;
+  const std::vector<int8_t> w_nk = packed_sdot ? unpack_4x16(weight_host, h->n, h->k)
+                                               : to_nk(weight_host, h->n, h->k, d->b_transpose);
   std::vector<int8_t> packed((size_t)h->n_pad * h->ldw, 0);
   std::vector<float> ws(h->n_pad, 0.0f), bs(h->n_pad, 0.0f);
   std::vector<int32_t> wsum(h->n_pad, 0);
@@ -1149,7 +1267,8 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
     memcpy(packed.data() + (size_t)c * h->ldw, w_nk.data() + (size_t)c * h->k, (size_t)h->k);
     int32_t s = 0;
     for (int i = 0; i < h->k; ++i) s += w_nk[(size_t)c * h->k + i];
-    wsum[c] = s;
+    // a model that carries its own weight sums is computed with those (matmul_dynamic_base_int8.cc:179-183)
+    wsum[c] = (packed_sdot && d->weight_sums != nullptr) ? d->weight_sums[c] : s;
     ws[c] = (float)d->filter_scales[d->filter_quant_num > 1 ? c : 0];
     if (bias_host != nullptr) bs[c] = bias_host[c];
   }
@@ -1162,6 +1281,16 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
   }
   *out = owner.release();
   return MI_OK;
+}
+
+int mi_unpack_weight_4x16(const int8_t *packed, int32_t col, int32_t deep, int8_t *weight_nk) {
+  if (packed == nullptr || weight_nk == nullptr) return MI_NULL_PTR;
+  if (col <= 0 || deep <= 0) return MI_PARAM_INVALID;
+  return guarded("mi_unpack_weight_4x16", [&] {
+    const std::vector<int8_t> w = unpack_4x16(packed, col, deep);
+    memcpy(weight_nk, w.data(), w.size());
+    return MI_OK;
+  });
 }
 
 int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const float *bias_host, mi_dynmm **out) {

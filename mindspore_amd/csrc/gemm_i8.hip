@@ -25,6 +25,8 @@
 #include "common.h"
 #include "quant_math.h"
 
+#include <stdlib.h>
+
 #include <type_traits>
 
 namespace mi {
@@ -47,6 +49,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   void *c;
   int64_t ldc;
+  int diag_same_panel;  // timing what-if (wrong results): every tile fetches the operands of tile (0, 0), see diag_same_panel()
 };
 
 // Asynchronous 16-byte-per-lane copy global -> LDS: lane L's 16 bytes land at lds_wave_base + 16 * L;
@@ -829,10 +832,11 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   // issuing one costs scalar instructions only.
   const int drow = lane >> 3;
   const int dchunk = (lane & 7) ^ (drow >> 1);  // for even i; odd i: ^ 4
+  const int ld_n0 = g.diag_same_panel ? 0 : n0, ld_m0 = g.diag_same_panel ? 0 : m0;
   const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<int8_t *>(g.w) + (int64_t)(n0 + wave * WROWS) * g.ldw, (short)0, -1, 0x00020000);
+      const_cast<int8_t *>(g.w) + (int64_t)(ld_n0 + wave * WROWS) * g.ldw, (short)0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t a_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(g.a) + (int64_t)m0 * g.lda, (short)0, -1, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(g.a) + (int64_t)ld_m0 * g.lda, (short)0, -1, 0x00020000);
   const int w_voff = drow * g.ldw + dchunk * 16;  // ldw is a multiple of 256: odd i is w_voff ^ 64
   int a_voff[LPW];
 #pragma unroll
@@ -1060,6 +1064,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 // ---- host side -----------------------------------------------------------------------------------------------
+// Measurement aid, off unless the environment says MI355X_DIAG_SAME_PANEL=1 when the library is first used: the
+// K-block kernels then fetch tile (0, 0)'s operands for every tile, so that every operand line is an L2 hit.  The
+// results are wrong; the launch time shows what the L2 misses of the real access pattern cost.
+static int diag_same_panel() {
+  static const int on = [] {
+    const char *e = getenv("MI355X_DIAG_SAME_PANEL");
+    return (e != nullptr && e[0] == '1') ? 1 : 0;
+  }();
+  return on;
+}
+
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4, int OCC = 1>
 static int launch_cfg(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
   g.tiles_m = (g.m + TILE_M - 1) / TILE_M;
@@ -1075,6 +1090,7 @@ template <int EPI, bool HAS_ZW, bool FAST>
 static int launch_kblock(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
   g.tiles_m = (g.m + 255) / 256;
   g.tiles_n = (g.n + 255) / 256;
+  if ((g.m & 255) != 0 || (g.n & 255) != 0) g.diag_same_panel = 0;  // (the row clamps of ragged tiles assume the tile's own base)
   hipLaunchKernelGGL((gemm_kblock_kernel<EPI, HAS_ZW, FAST>), dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g, rq,
                      dq);
   MI_HIP_CHECK(hipGetLastError());
@@ -1085,6 +1101,7 @@ template <int EPI, bool HAS_ZW, bool FAST>
 static int launch_kblock128(GemmArgs g, const RequantParams &rq, const DequantParams &dq, hipStream_t stream) {
   g.tiles_m = (g.m + 127) / 128;
   g.tiles_n = (g.n + 127) / 128;
+  if ((g.m & 127) != 0 || (g.n & 127) != 0) g.diag_same_panel = 0;
   hipLaunchKernelGGL((gemm_kblock128_kernel<EPI, HAS_ZW, FAST>), dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g,
                      rq, dq);
   MI_HIP_CHECK(hipGetLastError());
@@ -1163,7 +1180,7 @@ int launch_gemm_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream) {
   int rc = check_args(a, lda, m, k, w, n, c, ldc, 4);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc, diag_same_panel()};
   DequantParams dq{};
   if (rq.has_zw) {
     return rq.fast2 ? launch_pick_tile<EPI_REQUANT, true, true>(g, rq, dq, stream)
@@ -1220,7 +1237,7 @@ int launch_gemm_conv_requant(const int8_t *in, const ConvGeom &cg, const int8_t 
   ConvGather cv{cg.in_h,     cg.in_w,       cg.in_c,       cg.out_w,  cg.out_h * cg.out_w, cg.kernel_w, cg.stride_h,
                 cg.stride_w, cg.dilation_h, cg.dilation_w, cg.pad_u,  cg.pad_l,            magic(cg.in_c),
                 magic(cg.kernel_w), fill16};
-  GemmArgs g{in, 0, (int)m64, (int)k64, w.w, w.ldw, w.k_pad, cg.out_c, 0, 0, out, cg.out_c};
+  GemmArgs g{in, 0, (int)m64, (int)k64, w.w, w.ldw, w.k_pad, cg.out_c, 0, 0, out, cg.out_c, 0};
   if (rq.has_zw) {
     return rq.fast2 ? launch_conv_pick_tile<true, true>(g, cv, rq, stream)
                     : launch_conv_pick_tile<true, false>(g, cv, rq, stream);
@@ -1233,7 +1250,7 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream) {
   int rc = check_args(a, lda, m, k, w, n, c, ldc, 16);
   if (rc != MI_OK) return rc;
-  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc};
+  GemmArgs g{a, lda, m, k, w.w, w.ldw, w.k_pad, n, 0, 0, c, ldc, diag_same_panel()};
   RequantParams rq{};
   // the third parameter (the fast-rounding switch of the int8 epilogue) selects non-temporal stores here
   const bool nt = stream_out_hint((int64_t)m * n * 4);

@@ -207,3 +207,63 @@ extern "C" int mi_infer_conv2d(const int32_t *in_shape, int32_t in_dims, const i
   c.v[3] = w.v[0];
   return emit(c, out_shape, out_dims);
 }
+
+// The batch broadcast of MatMul operands (InitBroadcastParams, mindspore/lite/src/litert/kernel/cpu/fp32/
+// matmul_fp32_base.cc:576-646): both shapes are brought to the same rank (at least 4) with leading ones; a batch
+// extent of one operand may be smaller than the other's when it divides it, and output matrix i then takes the
+// operand's matrix at the proportionally scaled index.
+extern "C" int mi_matmul_broadcast_offsets(const int32_t *a_shape, int32_t a_dims, const int32_t *b_shape,
+                                           int32_t b_dims, int32_t capacity, int32_t *batch, int32_t *a_offsets,
+                                           int32_t *b_offsets) {
+  if (batch == nullptr || a_offsets == nullptr || b_offsets == nullptr) {
+    mi::set_error("mi_matmul_broadcast_offsets: null output");
+    return MI_NULL_PTR;
+  }
+  Dims a, b;
+  if (!a.load(a_shape, a_dims) || !b.load(b_shape, b_dims) || a.n < 2 || b.n < 2 || !a.known() || !b.known()) {
+    mi::set_error("mi_matmul_broadcast_offsets: operands must have rank 2..%d and known extents", MI_MAX_DIMS);
+    return MI_PARAM_INVALID;
+  }
+  const int rank = a.n > b.n ? (a.n > 4 ? a.n : 4) : (b.n > 4 ? b.n : 4);
+  if (rank > MI_MAX_DIMS) return MI_PARAM_INVALID;
+  while (a.n < rank) a.push_front(1);
+  while (b.n < rank) b.push_front(1);
+  const int nb = rank - 2;  // batch axes
+  int64_t sizes[MI_MAX_DIMS] = {0}, a_sizes[MI_MAX_DIMS] = {0}, b_sizes[MI_MAX_DIMS] = {0};  // products from axis j to the last batch axis
+  int64_t out_batch = 1;
+  for (int j = nb - 1; j >= 0; --j) {
+    const int64_t mx = a.v[j] > b.v[j] ? a.v[j] : b.v[j];
+    const int64_t mn_raw = a.v[j] < b.v[j] ? a.v[j] : b.v[j];
+    const int64_t mn = mn_raw > 0 ? mn_raw : 1;
+    if (mx != mn && mx % mn != 0) {
+      mi::set_error("mi_matmul_broadcast_offsets: batch extents %d and %d cannot be broadcast", a.v[j], b.v[j]);
+      return MI_PARAM_INVALID;
+    }
+    sizes[j] = (j == nb - 1 ? 1 : sizes[j + 1]) * mx;
+    a_sizes[j] = (j == nb - 1 ? 1 : a_sizes[j + 1]) * a.v[j];
+    b_sizes[j] = (j == nb - 1 ? 1 : b_sizes[j + 1]) * b.v[j];
+    out_batch *= mx;
+  }
+  if (out_batch > capacity || out_batch <= 0) {
+    mi::set_error("mi_matmul_broadcast_offsets: %lld output matrices, room for %d", (long long)out_batch, capacity);
+    return MI_PARAM_INVALID;
+  }
+  *batch = (int32_t)out_batch;
+  for (int64_t i = 0; i < out_batch; ++i) {
+    int64_t delta = i, ao = 0, bo = 0;
+    for (int j = 0; j < nb; ++j) {
+      if (j > 0) delta %= sizes[j];
+      const int64_t mx = a.v[j] > b.v[j] ? a.v[j] : b.v[j];
+      if (j < nb - 1) {
+        ao += (delta / sizes[j + 1] * a.v[j] / mx) * a_sizes[j + 1];
+        bo += (delta / sizes[j + 1] * b.v[j] / mx) * b_sizes[j + 1];
+      } else {
+        ao += delta * a.v[j] / mx;
+        bo += delta * b.v[j] / mx;
+      }
+    }
+    a_offsets[i] = (int32_t)ao;
+    b_offsets[i] = (int32_t)bo;
+  }
+  return MI_OK;
+}

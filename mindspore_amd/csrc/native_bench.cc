@@ -5,6 +5,11 @@
 //   native_bench warm <rows> <steps> <warmup>              each of the five matrices alone, back to back (its weights
 //                                                          stay in the 256 MB Infinity Cache between launches)
 //   native_bench read <mib> <steps> <warmup>               the library's plain read stream over slices of 3 GiB
+//   native_bench bert <steps> <warmup>                     the four dynamic-quant MatMuls of a BERT-base layer at 4096
+//                                                          rows (fp32 out), each launched back to back
+//   native_bench dynmm <rows> <n> <k> <steps> <warmup>     one dynamic-quant MatMul shape
+//   native_bench gemm <rows> <n> <k> <steps> <warmup>      one full-quant MatMul shape (int8 out)
+//   native_bench dw <h> <w> <c> <steps> <warmup>           a 3x3 stride-1 depthwise convolution (ReLU6)
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -246,15 +251,173 @@ static int run_read(int mib, int steps, int warmup) {
   return 0;
 }
 
+// One dynamic-quant MatMul (fp32 output) launched back to back; prints its JSON fragment.
+static int time_dynmm(const char *name, int rows, int n, int k, int steps, int warmup, hipStream_t st,
+                      double *ops_sum, double *ms_sum) {
+  Rng rng{(uint64_t)(1000 + n + 7 * k)};
+  std::vector<int8_t> w((size_t)n * k);
+  for (auto &x : w) x = (int8_t)((int)(rng.next() % 255) - 127);
+  std::vector<double> scales(n);
+  std::vector<int32_t> zps(n, 0);
+  std::vector<float> bias(n);
+  for (int c = 0; c < n; ++c) {
+    scales[c] = 0.001 + 0.009 * rng.uniform();
+    bias[c] = (float)(rng.uniform() - 0.5);
+  }
+  mi_dynmm_desc d{};
+  d.deep = k;
+  d.col = n;
+  d.b_transpose = 1;
+  d.act_type = MI_ACT_NONE;
+  d.filter_quant_num = n;
+  d.filter_scales = scales.data();
+  d.filter_zps = zps.data();
+  mi_dynmm *h = nullptr;
+  CHECK_MI(mi_dynmm_create(&d, w.data(), bias.data(), &h));
+  std::vector<int8_t> a((size_t)rows * k);
+  for (auto &x : a) x = (int8_t)(rng.next() & 0xff);
+  int8_t *a_dev = nullptr;
+  float *c_dev = nullptr;
+  CHECK_HIP(hipMalloc(&a_dev, a.size()));
+  CHECK_HIP(hipMalloc(&c_dev, (size_t)rows * n * 4));
+  CHECK_HIP(hipMemcpy(a_dev, a.data(), a.size(), hipMemcpyHostToDevice));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  auto run = [&]() -> int { return mi_dynmm_run(h, a_dev, rows, 0.031, -3, c_dev, st); };
+  for (int i = 0; i < warmup; ++i) CHECK_MI(run());
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i) CHECK_MI(run());
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+  const double us = ms / steps * 1e3, ops = 2.0 * rows * n * k;
+  const double bytes = (double)rows * k + (double)n * k + 4.0 * rows * n + 12.0 * n;
+  printf("\"%s\": {\"rows\": %d, \"n\": %d, \"k\": %d, \"us\": %.3f, \"tops\": %.1f, \"algorithmic_bytes\": %.0f, "
+         "\"gbps\": %.1f}",
+         name, rows, n, k, us, ops / (us * 1e-6) / 1e12, bytes, bytes / (us * 1e-6) / 1e9);
+  *ops_sum += ops;
+  *ms_sum += ms / steps;
+  mi_dynmm_destroy(h);
+  CHECK_HIP(hipFree(a_dev));
+  CHECK_HIP(hipFree(c_dev));
+  return 0;
+}
+
+static int run_bert(int steps, int warmup) {
+  const Shape shapes[4] = {{"qkv", 2304, 768}, {"out", 768, 768}, {"ffn1", 3072, 768}, {"ffn2", 768, 3072}};
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  double ops = 0, ms = 0;
+  printf("{\"mode\": \"bert\", \"rows\": 4096, ");
+  for (const Shape &s : shapes) {
+    if (time_dynmm(s.name, 4096, s.n, s.k, steps, warmup, st, &ops, &ms)) return 1;
+    printf(", ");
+  }
+  printf("\"total_us\": %.3f, \"total_tops\": %.1f}\n", ms * 1e3, ops / (ms * 1e-3) / 1e12);
+  return 0;
+}
+
+static int run_dynmm(int rows, int n, int k, int steps, int warmup) {
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  double ops = 0, ms = 0;
+  printf("{\"mode\": \"dynmm\", ");
+  if (time_dynmm("shape", rows, n, k, steps, warmup, st, &ops, &ms)) return 1;
+  printf("}\n");
+  return 0;
+}
+
+static int run_gemm(int rows, int n, int k, int steps, int warmup) {
+  const Shape sh{"gemm", n, k};
+  Matrix m;
+  Rng rng{99};
+  if (make_matrix(sh, rows, &rng, &m)) return 1;
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  for (int i = 0; i < warmup; ++i) CHECK_MI(mi_matmul_run(m.h, m.act, rows, m.out, st));
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i) CHECK_MI(mi_matmul_run(m.h, m.act, rows, m.out, st));
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+  const double us = ms / steps * 1e3;
+  printf("{\"mode\": \"gemm\", \"rows\": %d, \"n\": %d, \"k\": %d, \"us\": %.3f, \"tops\": %.1f}\n", rows, n, k, us,
+         2.0 * rows * n * k / (us * 1e-6) / 1e12);
+  mi_matmul_destroy(m.h);
+  return 0;
+}
+
+static int run_dw(int ih, int iw, int c, int steps, int warmup) {
+  Rng rng{31};
+  std::vector<int8_t> w((size_t)c * 9), x((size_t)ih * iw * c);
+  for (auto &v : w) v = (int8_t)((int)(rng.next() % 255) - 127);
+  for (auto &v : x) v = (int8_t)(rng.next() & 0xff);
+  std::vector<double> scales(c);
+  std::vector<int32_t> zps(c, 0), bias(c);
+  for (int i = 0; i < c; ++i) {
+    scales[i] = 0.001 + 0.009 * rng.uniform();
+    bias[i] = (int32_t)(rng.next() % 4001) - 2000;
+  }
+  mi_conv_desc d{};
+  d.in_channel = d.out_channel = d.group = c;
+  d.kernel_h = d.kernel_w = 3;
+  d.stride_h = d.stride_w = d.dilation_h = d.dilation_w = 1;
+  d.pad_u = d.pad_d = d.pad_l = d.pad_r = 1;
+  d.act_type = MI_ACT_RELU6;
+  d.in_scale = 6.0 / 140.0;
+  d.in_zp = -11;
+  d.out_scale = 6.0 / 140.0;
+  d.out_zp = 9;
+  d.filter_quant_num = c;
+  d.filter_scales = scales.data();
+  d.filter_zps = zps.data();
+  mi_conv *h = nullptr;
+  CHECK_MI(mi_conv_create(&d, w.data(), bias.data(), &h));
+  int8_t *in_dev = nullptr, *out_dev = nullptr;
+  CHECK_HIP(hipMalloc(&in_dev, x.size()));
+  CHECK_HIP(hipMalloc(&out_dev, x.size()));
+  CHECK_HIP(hipMemcpy(in_dev, x.data(), x.size(), hipMemcpyHostToDevice));
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  for (int i = 0; i < warmup; ++i) CHECK_MI(mi_conv_run(h, in_dev, 1, ih, iw, out_dev, st));
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i) CHECK_MI(mi_conv_run(h, in_dev, 1, ih, iw, out_dev, st));
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  CHECK_HIP(hipEventElapsedTime(&ms, e0, e1));
+  const double us = ms / steps * 1e3, bytes = 2.0 * x.size() + w.size();
+  printf("{\"mode\": \"dw\", \"h\": %d, \"w\": %d, \"c\": %d, \"us\": %.3f, \"algorithmic_bytes\": %.0f, \"gbps\": %.1f}\n", ih,
+         iw, c, us, bytes, bytes / (us * 1e-6) / 1e9);
+  mi_conv_destroy(h);
+  return 0;
+}
+
 int main(int argc, char **argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup> | shape <n> <k> <rows> <steps> <warmup>\n");
+    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup> | shape <n> <k> <rows> <steps> <warmup> | bert <steps> <warmup> | dynmm <rows> <n> <k> <steps> <warmup> | gemm <rows> <n> <k> <steps> <warmup> | dw <h> <w> <c> <steps> <warmup>\n");
     return 2;
   }
   CHECK_MI(mi_init(0));
   if (strcmp(argv[1], "shape") == 0 && argc >= 7) return run_shape(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
   if (strcmp(argv[1], "decode") == 0 && argc >= 6) return run_decode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
   if (strcmp(argv[1], "warm") == 0 && argc >= 5) return run_warm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
+  if (strcmp(argv[1], "bert") == 0 && argc >= 4) return run_bert(atoi(argv[2]), atoi(argv[3]));
+  if (strcmp(argv[1], "dynmm") == 0 && argc >= 7) return run_dynmm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
+  if (strcmp(argv[1], "gemm") == 0 && argc >= 7) return run_gemm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
+  if (strcmp(argv[1], "dw") == 0 && argc >= 7) return run_dw(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
   if (strcmp(argv[1], "read") == 0 && argc >= 5) return run_read(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
   fprintf(stderr, "bad arguments\n");
   return 2;

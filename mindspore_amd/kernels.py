@@ -77,9 +77,13 @@ class MatmulInt8Kernel(_Handle):
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)
-        if weight.ndim != 2:
-            raise ValueError("weight must be 2-D")
-        self.n, self.k = (weight.shape if transpose_b else weight.shape[::-1])
+        if weight.ndim < 2:
+            raise ValueError("weight must have at least two dimensions")
+        # a constant weight of rank > 2 is a batch of matrices (matmul_base_int8.cc:366-368)
+        self.w_shape = tuple(weight.shape)
+        self.b_batch = int(np.prod(weight.shape[:-2])) if weight.ndim > 2 else 1
+        self.n, self.k = (weight.shape[-2:] if transpose_b else weight.shape[-2:][::-1])
+        self.transpose_b = bool(transpose_b)
         if bias is not None:
             bias = np.ascontiguousarray(bias)
             if bias.dtype != np.int32:
@@ -89,7 +93,7 @@ class MatmulInt8Kernel(_Handle):
         nq, scales, zps = _quant_arrays(weight_quant)
         d = _lib.MatmulDesc(self.k, self.n, 1 if transpose_b else 0, act, float(in_quant.scale),
                             int(in_quant.zero_point), float(out_quant.scale), int(out_quant.zero_point), nq, scales,
-                            zps, 0 if decode_pack else _lib.MATMUL_NO_DECODE_PACK)
+                            zps, 0 if decode_pack else _lib.MATMUL_NO_DECODE_PACK, self.b_batch)
         _lib.check(L.mi_matmul_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                       C.byref(self._h)), "mi_matmul_create")
 
@@ -115,6 +119,31 @@ class MatmulInt8Kernel(_Handle):
         rows = a.size // self.k
         out = np.empty(a.shape[:-1] + (self.n,), np.int8)
         _lib.check(L.mi_matmul_run_host(self._h, a.ctypes.data, rows, out.ctypes.data), "mi_matmul_run_host")
+        return out
+
+    def run_batched(self, a):
+        """Batched MatMul against a weight of rank > 2 (or a rank-2 weight broadcast over a batched `a`): a is a
+        contiguous CUDA int8 tensor [..., rows, K]; the batch extents of `a` and of the weight are broadcast as the
+        reference does (MatmulFp32BaseCPUKernel::InitBroadcastParams).  Returns [batch..., rows, N]."""
+        import torch
+        L = _lib.load()
+        if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.ndim < 2 or a.shape[-1] != self.k:
+            raise ValueError("expected a contiguous CUDA int8 tensor [..., rows, %d]" % self.k)
+        rows = a.shape[-2]
+        a_shape, an = _shape_arg(a.shape)
+        w_shape, wn = _shape_arg(self.w_shape)
+        cap = 1 << 16
+        batch = C.c_int32(0)
+        a_off, b_off = (C.c_int32 * cap)(), (C.c_int32 * cap)()
+        _lib.check(L.mi_matmul_broadcast_offsets(a_shape, an, w_shape, wn, cap, C.byref(batch), a_off, b_off),
+                   "mi_matmul_broadcast_offsets")
+        rank = max(a.ndim, len(self.w_shape))
+        ash = (1,) * (rank - a.ndim) + tuple(a.shape)
+        wsh = (1,) * (rank - len(self.w_shape)) + self.w_shape
+        out_shape = tuple(max(x, y) for x, y in zip(ash[:-2], wsh[:-2])) + (rows, self.n)
+        out = torch.empty(out_shape, dtype=torch.int8, device=a.device)
+        _lib.check(L.mi_matmul_run_batched(self._h, a.data_ptr(), rows, batch.value, a_off, b_off, out.data_ptr(),
+                                           _stream()), "mi_matmul_run_batched")
         return out
 
     def reserve(self, max_rows):
@@ -290,11 +319,21 @@ class MatmulDynamicInt8Kernel(_Handle):
     """Dynamic-quant MatMul: int8 activations (scale / zero point supplied at every run) x int8 weights -> fp32."""
     _destroy = "mi_dynmm_destroy"
 
-    def __init__(self, weight, bias, weight_quant, transpose_b=True, act=ACT_NONE, device=0):
+    def __init__(self, weight, bias, weight_quant, transpose_b=True, act=ACT_NONE, device=0, packed_sdot=None,
+                 weight_sums=None):
+        """packed_sdot=(N, K): `weight` is the flat byte string a model converted for the ARM dot-product kernel
+        carries (blocks of 16 channels x 4 K-bytes, RowMajor2Row4x16MajorInt8 / RowMajor2Col4x16MajorInt8) and
+        weight_sums, if given, its int32 weight-sums tensor [round_up(N, 16)]."""
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)
-        self.n, self.k = (weight.shape if transpose_b else weight.shape[::-1])
+        if packed_sdot is not None:
+            self.n, self.k = int(packed_sdot[0]), int(packed_sdot[1])
+            need = -(-self.n // 16) * 16 * -(-self.k // 4) * 4
+            if weight.size != need:
+                raise ValueError("a packed weight for N=%d, K=%d has %d bytes, got %d" % (self.n, self.k, need, weight.size))
+        else:
+            self.n, self.k = (weight.shape if transpose_b else weight.shape[::-1])
         if bias is not None:
             bias = np.ascontiguousarray(bias)
             if bias.dtype != np.float32:
@@ -302,7 +341,14 @@ class MatmulDynamicInt8Kernel(_Handle):
             if bias.size != self.n:
                 raise ValueError("bias has %d entries, expected %d" % (bias.size, self.n))
         nq, scales, zps = _quant_arrays(weight_quant)
-        d = _lib.DynmmDesc(self.k, self.n, 1 if transpose_b else 0, act, nq, scales, zps)
+        sums = None
+        if weight_sums is not None:
+            weight_sums = np.ascontiguousarray(weight_sums, dtype=np.int32)
+            if packed_sdot is None or weight_sums.size < self.n:
+                raise ValueError("weight_sums goes with a packed weight and holds at least N entries")
+            sums = weight_sums.ctypes.data_as(C.POINTER(C.c_int32))
+        d = _lib.DynmmDesc(self.k, self.n, 1 if transpose_b else 0, act, nq, scales, zps,
+                           _lib.DYNMM_WEIGHT_PACKED_SDOT if packed_sdot is not None else 0, sums)
         _lib.check(L.mi_dynmm_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                      C.byref(self._h)), "mi_dynmm_create")
 

@@ -12,16 +12,16 @@ MI_OK, MI_ERROR, MI_NULL_PTR, MI_PARAM_INVALID, MI_MEMORY_FAILED, MI_NOT_SUPPORT
 ACT_NONE, ACT_RELU, ACT_RELU6 = 0, 1, 3
 
 EXPORTS = [
-    "mi_init", "mi_last_error", "mi_version", "mi_quantize_multiplier", "mi_quantize_multiplier_single", "mi_activation_range", "mi_requant_params",
+    "mi_init", "mi_last_error", "mi_debug_fail_alloc", "mi_debug_sync_count", "mi_version", "mi_quantize_multiplier", "mi_quantize_multiplier_single", "mi_activation_range", "mi_requant_params",
     "mi_multiply_by_quantized_multiplier",
-    "mi_matmul_create", "mi_matmul_reserve", "mi_matmul_run", "mi_matmul_run_noalloc", "mi_matmul_run_host", "mi_matmul_run_group", "mi_matmul_get_params", "mi_matmul_destroy",
+    "mi_matmul_create", "mi_matmul_reserve", "mi_matmul_run", "mi_matmul_run_noalloc", "mi_matmul_run_host", "mi_matmul_run_group", "mi_matmul_run_batched", "mi_matmul_broadcast_offsets", "mi_matmul_get_params", "mi_matmul_destroy",
     "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_reserve", "mi_conv_destroy",
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
     "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
-    "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
+    "mi_unpack_weight_4x16", "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
     "mi_dynmm_destroy",
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
-    "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_stream_synchronize", "mi_stream_create", "mi_stream_destroy",
+    "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_copy_to_host_async", "mi_stream_synchronize", "mi_stream_create", "mi_stream_destroy",
     "mi_host_malloc", "mi_host_free",
 ]
 # libmi355x_diag.so (include/mi355x_diag.h): the benchmark's measurement aids, not part of the product library
@@ -33,7 +33,7 @@ class MatmulDesc(C.Structure):
     _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
                 ("in_scale", C.c_double), ("in_zp", C.c_int32), ("out_scale", C.c_double), ("out_zp", C.c_int32),
                 ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
-                ("filter_zps", C.POINTER(C.c_int32)), ("flags", C.c_int32)]
+                ("filter_zps", C.POINTER(C.c_int32)), ("flags", C.c_int32), ("b_batch", C.c_int32)]
 
 
 MATMUL_NO_DECODE_PACK = 1
@@ -54,7 +54,10 @@ CONV_3X3_EXACT = 1
 class DynmmDesc(C.Structure):
     _fields_ = [("deep", C.c_int32), ("col", C.c_int32), ("b_transpose", C.c_int32), ("act_type", C.c_int32),
                 ("filter_quant_num", C.c_int32), ("filter_scales", C.POINTER(C.c_double)),
-                ("filter_zps", C.POINTER(C.c_int32))]
+                ("filter_zps", C.POINTER(C.c_int32)), ("flags", C.c_int32), ("weight_sums", C.POINTER(C.c_int32))]
+
+
+DYNMM_WEIGHT_PACKED_SDOT = 1
 
 
 class ConvInfer(C.Structure):
@@ -110,6 +113,9 @@ def load():
     L.mi_matmul_run_noalloc.argtypes = [vp, vp, i32, vp, vp]
     L.mi_matmul_run_group.argtypes = [C.POINTER(vp), i32, vp, i32, C.POINTER(vp), vp]
     L.mi_matmul_run_host.argtypes = [vp, vp, i32, vp]
+    L.mi_matmul_run_batched.argtypes = [vp, vp, i32, i32, pi32, pi32, vp, vp]
+    L.mi_matmul_broadcast_offsets.argtypes = [pi32, i32, pi32, i32, i32, pi32, pi32, pi32]
+    L.mi_debug_fail_alloc.argtypes = [C.c_size_t]
     L.mi_matmul_get_params.argtypes = [vp, vp, vp, vp, vp, pi32, pi32]
     L.mi_matmul_destroy.argtypes = [vp]
     L.mi_matmul_destroy.restype = None
@@ -131,6 +137,7 @@ def load():
     L.mi_dynquant_run_segments_host.argtypes = [vp, vp, i64, i64, vp, vp]
     L.mi_dynquant_destroy.argtypes = [vp]
     L.mi_dynquant_destroy.restype = None
+    L.mi_unpack_weight_4x16.argtypes = [vp, i32, i32, vp]
     L.mi_dynmm_create.argtypes = [C.POINTER(DynmmDesc), vp, vp, C.POINTER(vp)]
     L.mi_dynmm_run.argtypes = [vp, vp, i32, dbl, i32, vp, vp]
     L.mi_dynmm_run_chained.argtypes = [vp, vp, i32, vp, vp, vp]
@@ -149,6 +156,8 @@ def load():
     L.mi_host_free.argtypes = [vp]
     L.mi_copy_to_device.argtypes = [vp, vp, C.c_size_t, vp]
     L.mi_copy_to_host.argtypes = [vp, vp, C.c_size_t, vp]
+    L.mi_copy_to_host_async.argtypes = [vp, vp, C.c_size_t, vp]
+    L.mi_debug_sync_count.restype = C.c_int64
     L.mi_stream_synchronize.argtypes = [vp]
     L.mi_stream_create.argtypes = [C.POINTER(vp)]
     L.mi_stream_destroy.argtypes = [vp]

@@ -42,7 +42,7 @@
 #include <memory>
 #include <mutex>
 #include <string>
-#include <unordered_set>
+#include <unordered_map>
 #include <vector>
 
 #include "include/api/kernel.h"
@@ -89,19 +89,44 @@ int ToStatus(int mi_code) { return mi_code == MI_OK ? static_cast<int>(kSuccess)
 
 // One HIP stream per session: every kernel of a session is handed the same mindspore::Context, and everything it
 // launches or copies goes to that session's stream, so that sessions running on different threads neither share a
-// queue nor wait for each other's copies.  Streams live as long as the process (a provider is never told that a
-// session ended).
-void *SessionStream(const Context *ctx) {
-  static std::mutex *mutex = new std::mutex;
-  static std::map<const Context *, void *> *streams = new std::map<const Context *, void *>;
-  std::lock_guard<std::mutex> lock(*mutex);
-  auto it = streams->find(ctx);
-  if (it != streams->end()) return it->second;
-  void *stream = nullptr;
-  if (mi_stream_create(&stream) != MI_OK) stream = nullptr;  // the null stream still works, only without overlap
-  (*streams)[ctx] = stream;
-  return stream;
-}
+// queue nor wait for each other's copies.  A provider is never told that a session ended, so the stream is counted:
+// every kernel takes a reference in Prepare and gives it back when it is destroyed, and the last one destroys the
+// stream (its own work on it has finished by then: a kernel's buffers are freed first, which waits for the device).
+class SessionStreams {
+ public:
+  static void *Acquire(const Context *ctx) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    Entry &e = Map()[ctx];
+    if (e.refs == 0 && mi_stream_create(&e.stream) != MI_OK) e.stream = nullptr;  // the null stream still works, only without overlap
+    ++e.refs;
+    return e.stream;
+  }
+  static void Release(const Context *ctx) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    auto it = Map().find(ctx);
+    if (it == Map().end() || --it->second.refs > 0) return;
+    mi_stream_destroy(it->second.stream);
+    Map().erase(it);
+  }
+  static size_t Count() {
+    std::lock_guard<std::mutex> lock(Mutex());
+    return Map().size();
+  }
+
+ private:
+  struct Entry {
+    void *stream = nullptr;
+    int refs = 0;
+  };
+  static std::mutex &Mutex() {
+    static std::mutex *m = new std::mutex;
+    return *m;
+  }
+  static std::map<const Context *, Entry> &Map() {
+    static auto *m = new std::map<const Context *, Entry>;
+    return *m;
+  }
+};
 
 // Rows of a MatMul / FullConnection: the product of the output's leading dimensions, as the reference kernels take
 // it (fullconnection_int8.cc:49-58, which also covers use_axis; matmul_int8.cc InitParameter).
@@ -114,30 +139,63 @@ int64_t RowsOfOutput(const MSTensor &out) {
 
 // Device addresses this provider has published on tensors.  GetDeviceData() of an input is trusted only when it is
 // one of them: an application may have attached memory of some other device to a graph input.
+// Each address also carries a version, counted up whenever its owner delivers a new result into it, and -- for the
+// output of a DynamicQuant kernel -- where that run's scales and zero points lie in device memory.
+struct QuantOnDevice {
+  const mi_dq_params *params = nullptr;  // one block (per tensor), or one per row
+  bool per_row = false;
+  int64_t rows = 0;
+};
+
 class Published {
  public:
   static void Add(void *p) {
     std::lock_guard<std::mutex> lock(Mutex());
-    Set().insert(p);
+    (void)Table()[p];
   }
   static void Remove(void *p) {
     std::lock_guard<std::mutex> lock(Mutex());
-    Set().erase(p);
+    Table().erase(p);
   }
   static bool Has(void *p) {
     std::lock_guard<std::mutex> lock(Mutex());
-    return Set().count(p) != 0;
+    return Table().count(p) != 0;
+  }
+  // a new result was written into p (its owner's Deliver)
+  static void Bump(void *p, const QuantOnDevice *quant) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    auto it = Table().find(p);
+    if (it == Table().end()) return;
+    ++it->second.version;
+    it->second.quant = quant != nullptr ? *quant : QuantOnDevice{};
+  }
+  // 0 for an address that is not one of this provider's
+  static int64_t Version(void *p) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    auto it = Table().find(p);
+    return it == Table().end() ? 0 : it->second.version;
+  }
+  static bool Quant(void *p, QuantOnDevice *out) {
+    std::lock_guard<std::mutex> lock(Mutex());
+    auto it = Table().find(p);
+    if (it == Table().end() || it->second.quant.params == nullptr) return false;
+    *out = it->second.quant;
+    return true;
   }
 
  private:
+  struct Entry {
+    int64_t version = 1;
+    QuantOnDevice quant;
+  };
   // never destroyed: kernels owned by a session with static storage may be torn down after this file's statics
   static std::mutex &Mutex() {
     static std::mutex *m = new std::mutex;
     return *m;
   }
-  static std::unordered_set<void *> &Set() {
-    static std::unordered_set<void *> *s = new std::unordered_set<void *>;
-    return *s;
+  static std::unordered_map<void *, Entry> &Table() {
+    static auto *t = new std::unordered_map<void *, Entry>;
+    return *t;
   }
 };
 
@@ -157,8 +215,6 @@ class DeviceBuffer {
     return p_;
   }
   void *get() const { return p_; }
-
- private:
   void Release() {
     if (p_ != nullptr) {
       Published::Remove(p_);
@@ -167,6 +223,8 @@ class DeviceBuffer {
     p_ = nullptr;
     cap_ = 0;
   }
+
+ private:
   void *p_ = nullptr;
   size_t cap_ = 0;
 };
@@ -175,9 +233,22 @@ class DeviceBuffer {
 // this provider left it there, uploaded otherwise) and hand the output on.
 class DeviceIo {
  public:
+  DeviceIo() = default;
+  DeviceIo(const DeviceIo &) = delete;
+  DeviceIo &operator=(const DeviceIo &) = delete;
+  ~DeviceIo() {
+    in_.Release();  // (waits for the device: nothing of this kernel is left on the stream)
+    out_.Release();
+    if (configured_) SessionStreams::Release(ctx_);
+  }
+
   // the session's stream, and [mi355x] device_only_outputs for the given output tensor
-  void Configure(void *stream, const std::map<std::string, std::string> &section, const std::string &output_name) {
-    stream_ = stream;
+  void Configure(const Context *ctx, const std::map<std::string, std::string> &section, const std::string &output_name) {
+    if (!configured_) {
+      ctx_ = ctx;
+      stream_ = SessionStreams::Acquire(ctx);
+      configured_ = true;
+    }
     const auto it = section.find("device_only_outputs");
     if (it == section.end()) return;
     const std::string &list = it->second;
@@ -214,7 +285,8 @@ class DeviceIo {
 
   // after the launch: publish the device address; copy to the host unless the output was declared device-only (the
   // copy waits for this session's stream only; a device-only output is ordered by the stream itself)
-  int Deliver(MSTensor *t) {
+  int Deliver(MSTensor *t, const QuantOnDevice *quant = nullptr) {
+    Published::Bump(out_.get(), quant);
     t->SetDeviceData(out_.get());
     if (!host_copy_) return kSuccess;
     void *host = t->MutableData();
@@ -223,6 +295,7 @@ class DeviceIo {
                                                                                : static_cast<int>(kLiteError);
   }
   void *stream() const { return stream_; }
+  bool host_copy() const { return host_copy_; }
 
   void Withdraw(MSTensor *t) {
     if (t->GetDeviceData() == out_.get()) t->SetDeviceData(nullptr);
@@ -232,6 +305,8 @@ class DeviceIo {
   DeviceBuffer in_, out_;
   bool host_copy_ = true;
   void *stream_ = nullptr;
+  const Context *ctx_ = nullptr;
+  bool configured_ = false;
 };
 
 // ---- MatMulFusion / FullConnection, int8 in -> int8 out (full quant) or fp32 out (dynamic quant) ----------------
@@ -313,13 +388,18 @@ class MatmulKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(context_, GetConfig("mi355x"), outputs_[0].Name());
     const MSTensor &w = inputs_[kWeightIndex];
     const auto wshape = w.Shape();
-    if (wshape.size() != 2 || w.Data() == nullptr) return kLiteError;
-    const int32_t n = static_cast<int32_t>(b_transpose_ ? wshape[0] : wshape[1]);
-    const int32_t k = static_cast<int32_t>(b_transpose_ ? wshape[1] : wshape[0]);
+    if (wshape.size() < 2 || w.Data() == nullptr) return kLiteError;
+    const size_t r = wshape.size();
+    const int32_t n = static_cast<int32_t>(b_transpose_ ? wshape[r - 2] : wshape[r - 1]);
+    const int32_t k = static_cast<int32_t>(b_transpose_ ? wshape[r - 1] : wshape[r - 2]);
     k_ = k;
+    n_ = n;
+    int64_t b_batch = 1;  // a constant weight of rank > 2 is a batch of matrices (matmul_base_int8.cc:366-368)
+    for (size_t i = 0; i + 2 < r; ++i) b_batch *= wshape[i];
+    batched_ = r > 2;
     std::vector<double> scales;
     std::vector<int32_t> zps;
     FilterQuant(w, &scales, &zps);
@@ -329,14 +409,25 @@ class MatmulKernel : public kernel::Kernel {
       const auto oq = outputs_[0].QuantParams().front();
       mi_matmul_desc d{k, n, b_transpose_ ? 1 : 0, act_, iq.scale, iq.zero_point, oq.scale, oq.zero_point,
                        static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
+      d.b_batch = static_cast<int32_t>(b_batch);
+      // The second packed form of the weights serves 2..32 activation rows; a node whose inferred output already has
+      // more rows than that does without it (half the device memory per weight).  Should the model later be resized
+      // to a few rows, they run on the GEMM tiles.
+      const auto oshape = outputs_[0].Shape();
+      bool rows_known = !oshape.empty();
+      for (int64_t e : oshape) rows_known = rows_known && e >= 0;
+      const int64_t rows_now = batched_ && oshape.size() >= 2 ? oshape[oshape.size() - 2] : RowsOfOutput(outputs_[0]);
+      if (rows_known && rows_now > kSiblingMaxRows) d.flags |= MI_MATMUL_NO_DECODE_PACK;
       const int rc = mi_matmul_create(&d, static_cast<const int8_t *>(w.Data().get()),
                                       static_cast<const int32_t *>(bias), &full_);
       // (a session that runs its nodes in parallel gives no order to lean on: no groups there)
-      if (rc == MI_OK && !inputs_[0].IsConst() && context_ != nullptr && !context_->GetEnableParallel()) {
+      if (rc == MI_OK && !batched_ && !inputs_[0].IsConst() && context_ != nullptr && !context_->GetEnableParallel() &&
+          getenv("MI355X_NO_SIBLING_GROUPS") == nullptr) {
         group_ = SiblingGroup::Join(context_, inputs_[0], k, this);
       }
       return ToStatus(rc);
     }
+    if (batched_) return kLiteError;  // (the creator declines batched weights for the dynamic MatMul)
     mi_dynmm_desc d{k, n, b_transpose_ ? 1 : 0, act_, static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
     return ToStatus(
       mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_));
@@ -348,14 +439,19 @@ class MatmulKernel : public kernel::Kernel {
   }
 
   int Execute() override {
+    if (batched_) return ExecuteBatched();
     const int32_t rows = static_cast<int32_t>(RowsOfOutput(outputs_[0]));
     if (rows == 0) return kSuccess;
     if (inputs_[0].ElementNum() != static_cast<int64_t>(rows) * k_) return kLiteError;
     if (computed_by_sibling_) {
-      // a sibling's launch wrote this kernel's output buffer during this run, on the session's stream
+      // A sibling's launch wrote this kernel's output buffer, on the session's stream.  It is this run's result if
+      // the input is still the memory the sibling read -- and, where a kernel of this provider produces the input,
+      // still the version it read (a producer counts its deliveries).  Where the producer is a builtin kernel the
+      // order of a Lite session is what is left to lean on: siblings execute in the same run as the member that
+      // launched for them.  MI355X_NO_SIBLING_GROUPS=1 in the environment switches the grouping off.
       computed_by_sibling_ = false;
       if (sibling_rows_ == rows && sibling_host_ == inputs_[0].Data().get() &&
-          sibling_dev_ == inputs_[0].GetDeviceData()) {
+          sibling_dev_ == inputs_[0].GetDeviceData() && sibling_version_ == Published::Version(sibling_dev_)) {
         return io_.Deliver(&outputs_[0]);
       }
     }
@@ -367,8 +463,15 @@ class MatmulKernel : public kernel::Kernel {
     void *c = io_.Output(outputs_[0].DataSize());
     if (a == nullptr || c == nullptr) return kLiteNullptr;
     int rc = MI_ERROR;
+    QuantOnDevice on_dev;
     if (full_ != nullptr) {
       rc = mi_matmul_run(full_, a, rows, static_cast<int8_t *>(c), io_.stream());
+    } else if (a == inputs_[0].GetDeviceData() && Published::Quant(const_cast<int8_t *>(a), &on_dev) &&
+               (!on_dev.per_row || on_dev.rows == rows)) {
+      // the input was left on the device by this provider's DynamicQuant kernel, and so were its scale and zero
+      // point (one block, or one per row): they are read there, in stream order, and the host has nothing to wait for
+      rc = on_dev.per_row ? mi_dynmm_run_rows(dyn_, a, rows, on_dev.params, static_cast<float *>(c), io_.stream())
+                          : mi_dynmm_run_chained(dyn_, a, rows, on_dev.params, static_cast<float *>(c), io_.stream());
     } else {
       // dynamic quant: the input's scale and zero point were written by the preceding DynamicQuant kernel during
       // this very inference, so they are read now, not in Prepare (matmul_dynamic_base_int8.cc:146-176)
@@ -429,18 +532,48 @@ class MatmulKernel : public kernel::Kernel {
       m->sibling_rows_ = rows;
       m->sibling_host_ = inputs_[0].Data().get();
       m->sibling_dev_ = inputs_[0].GetDeviceData();
+      m->sibling_version_ = Published::Version(m->sibling_dev_);
+    }
+    return io_.Deliver(&outputs_[0]);
+  }
+
+  // A constant weight of rank > 2: output matrix i = activation matrix a_offsets[i] x weight matrix b_offsets[i], the
+  // indices by the reference's broadcast rule (MatmulBaseInt8CPUKernel::Run, matmul_base_int8.cc:549-568).
+  int ExecuteBatched() {
+    const auto ashape = inputs_[0].Shape(), wshape = inputs_[kWeightIndex].Shape();
+    if (ashape.size() < 2 || ashape.size() > MI_MAX_DIMS || wshape.size() > MI_MAX_DIMS || ashape.back() != k_) return kLiteError;
+    if (inputs_[0].ElementNum() == 0) return kSuccess;
+    std::vector<int32_t> a32(ashape.begin(), ashape.end()), w32(wshape.begin(), wshape.end());
+    int32_t batch = 0;
+    const int64_t cap = outputs_[0].ElementNum() / n_;  // at least one row per output matrix
+    std::vector<int32_t> a_off(static_cast<size_t>(cap)), b_off(static_cast<size_t>(cap));
+    if (mi_matmul_broadcast_offsets(a32.data(), static_cast<int32_t>(a32.size()), w32.data(),
+                                    static_cast<int32_t>(w32.size()), static_cast<int32_t>(cap), &batch, a_off.data(),
+                                    b_off.data()) != MI_OK) {
+      return kLiteError;
+    }
+    const int32_t rows = static_cast<int32_t>(ashape[ashape.size() - 2]);
+    if (outputs_[0].ElementNum() != static_cast<int64_t>(batch) * rows * n_) return kLiteError;
+    const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
+    void *c = io_.Output(outputs_[0].DataSize());
+    if (a == nullptr || c == nullptr) return kLiteNullptr;
+    if (mi_matmul_run_batched(full_, a, rows, batch, a_off.data(), b_off.data(), static_cast<int8_t *>(c),
+                              io_.stream()) != MI_OK) {
+      return kLiteError;
     }
     return io_.Deliver(&outputs_[0]);
   }
 
   bool b_transpose_;
   int act_;
-  int32_t k_ = 0;
+  int32_t k_ = 0, n_ = 0;
+  bool batched_ = false;
   std::shared_ptr<SiblingGroup> group_;
   bool computed_by_sibling_ = false;  // the output buffer already holds this run's result
   int32_t sibling_rows_ = 0;          // ... for this row count and this input memory
   const void *sibling_host_ = nullptr;
   void *sibling_dev_ = nullptr;
+  int64_t sibling_version_ = 0;
   mi_matmul *full_ = nullptr;
   mi_dynmm *dyn_ = nullptr;
   DeviceIo io_;
@@ -466,7 +599,11 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
   const MSTensor &w = in[kWeightIndex];
   const bool out_i8 = out[0].DataType() == DataType::kNumberTypeInt8;
   const bool out_f32 = out[0].DataType() == DataType::kNumberTypeFloat32;
-  if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || w.Shape().size() != 2) return nullptr;
+  if (!w.IsConst() || w.DataType() != DataType::kNumberTypeInt8 || w.Shape().size() < 2) return nullptr;
+  // a weight of rank > 2 (a batch of matrices) is taken for the full-quant MatMul; FullConnection has none, and the
+  // dynamic MatMul's batched form stays with the builtin kernel
+  const bool batched_w = w.Shape().size() > 2;
+  if (batched_w && (prim->value_as_MatMulFusion() == nullptr || !out_i8 || w.Shape().size() > MI_MAX_DIMS)) return nullptr;
   // full quant needs per-tensor activations; the dynamic MatMul also takes one input scale per row
   if (!(out_i8 || out_f32) || (out_i8 && (!PerTensor(in[0]) || !PerTensor(out[0])))) return nullptr;
   if (act != MI_ACT_NONE && act != MI_ACT_RELU && act != MI_ACT_RELU6) return nullptr;
@@ -479,7 +616,10 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
   // (a dynamic-quant MatMul finds its input's scale on the tensor only at run time: DynamicQuant writes it there)
   if (in[0].DataType() != DataType::kNumberTypeInt8) return nullptr;
   const auto wshape = w.Shape();
-  const int64_t n = b_transpose ? wshape[0] : wshape[1], k = b_transpose ? wshape[1] : wshape[0];
+  const size_t wr = wshape.size();
+  const int64_t n = b_transpose ? wshape[wr - 2] : wshape[wr - 1], k = b_transpose ? wshape[wr - 1] : wshape[wr - 2];
+  for (size_t i = 0; i + 2 < wr; ++i)
+    if (wshape[i] <= 0) return nullptr;
   const size_t nfilter = w.QuantParams().size();
   if (n <= 0 || k <= 0 || (nfilter != 1 && nfilter != static_cast<size_t>(n))) return nullptr;
   const auto ashape = in[0].Shape();
@@ -491,6 +631,16 @@ std::shared_ptr<kernel::Kernel> MatmulCreator(const std::vector<MSTensor> &in, c
   }
   if (known) {
     if (prim->value_as_MatMulFusion() != nullptr ? ashape.back() != k : elements % k != 0) return nullptr;
+    if (batched_w) {  // the batch extents must broadcast (InitBroadcastParams, matmul_fp32_base.cc:611-620)
+      if (ashape.size() < 2 || ashape.size() > MI_MAX_DIMS) return nullptr;
+      std::vector<int32_t> a32(ashape.begin(), ashape.end()), w32(wshape.begin(), wshape.end());
+      int32_t batch = 0;
+      std::vector<int32_t> ao(1 << 16), bo(1 << 16);
+      if (mi_matmul_broadcast_offsets(a32.data(), static_cast<int32_t>(a32.size()), w32.data(),
+                                      static_cast<int32_t>(w32.size()), 1 << 16, &batch, ao.data(), bo.data()) != MI_OK) {
+        return nullptr;
+      }
+    }
   }
   return std::make_shared<MatmulKernel>(in, out, prim, ctx, b_transpose, act);
 }
@@ -505,7 +655,7 @@ class ConvKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(context_, GetConfig("mi355x"), outputs_[0].Name());
     return Build();
   }
 
@@ -634,7 +784,7 @@ class DynamicQuantKernel : public kernel::Kernel {
   }
 
   int Prepare() override {
-    io_.Configure(SessionStream(context_), GetConfig("mi355x"), outputs_[0].Name());
+    io_.Configure(context_, GetConfig("mi355x"), outputs_[0].Name());
     const auto *p = primitive_->value_as_DynamicQuant();
     per_row_ = p->prefer_axes() != nullptr && p->prefer_axes()->size() > 0;
     return ToStatus(mi_dynquant_create(p->symmetric() ? 1 : 0, &dq_));
@@ -646,49 +796,77 @@ class DynamicQuantKernel : public kernel::Kernel {
     const auto *x = static_cast<const float *>(io_.Input(&inputs_[0]));
     auto *q = static_cast<int8_t *>(io_.Output(outputs_[0].DataSize()));
     if (x == nullptr || q == nullptr) return kLiteNullptr;
-    // the scales and zero points always travel to the host: the consumer, builtin or not, reads them from the tensor
+    // The scales and zero points stay on the device for the consumers of this provider (QuantOnDevice).  A builtin
+    // consumer reads them from the tensor, so they also travel to the host -- as a copy into page-locked memory
+    // queued behind the kernels, complete once Deliver has waited for the output's own copy: one wait per run instead
+    // of two.  An output declared device-only has no builtin consumer: nothing is waited for, and the tensor's quant
+    // parameters are left as they are.
+    QuantOnDevice quant;
+    quant.per_row = per_row_;
+    size_t blocks = 1;
     if (per_row_) {  // the creator admitted only "every axis but the last": one run per row of the last axis
       const int64_t unit = inputs_[0].Shape().back();
       const int64_t segments = n / unit;
-      std::vector<mi_dq_params> ps(static_cast<size_t>(segments));
-      const size_t bytes = ps.size() * sizeof(mi_dq_params);
-      auto *dev = static_cast<mi_dq_params *>(row_params_.Reserve(bytes));
-      if (dev == nullptr || mi_dynquant_run_segments(dq_, x, segments, unit, q, dev, io_.stream()) != MI_OK ||
-          mi_copy_to_host(ps.data(), dev, bytes, io_.stream()) != MI_OK) {
+      blocks = static_cast<size_t>(segments);
+      auto *dev = static_cast<mi_dq_params *>(row_params_.Reserve(blocks * sizeof(mi_dq_params)));
+      if (dev == nullptr || mi_dynquant_run_segments(dq_, x, segments, unit, q, dev, io_.stream()) != MI_OK) {
         return kLiteError;
       }
-      std::vector<QuantParam> qps(ps.size());
-      for (size_t i = 0; i < ps.size(); ++i) {
-        qps[i].bit_num = 8;
-        qps[i].scale = ps[i].scale;
-        qps[i].zero_point = ps[i].zero_point;
-        qps[i].min = ps[i].real_min;
-        qps[i].max = ps[i].real_max;
-      }
-      outputs_[0].SetQuantParams(qps);
-      return io_.Deliver(&outputs_[0]);
+      quant.params = dev;
+      quant.rows = segments;
+    } else {
+      if (mi_dynquant_run(dq_, x, n, q, io_.stream()) != MI_OK) return kLiteError;
+      quant.params = mi_dynquant_device_params(dq_);
     }
-    mi_dq_params p{};
-    if (mi_dynquant_run(dq_, x, n, q, io_.stream()) != MI_OK ||
-        mi_dynquant_get_params(dq_, io_.stream(), &p) != MI_OK) {
-      return kLiteError;
+    if (!io_.host_copy()) return io_.Deliver(&outputs_[0], &quant);
+    const size_t bytes = blocks * sizeof(mi_dq_params);
+    auto *ps = static_cast<mi_dq_params *>(host_params_.Reserve(bytes));
+    if (ps == nullptr || mi_copy_to_host_async(ps, quant.params, bytes, io_.stream()) != MI_OK) return kLiteError;
+    const int rc = io_.Deliver(&outputs_[0], &quant);  // copies the output to the host and waits for the stream
+    if (rc != kSuccess) return rc;
+    // what DynamicQuantCPUKernel::CalculatePerlayerScaleZp / CalculatePerChannelScaleZp publish on the output tensor
+    // (dynamic_quant.cc:156-218)
+    std::vector<QuantParam> qps(blocks);
+    for (size_t i = 0; i < blocks; ++i) {
+      qps[i].bit_num = 8;
+      qps[i].scale = ps[i].scale;
+      qps[i].zero_point = ps[i].zero_point;
+      qps[i].min = ps[i].real_min;
+      qps[i].max = ps[i].real_max;
     }
-    // what DynamicQuantCPUKernel::CalculatePerlayerScaleZp publishes on the output tensor (dynamic_quant.cc:156-186)
-    QuantParam qp{};
-    qp.bit_num = 8;
-    qp.scale = p.scale;
-    qp.zero_point = p.zero_point;
-    qp.min = p.real_min;
-    qp.max = p.real_max;
-    outputs_[0].SetQuantParams({qp});
-    return io_.Deliver(&outputs_[0]);
+    outputs_[0].SetQuantParams(qps);
+    return kSuccess;
   }
 
  private:
+  // page-locked host memory (grows, never shrinks)
+  class PinnedBuffer {
+   public:
+    PinnedBuffer() = default;
+    PinnedBuffer(const PinnedBuffer &) = delete;
+    PinnedBuffer &operator=(const PinnedBuffer &) = delete;
+    ~PinnedBuffer() { mi_host_free(p_); }
+    void *Reserve(size_t bytes) {
+      if (bytes > cap_) {
+        mi_host_free(p_);
+        p_ = nullptr;
+        cap_ = 0;
+        if (mi_host_malloc(bytes, &p_) != MI_OK) return nullptr;
+        cap_ = bytes;
+      }
+      return p_;
+    }
+
+   private:
+    void *p_ = nullptr;
+    size_t cap_ = 0;
+  };
+
   mi_dynquant *dq_ = nullptr;
   bool per_row_ = false;
   DeviceIo io_;
   DeviceBuffer row_params_;
+  PinnedBuffer host_params_;
 };
 
 std::shared_ptr<kernel::Kernel> DynamicQuantCreator(const std::vector<MSTensor> &in, const std::vector<MSTensor> &out,
@@ -734,5 +912,7 @@ struct Registrar {
 
 // How many times sibling MatMuls went out as one launch (for tests and for checking that a model's siblings were found).
 extern "C" int64_t mi355x_provider_group_launches() { return g_group_launches.load(std::memory_order_relaxed); }
+// How many sessions currently hold a stream (for tests: destroying a session's last kernel gives its stream back).
+extern "C" int64_t mi355x_provider_session_streams() { return static_cast<int64_t>(SessionStreams::Count()); }
 }  // namespace mi355x
 }  // namespace mindspore

@@ -351,6 +351,44 @@ _oracle = None
 _reference = None
 
 
+def pack_weight_4x16(w_nk):
+    """The offline weight layout of MatMulDynamicSdotInt8Kernel for a weight given as [N][K]: blocks
+    [N / 16][K / 4][16 channels][4 K-bytes], N padded to 16 and K to 4 with zeros.  Restates
+    RowMajor2Row4x16MajorInt8 (on the [N, K] weight of transpose_b) and RowMajor2Col4x16MajorInt8 (on its [K, N]
+    transpose), nnacl/int8/matmul_int8.c:143-156 and :770-784, which produce the same bytes."""
+    w_nk = np.ascontiguousarray(w_nk, dtype=np.int8)
+    n, k = w_nk.shape
+    n16, k4 = -(-n // 16) * 16, -(-k // 4) * 4
+    padded = np.zeros((n16, k4), np.int8)
+    padded[:n, :k] = w_nk
+    return np.ascontiguousarray(padded.reshape(n16 // 16, 16, k4 // 4, 4).transpose(0, 2, 1, 3)).reshape(-1)
+
+
+def broadcast_offsets(a_shape, b_shape):
+    """(a_offsets, b_offsets) per output matrix of a batched MatMul: restates
+    MatmulFp32BaseCPUKernel::InitBroadcastParams (mindspore/lite/src/litert/kernel/cpu/fp32/matmul_fp32_base.cc:
+    576-646) in the terms of NumPy broadcasting over the batch axes, with the reference's extension that a batch
+    extent may divide the other operand's (index scaled proportionally)."""
+    rank = max(len(a_shape), len(b_shape), 4)
+    a = [1] * (rank - len(a_shape)) + list(a_shape)
+    b = [1] * (rank - len(b_shape)) + list(b_shape)
+    nb = rank - 2
+    mx = [max(a[j], b[j]) for j in range(nb)]
+    for j in range(nb):
+        mn = max(min(a[j], b[j]), 1)
+        if mx[j] != mn and mx[j] % mn != 0:
+            raise ValueError("batch extents %d and %d cannot be broadcast" % (a[j], b[j]))
+    a_off, b_off = [], []
+    for idx in np.ndindex(*mx) if nb else [()]:
+        ao = bo = 0
+        for j in range(nb):
+            ao = ao * a[j] + idx[j] * a[j] // mx[j]
+            bo = bo * b[j] + idx[j] * b[j] // mx[j]
+        a_off.append(ao)
+        b_off.append(bo)
+    return a_off, b_off
+
+
 def oracle():
     global _oracle
     if _oracle is None:

@@ -178,6 +178,35 @@ def test_matmul_reuse_and_row_counts(orc):
         assert np.array_equal(kern.run(a), orc.matmul_int8(**case)), m
 
 
+def test_handle_survives_a_failed_allocation_of_the_decode_copy(orc):
+    """The blocked second copy of the weights is an optimisation: when the device has no room for it the handle is
+    still created, and 2..32 rows run on the kernels that read the row-major weights."""
+    from mindspore_amd import lib
+    rng = np.random.default_rng(77)
+    L = lib.init(0)
+    n, k = 100, 300
+    blocked_bytes = 256 * 512  # n and k padded to 256
+    for rows in (2, 7, 32):
+        c = _mm_case(rng, rows, n, k, True, True, True, 0)
+        want = orc.matmul_int8(**c)
+        assert L.mi_debug_fail_alloc(blocked_bytes) == 0
+        try:
+            got, kern = _gpu_matmul(c, device_tensors=True)
+        finally:
+            L.mi_debug_fail_alloc(0)
+        assert np.array_equal(got, want), rows
+        got2, _ = _gpu_matmul(c, device_tensors=True)  # with the copy: the matrix-core decode kernel
+        assert np.array_equal(got2, want), rows
+    # an allocation the handle cannot do without still fails the create, with the memory status
+    assert L.mi_debug_fail_alloc(256 * 768 + 16) == 0  # the row-major packed weights
+    try:
+        with pytest.raises(lib.MiError) as err:
+            _gpu_matmul(c)
+        assert err.value.code == lib.MI_MEMORY_FAILED
+    finally:
+        L.mi_debug_fail_alloc(0)
+
+
 def test_golden_small_cases(orc):
     g = np.load(GOLDEN)
     for i in range(int(g["mm_count"][0])):

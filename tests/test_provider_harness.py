@@ -378,6 +378,42 @@ def test_sibling_fullconnections_run_as_one_launch(H, orc):
 
 
 @pytest.mark.gpu
+def test_a_sibling_result_is_not_delivered_for_a_later_version_of_the_input(H, orc):
+    """Two siblings behind a provider kernel.  Run 1 executes only the first sibling, which launches for both; run 2
+    (new input, same tensor memory) executes only the second: it must not hand out what run 1 left in its buffer.
+    The producer counts its deliveries, and the second sibling sees that the count moved on."""
+    rng = np.random.default_rng(23)
+    k0, k = 96, 256
+
+    def fc(n, kk, producer=None):
+        a, w, sw, b, ins = _fc_inputs(rng, 4, n, kk)
+        ins[0] = tensor(I8, (4, kk), None, False, [(0.05, 5)]) if producer is not None else ins[0]
+        node = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)], producer=producer)
+        assert node.stage == OK, (node.stage, node.code)
+        return node, w, sw, b
+
+    head, w0, sw0, b0 = fc(k, k0)
+    (first, w1, s1, b1), (second, w2, s2, b2) = fc(128, k, head), fc(64, k, head)
+    before = H.mi355x_provider_group_launches()
+    x1 = rng.integers(-128, 128, (4, k0), dtype=np.int8)
+    h1, _ = head.run(x1)
+    first.run_linked()   # launches for both siblings; the second one is not executed in this run
+    assert H.mi355x_provider_group_launches() == before + 1
+    x2 = rng.integers(-128, 128, (4, k0), dtype=np.int8)
+    h2, _ = head.run(x2)
+    assert not np.array_equal(h1, h2)
+    second.run_linked()  # first in this run: computes from the new input
+    got, _ = second.output()
+    want = orc.matmul_int8(h2, w2, b2, 0.05, 5, s2, np.zeros(64, np.int32), 0.05, 5, 0, True)
+    assert np.array_equal(got, want)
+    first.run_linked()
+    got, _ = first.output()
+    assert np.array_equal(got, orc.matmul_int8(h2, w1, b1, 0.05, 5, s1, np.zeros(128, np.int32), 0.05, 5, 0, True))
+    for node in (second, first, head):
+        node.close()
+
+
+@pytest.mark.gpu
 def test_what_the_provider_declines(H):
     rng = np.random.default_rng(2)
     a, w, sw, b, ins = _fc_inputs(rng, 4, 8, 16, w_const=False)            # weight produced at run time
@@ -577,38 +613,150 @@ def test_activations_stay_on_the_device_between_provider_kernels(H, orc):
 
 @pytest.mark.gpu
 def test_dynamic_quant_feeds_the_dynamic_matmul_on_the_device(H, orc):
-    """DynamicQuant -> dynamic MatMul sharing the int8 tensor: the bytes stay in device memory (declared device-only),
-    the scale and zero point still reach the host tensor, where the MatMul reads them at Execute."""
+    """DynamicQuant -> dynamic MatMul sharing the int8 tensor.  The MatMul takes the bytes AND the scale / zero point
+    (one block, or one per row) from device memory, where the DynamicQuant kernel of this provider left them.  By
+    default the quant parameters also reach the host tensor (a builtin consumer would read them there); with the
+    tensor declared device-only nothing travels to the host and nothing is waited for."""
+    from mindspore_amd import lib
+    L = lib.load()
     rng = np.random.default_rng(14)
     w = rng.integers(-127, 128, (80, 96), dtype=np.int8)
     sw = rng.uniform(1e-3, 1e-2, 80).astype(np.float32).astype(np.float64)
     bias = rng.standard_normal(80).astype(np.float32)
     zw = np.zeros(80, np.int32)
     for per_row in (False, True):
-        dq_op = op(DYNQUANT, symmetric=1, n_prefer_axes=1, prefer_axes=(0,)) if per_row else op(DYNQUANT)
-        dq = Node(H, dq_op, [tensor(F32, (37, 96), None)], I8, out_name=b"q", device_only=b"q")
-        assert dq.stage == OK, (dq.stage, dq.code)
+        for device_only in (None, b"q", b"*"):
+            dq_op = op(DYNQUANT, symmetric=1, n_prefer_axes=1, prefer_axes=(0,)) if per_row else op(DYNQUANT)
+            dq = Node(H, dq_op, [tensor(F32, (37, 96), None)], I8, out_name=b"q", device_only=device_only)
+            assert dq.stage == OK, (dq.stage, dq.code)
+            mm = Node(H, op(MATMUL, transpose_b=1),
+                      [tensor(I8, (37, 96), None), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+                       tensor(F32, (80,), bias, True)], F32, producer=dq, out_name=b"y", device_only=device_only)
+            assert mm.stage == OK, (mm.stage, mm.code)
+            for rows in (37, 5, 64):
+                x = (rng.standard_normal((rows, 96)) * 3).astype(np.float32)
+                syncs0 = L.mi_debug_sync_count()
+                _, qp = dq.run(x)
+                syncs1 = L.mi_debug_sync_count()
+                mm.run_linked()
+                syncs2 = L.mi_debug_sync_count()
+                if per_row:
+                    q_ref, scales_ref, _ = orc.dynamic_quant_segments(x, True)
+                    ref = orc.dynamic_matmul_rows(q_ref, w, bias, scales_ref, 0, sw, zw)
+                    qp_ref = [(sc, 0) for sc in scales_ref]
+                else:
+                    q_ref, s_ref, z_ref = orc.dynamic_quant(x, False)
+                    ref = orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw)
+                    qp_ref = [(s_ref, z_ref)]
+                if device_only is None:
+                    # upload of x, then ONE wait for both the int8 bytes and the parameters; upload-free MatMul, one
+                    # wait for its output
+                    assert dq.state() == (True, True) and qp == qp_ref
+                    assert (syncs1 - syncs0, syncs2 - syncs1) == (2, 1)
+                else:
+                    assert dq.state() == (False, True)
+                    # after the upload of x the host waits for nothing until an output has to reach it
+                    assert syncs1 - syncs0 == 1
+                    assert syncs2 - syncs1 == (1 if device_only == b"q" else 0)
+                if device_only != b"*":
+                    y, _ = mm.output()
+                    assert y.shape == ref.shape and np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (per_row, rows)
+            mm.close()
+            dq.close()
+
+
+@pytest.mark.gpu
+def test_time_of_dynamic_quant_into_the_qkv_matmul(H, orc):
+    """Per-layer host time of DynamicQuant (4096 x 768) -> QKV dynamic MatMul (2304 channels) through the provider:
+    with every tensor handed over on the host, with the int8 tensor device-only, and with both outputs device-only
+    (the part a following provider kernel would see).  Printed (-s shows it); the one assertion is that keeping the
+    tensors on the device is not slower than copying them."""
+    import time
+    from mindspore_amd import lib, workloads as wl
+    L = lib.load()
+    x = wl.bert_c3_activation(768)
+    wt = wl.bert_c3_weights("qkv", 2304, 768)
+    times = {}
+    for device_only in (None, b"q", b"*"):
+        dq = Node(H, op(DYNQUANT), [tensor(F32, x.shape, None)], I8, out_name=b"q", device_only=device_only)
         mm = Node(H, op(MATMUL, transpose_b=1),
-                  [tensor(I8, (37, 96), None), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
-                   tensor(F32, (80,), bias, True)], F32, producer=dq, out_name=b"y", device_only=b"q")
-        assert mm.stage == OK, (mm.stage, mm.code)
-        for rows in (37, 5, 64):
-            x = (rng.standard_normal((rows, 96)) * 3).astype(np.float32)
-            _, qp = dq.run(x)
-            assert dq.state() == (False, True)
+                  [tensor(I8, x.shape, None), tensor(I8, wt["w"].shape, wt["w"], True, [(s, 0) for s in wt["sw"]]),
+                   tensor(F32, (2304,), wt["bias"], True)], F32, producer=dq, out_name=b"y", device_only=device_only)
+        assert dq.stage == OK and mm.stage == OK
+        for _ in range(3):
+            dq.run(x)
             mm.run_linked()
-            y, _ = mm.output()
-            if per_row:
-                q_ref, scales_ref, _ = orc.dynamic_quant_segments(x, True)
-                assert [p[0] for p in qp] == list(scales_ref)
-                ref = orc.dynamic_matmul_rows(q_ref, w, bias, scales_ref, 0, sw, zw)
-            else:
-                q_ref, s_ref, z_ref = orc.dynamic_quant(x, False)
-                assert qp == [(s_ref, z_ref)]
-                ref = orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw)
-            assert y.shape == ref.shape and np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (per_row, rows)
+        L.mi_stream_synchronize(None)
+        syncs = L.mi_debug_sync_count()
+        t0 = time.perf_counter()
+        reps = 10
+        for _ in range(reps):
+            dq.run(x)
+            mm.run_linked()
+        L.mi_device_free(None)  # (no-op)
+        t = (time.perf_counter() - t0) / reps
+        times[device_only] = (t, (L.mi_debug_sync_count() - syncs) / reps)
         mm.close()
         dq.close()
+    print("DynamicQuant -> QKV per layer (host clock, incl. the harness's copy of x into the input tensor): "
+          + ", ".join("%s: %.0f us, %.0f waits" % (k.decode() if k else "host hand-over", v[0] * 1e6, v[1])
+                      for k, v in times.items()))
+    assert times[b"*"][0] <= times[None][0]
+
+
+@pytest.mark.gpu
+def test_batched_constant_weight_through_the_provider(H, orc):
+    """MatMulFusion whose constant weight has rank 3: one output matrix per (activation matrix, weight matrix) pair
+    by the reference's broadcast rule; the creator declines the same weight for FullConnection and for fp32 output."""
+    from oracle import pyoracle
+    rng = np.random.default_rng(21)
+    n, k = 44, 80
+    sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
+    bias = rng.integers(-3000, 3001, n).astype(np.int32)
+    for a_shape, w_batch in (((3, 9, k), (3,)), ((2, 3, 40, k), (3,)), ((6, 5, k), (2,)), ((50, k), (4,))):
+        w = rng.integers(-128, 128, w_batch + (n, k), dtype=np.int8)
+        ins = [tensor(I8, a_shape, None, False, [(0.02, -3)]), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+               tensor(I32, (n,), bias, True)]
+        node = Node(H, op(MATMUL, transpose_b=1), ins, I8, [(0.05, 5)])
+        assert node.stage == OK, (node.stage, node.code)
+        a = rng.integers(-128, 128, a_shape, dtype=np.int8)
+        got, _ = node.run(a)
+        a_off, b_off = pyoracle.broadcast_offsets(a_shape, w.shape)
+        rows = a_shape[-2]
+        assert got.size == len(a_off) * rows * n
+        got = got.reshape(len(a_off), rows, n)
+        for i, (ai, bi) in enumerate(zip(a_off, b_off)):
+            want = orc.matmul_int8(a.reshape(-1, rows, k)[ai], w.reshape(-1, n, k)[bi], bias, 0.02, -3, sw,
+                                   np.zeros(n, np.int32), 0.05, 5, 0, True)
+            assert np.array_equal(got[i], want), (a_shape, w_batch, i)
+        node.close()
+    w = rng.integers(-128, 128, (3, n, k), dtype=np.int8)
+    wq = [(s, 0) for s in sw]
+    fc = Node(H, op(FC, has_bias=0), [tensor(I8, (3, 9, k), None, False, [(0.02, -3)]), tensor(I8, w.shape, w, True, wq)],
+              I8, [(0.05, 5)])
+    assert fc.stage in (DECLINED, INFER_FAILED), fc.stage
+    dyn = Node(H, op(MATMUL, transpose_b=1), [tensor(I8, (3, 9, k), None), tensor(I8, w.shape, w, True, wq)], F32)
+    assert dyn.stage == DECLINED, dyn.stage
+    bad = Node(H, op(MATMUL, transpose_b=1), [tensor(I8, (2, 9, k), None, False, [(0.02, -3)]),
+                                              tensor(I8, w.shape, w, True, wq)], I8, [(0.05, 5)])
+    assert bad.stage in (DECLINED, INFER_FAILED), bad.stage  # batch extents 2 and 3 do not broadcast
+
+
+@pytest.mark.gpu
+def test_a_session_gives_its_stream_back(H, orc):
+    """Every kernel holds a reference on its session's stream; destroying the session's last kernel destroys it."""
+    H.mi355x_provider_session_streams.restype = C.c_int64
+    rng = np.random.default_rng(22)
+    before = H.mi355x_provider_session_streams()
+    a, w, sw, b, ins = _fc_inputs(rng, 4, 16, 32)
+    one = Node(H, op(FC, has_bias=1), ins, I8, [(0.05, 5)])
+    two = Node(H, op(FC, has_bias=1), _fc_inputs(rng, 4, 16, 32)[4], I8, [(0.05, 5)])
+    assert H.mi355x_provider_session_streams() == before + 2  # the harness gives every unlinked node a session of its own
+    one.run(a)
+    one.close()
+    assert H.mi355x_provider_session_streams() == before + 1
+    two.close()
+    assert H.mi355x_provider_session_streams() == before
 
 
 @pytest.mark.gpu

@@ -89,3 +89,40 @@ def test_no_alloc_entry_point_rejects_what_does_not_fit():
     assert L.mi_matmul_run_noalloc(None, a.data_ptr(), 1, c.data_ptr(), None) == lib.MI_NULL_PTR
     assert L.mi_matmul_run_noalloc(kern._h, a.data_ptr(), -1, c.data_ptr(), None) == lib.MI_PARAM_INVALID
     assert L.mi_matmul_run_noalloc(kern._h, a.data_ptr(), 0, c.data_ptr(), None) == lib.MI_OK
+
+
+def test_no_alloc_entry_point_leaves_free_device_memory_unchanged(orc):
+    """Free device memory (hipMemGetInfo) before and after a series of calls on fresh shapes: the entry point takes
+    its padded rows and padded output from the static scratch area, so nothing may be allocated, whereas the
+    allocating entry point grows the handle's workspaces on the same calls."""
+    import torch
+    L = lib.load()
+    rng = np.random.default_rng(9)
+    n, k = 1030, 4000  # deep % 16 != 0 and col % 4 != 0: both workspaces are needed
+    case = _case(rng, n, k, True)
+
+    def make():
+        return K.MatmulInt8Kernel(case["w"], case["bias"], QP(case["sx"], case["zx"]),
+                                  [QP(float(s), int(z)) for s, z in zip(case["sw"], case["zw"])],
+                                  QP(case["so"], case["zo"]), True, 0)
+    kern = make()
+    rows_list = (900, 1500, 33, 1600)
+    a = torch.from_numpy(rng.integers(-128, 128, (max(rows_list), k), dtype=np.int8)).cuda()
+    c = torch.empty((max(rows_list), n), dtype=torch.int8, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for rows in rows_list:
+        assert L.mi_matmul_run_noalloc(kern._h, a.data_ptr(), rows, c.data_ptr(), stream) == lib.MI_OK
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    got = c[:rows_list[-1]].cpu().numpy()
+    case["a"] = a[:rows_list[-1]].cpu().numpy()
+    assert np.array_equal(got, orc.matmul_int8(**case))
+    # the same calls through the allocating entry point do take device memory (the check above can see allocations)
+    for rows in rows_list:
+        assert L.mi_matmul_run(kern._h, a.data_ptr(), rows, c.data_ptr(), stream) == lib.MI_OK
+    torch.cuda.synchronize()
+    free_alloc, _ = torch.cuda.mem_get_info()
+    assert free_alloc < free_before
