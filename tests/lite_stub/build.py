@@ -10,12 +10,31 @@ OUT = os.path.join(HERE, "_build", "libprovider_harness.so")
 REFERENCE = "/root/reference"
 
 
+# The reference's own kernel registry: three sources that compile against the stand-in API headers of this directory
+# (they only store and hand back the creator functors) plus the reference's public registration header.
+REAL_REGISTRY_HEADER = os.path.join(REFERENCE, "mindspore", "lite", "include", "registry", "register_kernel.h")
+REAL_REGISTRY_SOURCES = [os.path.join(REFERENCE, "mindspore", "lite", "src", p) for p in (
+    "registry/register_kernel.cc", "registry/register_kernel_impl.cc", "common/log.cc")]
+
+
+def real_registry_available():
+    return all(os.path.exists(p) for p in [REAL_REGISTRY_HEADER] + REAL_REGISTRY_SOURCES)
+
+
 def build_harness():
+    """With the reference tree present the harness is linked with the reference's own RegisterKernel /
+    RegistryKernelImpl (compiled from where they lie); without it, with the stand-in table of
+    include/registry/register_kernel.h.  ph_registry_is_real() tells which one a built harness holds."""
     os.makedirs(os.path.dirname(OUT), exist_ok=True)
-    subprocess.check_call([
-        "g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-pthread", "-Wall", "-I" + HERE, "-I" + os.path.join(ROOT, "include"),
-        os.path.join(HERE, "harness.cc"), "-L" + os.path.join(ROOT, "mindspore_amd"), "-lmi355x_int8",
-        "-Wl,-rpath,$ORIGIN/../../../mindspore_amd", "-o", OUT])
+    cmd = ["g++", "-std=c++17", "-O1", "-fPIC", "-shared", "-pthread", "-Wall", "-I" + HERE,
+           "-I" + os.path.join(ROOT, "include")]
+    sources = [os.path.join(HERE, "harness.cc")]
+    if real_registry_available():
+        cmd += ["-DPH_REAL_REGISTRY_HEADER=\"%s\"" % REAL_REGISTRY_HEADER, "-I" + os.path.join(REFERENCE, "mindspore", "lite"),
+                "-I" + REFERENCE, "-I" + os.path.join(REFERENCE, "mindspore", "core")]
+        sources += REAL_REGISTRY_SOURCES
+    subprocess.check_call(cmd + sources + ["-L" + os.path.join(ROOT, "mindspore_amd"), "-lmi355x_int8",
+                                           "-Wl,-rpath,$ORIGIN/../../../mindspore_amd", "-o", OUT])
     return OUT
 
 

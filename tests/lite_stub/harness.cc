@@ -359,6 +359,34 @@ int32_t ph_infer(const ph_op *op, const char *provider, const ph_tensor *inputs,
 
 void ph_destroy(void *h) { delete static_cast<Session *>(h); }
 
+// 1 when this harness was built with the reference's own RegisterKernel / RegistryKernelImpl, 0 with the stand-in.
+int32_t ph_registry_is_real(void) {
+#ifdef PH_REAL_REGISTRY_HEADER
+  return 1;
+#else
+  return 0;
+#endif
+}
+
+// Registry lookup alone, as the scheduler makes it (scheduler.cc:1131-1177): 1 when a creator is registered under
+// exactly (arch, provider, data type, op type).
+int32_t ph_lookup(const char *arch, const char *provider, int32_t dtype, int32_t op_type) {
+  schema::Primitive prim;
+  prim.type_ = static_cast<schema::PrimitiveType>(op_type);
+  mindspore::registry::KernelDesc desc{static_cast<mindspore::DataType>(dtype), op_type, arch, provider};
+  return mindspore::registry::RegisterKernel::GetCreator(&prim, &desc) != nullptr ? 1 : 0;
+}
+
+// Registers a creator that declines everything under (arch, provider, dtype, op type); returns the registry's status
+// code (0 = registered).
+int32_t ph_register_declining(const char *arch, const char *provider, int32_t dtype, int32_t op_type) {
+  const auto creator = [](const std::vector<MSTensor> &, const std::vector<MSTensor> &, const schema::Primitive *,
+                          const mindspore::Context *) -> std::shared_ptr<mindspore::kernel::Kernel> { return nullptr; };
+  const mindspore::Status st = mindspore::registry::RegisterKernel::RegKernel(
+    arch, provider, static_cast<mindspore::DataType>(dtype), op_type, creator);
+  return st.IsOk() ? 0 : static_cast<int32_t>(st.StatusCode());
+}
+
 // 1 when a KernelInterface is registered under `provider` for the operator type, else 0.
 int32_t ph_has_provider_interface(const char *provider, int32_t op_type) {
   schema::Primitive prim;

@@ -4,10 +4,12 @@
 namespace mindspore {
 enum class DataType : int {
   kTypeUnknown = 0,
+  kNumberTypeBegin = 29,
   kNumberTypeInt8 = 32,
   kNumberTypeInt32 = 34,
   kNumberTypeUInt8 = 37,
   kNumberTypeFloat32 = 43,
+  kNumberTypeEnd = 52,
 };
 }  // namespace mindspore
 #endif  // TESTS_LITE_STUB_INCLUDE_API_DATA_TYPE_H_

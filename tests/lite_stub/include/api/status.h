@@ -4,7 +4,19 @@
 #define TESTS_LITE_STUB_INCLUDE_API_STATUS_H_
 #include <stdint.h>
 
+#include <functional>
+#include <string>
+#include <vector>
+
+#ifndef MS_API
+#define MS_API
+#endif
+
 namespace mindspore {
+// the string <-> char-vector helpers of include/api/dual_abi_helper.h that the registration headers use
+inline std::vector<char> StringToChar(const std::string &s) { return std::vector<char>(s.begin(), s.end()); }
+inline std::string CharToString(const std::vector<char> &c) { return std::string(c.begin(), c.end()); }
+
 enum CompCode : uint32_t { kCore = 0x00000000u, kLite = 0xF0000000u };
 enum StatusCode : uint32_t {
   kSuccess = 0,

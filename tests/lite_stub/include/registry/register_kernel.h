@@ -1,6 +1,14 @@
 // TEST INFRASTRUCTURE.  Stand-in for mindspore/lite/include/registry/register_kernel.h (:34-102): the same
 // registration call, kept in a process-wide table that the harness queries the way the scheduler does
 // (exact match on arch, provider, data type and op type; scheduler.cc:1131-1177).
+//
+// Where the reference tree is at hand the harness is built with the reference's OWN registry instead: its header
+// (named by PH_REAL_REGISTRY_HEADER on the compiler's command line) and its sources register_kernel.cc /
+// register_kernel_impl.cc, compiled from where they lie (tests/lite_stub/build.py).  The table below is then unused.
+#ifdef PH_REAL_REGISTRY_HEADER
+#include PH_REAL_REGISTRY_HEADER
+#endif
+#ifndef PH_REAL_REGISTRY_HEADER
 #ifndef TESTS_LITE_STUB_INCLUDE_REGISTRY_REGISTER_KERNEL_H_
 #define TESTS_LITE_STUB_INCLUDE_REGISTRY_REGISTER_KERNEL_H_
 #include <functional>
@@ -49,3 +57,4 @@ class RegisterKernel {
 }  // namespace registry
 }  // namespace mindspore
 #endif  // TESTS_LITE_STUB_INCLUDE_REGISTRY_REGISTER_KERNEL_H_
+#endif  // PH_REAL_REGISTRY_HEADER

@@ -8,6 +8,7 @@
 
 #include <stdint.h>
 
+#include <string>
 #include <vector>
 
 namespace flatbuffers {
@@ -34,6 +35,9 @@ enum PrimitiveType : int {
   PrimitiveType_MatMulFusion = 89,
   PrimitiveType_Custom = 191,
   PrimitiveType_DynamicQuant = 203,
+  PrimitiveType_FillV2 = 221,  // the union's last member
+  PrimitiveType_MIN = PrimitiveType_NONE,
+  PrimitiveType_MAX = PrimitiveType_FillV2,
 };
 enum QuantType : int {  // model.fbs:76-84
   QuantType_QUANT_NONE = 0,
@@ -93,13 +97,25 @@ struct DynamicQuant {  // ops.fbs:1248-1255
   const flatbuffers::Vector<int32_t> *prefer_axes() const { return has_prefer_axes_ ? &prefer_axes_ : nullptr; }
 };
 
+struct String {  // flatbuffers::String, as far as the kernel registry reads it
+  std::string s_;
+  std::string str() const { return s_; }
+};
+
+struct Custom {  // ops.fbs: table Custom { type: string; attr: [Attribute]; }
+  String type_;
+  const String *type() const { return &type_; }
+};
+
 struct Primitive {  // model.fbs:86-88 (a union in the real schema: exactly one member is meaningful)
   PrimitiveType type_ = PrimitiveType_NONE;
   MatMulFusion matmul_;
   FullConnection fc_;
   Conv2DFusion conv_;
   DynamicQuant dynquant_;
+  Custom custom_;
   PrimitiveType value_type() const { return type_; }
+  const Custom *value_as_Custom() const { return type_ == PrimitiveType_Custom ? &custom_ : nullptr; }
   const MatMulFusion *value_as_MatMulFusion() const { return type_ == PrimitiveType_MatMulFusion ? &matmul_ : nullptr; }
   const FullConnection *value_as_FullConnection() const {
     return type_ == PrimitiveType_FullConnection ? &fc_ : nullptr;

@@ -66,6 +66,8 @@ def _load_harness():
     h.ph_register_test_interface.argtypes = [C.c_char_p, C.c_int32]
     h.ph_register_test_interface.restype = None
     h.ph_execute_concurrently.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32]
+    h.ph_lookup.argtypes = [C.c_char_p, C.c_char_p, C.c_int32, C.c_int32]
+    h.ph_register_declining.argtypes = [C.c_char_p, C.c_char_p, C.c_int32, C.c_int32]
     return h
 
 
@@ -232,6 +234,44 @@ def test_a_declined_node_can_still_fall_back(H):
             % os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
     out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert "stage %d" % DECLINED_NO_FALLBACK in out.stdout, (out.stdout, out.stderr[-2000:])
+
+
+def test_lookup_rules_of_the_kernel_registry(H):
+    """The provider's registrations as the registry answers for them -- the reference's own RegisterKernel /
+    RegistryKernelImpl (src/registry/register_kernel_impl.cc) when the harness was built with the reference tree at
+    hand, the stand-in table otherwise: exact match on provider and arch (so the stock benchmark tool, which leaves
+    the arch empty, needs the second registration), the data type of input 0 as part of the key, and at most ten
+    providers per process."""
+    real = bool(H.ph_registry_is_real())
+    assert real == stub_build.real_registry_available() or not os.path.isdir(stub_build.REFERENCE)
+    for arch in (b"CPU", b""):
+        for dtype, ops in ((I8, (MATMUL, FC, CONV)), (F32, (DYNQUANT,))):
+            for o in ops:
+                assert H.ph_lookup(arch, b"mi355x", dtype, o) == 1, (arch, dtype, o)
+    assert H.ph_lookup(b"GPU", b"mi355x", I8, MATMUL) == 0          # another arch
+    assert H.ph_lookup(b"CPU", b"mi355", I8, MATMUL) == 0           # another provider name
+    assert H.ph_lookup(b"CPU", b"", I8, MATMUL) == 0                # no provider: builtin kernels only
+    assert H.ph_lookup(b"CPU", b"mi355x", F32, MATMUL) == 0         # fp32 MatMul is not this provider's
+    assert H.ph_lookup(b"CPU", b"mi355x", I8, DYNQUANT) == 0        # DynamicQuant is keyed by its fp32 input
+    assert H.ph_lookup(b"CPU", b"mi355x", I8, 36) == 0              # an operator type nobody registered
+    if not real:
+        return
+    # register_kernel_impl.cc:32-36,105-117: op types outside (MIN, MAX] and data types outside the number range are
+    # refused; an eleventh provider is refused (kMaxProviderNum = 10)
+    assert H.ph_register_declining(b"CPU", b"probe0", I8, 0) != 0
+    assert H.ph_register_declining(b"CPU", b"probe0", I8, 222) != 0
+    assert H.ph_register_declining(b"CPU", b"probe0", 52, MATMUL) != 0
+    assert H.ph_lookup(b"CPU", b"probe0", I8, MATMUL) == 0
+    for i in range(9):  # mi355x is the first provider of the process
+        assert H.ph_register_declining(b"CPU", b"probe%d" % i, I8, MATMUL) == 0, i
+        assert H.ph_lookup(b"CPU", b"probe%d" % i, I8, MATMUL) == 1
+    assert H.ph_register_declining(b"CPU", b"probe9", I8, MATMUL) != 0
+    assert H.ph_lookup(b"CPU", b"probe9", I8, MATMUL) == 0
+    assert H.ph_lookup(b"CPU", b"mi355x", I8, MATMUL) == 1          # the earlier registrations are untouched
+    # a provider's eleventh arch is refused as well (kMaxArchPerProviderNum = 10); mi355x holds "CPU" and ""
+    for i in range(8):
+        assert H.ph_register_declining(b"arch%d" % i, b"mi355x", I8, 36) == 0, i
+    assert H.ph_register_declining(b"arch8", b"mi355x", I8, 36) != 0
 
 
 def test_registration_keys_and_decline_without_a_gpu(H):
