@@ -218,6 +218,40 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+def bench_tile_fixed_cost(size=8192, ks=(1024, 4096, 8192), steps=20):
+    """What a 256 x 256 tile costs beyond its K loop when a CU runs several tiles one after the other (1024 tiles on
+    256 CUs at 8192 x 8192): the launch time at three K, a line through them, and its intercept divided by the tiles
+    per CU.  That intercept is dispatch + parameter fetch + first operand fetch + epilogue of one tile; a persistent
+    kernel that prefetches the next tile under the epilogue can at most save the part of it that is not epilogue."""
+    import numpy as np
+    import torch
+    from mindspore_amd import kernels as K
+    rng = np.random.default_rng(5)
+    a_full = torch.from_numpy(rng.integers(-128, 128, (size, max(ks)), dtype=np.int8)).cuda()
+    out = torch.empty((size, size), dtype=torch.int8, device="cuda")
+    sw = rng.uniform(1e-4, 1e-2, size).astype(np.float32)
+    times = {}
+    for k in ks:
+        w = rng.integers(-128, 128, (size, k), dtype=np.int8)
+        so = float(np.float32(0.02 * float(np.mean(sw)) * np.sqrt(k) * 150.0))
+        kern = K.MatmulInt8Kernel(w, None, K.QuantParam(0.02, 7), [K.QuantParam(float(s), 0) for s in sw],
+                                  K.QuantParam(so, 0), True, 0, decode_pack=False)
+        a = a_full[:, :k].contiguous()
+        for _ in range(60):  # ~20 ms: the settled state
+            kern.run(a, out=out)
+        ms, _ = time_steps(lambda: kern.run(a, out=out), steps, 2)
+        times[k] = ms * 1e3
+        kern.close()
+    xs, ys = np.array(sorted(times)), np.array([times[k] for k in sorted(times)])
+    slope, intercept = np.polyfit(xs, ys, 1)
+    tiles_per_cu = (size // 256) ** 2 / 256.0
+    return dict(us_by_k={int(k): float(v) for k, v in times.items()}, us_per_128_bytes_of_k=float(slope * 128),
+                fixed_us_per_launch=float(intercept), tiles_per_cu=tiles_per_cu,
+                fixed_us_per_tile=float(intercept / tiles_per_cu),
+                note="launch time = fixed + K x slope; fixed / tiles per CU is what one tile costs outside its K loop "
+                     "(of which the epilogue is 5.3-5.7 us)")
+
+
 def bench_hbm_read(steps, warmup):
     """What a kernel that only reads can reach on this device: the library's plain read stream over 48 MiB slices
     (the size of one decode weight matrix) of a 3 GiB buffer, so no slice is still in the 256 MB Infinity Cache when
@@ -570,6 +604,10 @@ def main():
         o = section("gemm%d" % other, lambda: bench_gemm(other, max(3, args.steps // 5), 2))
         if o:
             extra["gemm%d" % other] = dict(ms=o["ms"], tops=o["tops"], frac_of_int8_peak=o["tops"] / PEAK_INT8_TOPS)
+        if size == 4096:
+            fx = section("gemm8192_fixed_cost_per_tile", bench_tile_fixed_cost)
+            if fx:
+                extra["gemm8192_fixed_cost_per_tile"] = fx
         mf = section("mfma_only", bench_mfma_rate)
         if mf:
             extra["mfma_only"] = mf

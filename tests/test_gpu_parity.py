@@ -106,6 +106,24 @@ def test_matmul_whole_cu_tile_ragged(orc, m, n, k):
         assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("m,n,k", [(4352, 4096, 256), (4096, 4352, 384), (8448, 2304, 128 * 5), (2304, 8448, 256),
+                                   (16640, 1024, 256), (4352, 4096, 2048)])
+def test_matmul_more_full_tiles_than_cus(orc, m, n, k):
+    """More full 256 x 256 tiles than CUs (272 to 297 of them: some CUs run a second tile), K a whole number of
+    128-byte blocks (2, 3, 5 and 16 per tile).  Per-tensor / per-channel, zero and non-zero weight zero points, the
+    generic rounding path."""
+    rng = np.random.default_rng(m + 3 * n + k)
+    orc.set_threads(16)
+    for it in range(4):
+        case = _mm_case(rng, m, n, k, bool(it & 1), bool(it & 2), it != 2, [0, 1, 3, 0][it], it != 3,
+                        1e-3 if it == 3 else 100.0)
+        if it == 3:
+            case["bias"] = rng.integers(-2 ** 31, 2 ** 31 - 1, n).astype(np.int32)
+        got, _ = _gpu_matmul(case, device_tensors=True)
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (m, n, k, it, int((got != want).sum()))
+
+
 @pytest.mark.parametrize("m,n,k", [(1408, 1408, 144), (1500, 1420, 144), (1536, 1536, 112), (1300, 1700, 400),
                                    (2050, 1030, 1168), (700, 5000, 128), (1664, 1280, 256)])
 def test_matmul_128_tile_k_block_loop(orc, m, n, k):
