@@ -422,7 +422,7 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
   // one row: the dot kernel on the row-major weights; 2..32 rows: the matrix-core decode kernel on the blocked copy
   // made at create time -- a handle without it runs two rows on the dot kernel and 3..32 on the GEMM tiles
   const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
-                                           : rows <= kGemvMaxRows && st.w_blocked.p != nullptr;
+                                           : rows <= kGemvMaxRows && st.w_blocked.p != nullptr && st.k_pad <= 1 << 20;
   if (skinny) {
     if (rows >= 2) w.blocked = static_cast<const int8_t *>(st.w_blocked.p);  // (may be absent: two rows then take the v_dot4 kernel)
     return launch_gemv_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
@@ -816,7 +816,8 @@ int mi_matmul_run_group(mi_matmul *const *handles, int32_t count, const int8_t *
   // decode-sized runs of up to four members go out as one launch; anything else runs member by member
   bool one_launch = count >= 2 && count <= 4 && rows <= kGemvMaxRows;
   for (int i = 0; i < count && one_launch; ++i)
-    one_launch = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024 : handles[i]->st.w_blocked.p != nullptr;
+    one_launch = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
+                                      : handles[i]->st.w_blocked.p != nullptr && handles[i]->st.k_pad <= 1 << 20;
   if (one_launch) {
     WeightView wv[4];
     RequantParams rq[4];

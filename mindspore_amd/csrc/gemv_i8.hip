@@ -1,18 +1,21 @@
 // Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 32 activation rows
-// against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw): a v_dot4 kernel for M <= 2, a
-// matrix-core kernel for 3 <= M <= 32.  The kernels are HBM-bound on the weight stream, so the design goal
-// is "every weight byte crosses HBM once, in 1 KiB coalesced wave loads, with enough loads in flight":
-//   - a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes);
-//   - it keeps D 16-byte loads per lane (D KiB per wave) in flight at all times, refilling a register slot as soon
-//     as its chunk has been consumed;
-//   - the M activation rows are staged once per workgroup in LDS and re-read as 16-byte fragments;
-//   - products use v_dot4_i32_i8; the K reduction across lanes happens once at the end.
+// against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw): a v_dot4 kernel for one row (and
+// for two on a handle without the blocked weight copy), matrix-core kernels on the blocked copy for 2 <= M <= 32.
+// The kernels are HBM-bound on the weight stream, so the design goal is "every weight byte crosses HBM once, in 1 KiB
+// coalesced wave loads, with enough loads in flight":
+//   - v_dot4 kernel: a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes),
+//     with its whole share in flight where that fits (D 16-byte loads per lane); the K reduction across lanes happens
+//     once at the end;
+//   - matrix-core kernels: a workgroup of eight waves owns RG x 16 channels, the waves split K, the weights are the
+//     16-row operand of v_mfma_i32_16x16x64_i8 and are read from 1 KiB blocks laid out in lane order; the activation
+//     rows go through LDS (up to 16 rows) or straight into fragments (17..32 rows).
 // Arithmetic reference: MatmulInt8Opt, mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/matmul_int8.c:296-331.
 #include "common.h"
 #include "quant_math.h"
 
 #include <algorithm>
 #include <type_traits>
+
 
 namespace mi {
 
@@ -346,8 +349,9 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 }
 
 // =====================================================================================================================
-// 3 <= M <= 32 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M
-// (MG = 1 up to 16 rows, MG = 2 row groups of 16 above).
+// 2 <= M <= 32 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
+// This form (activation fragments fetched straight from global memory) serves 17..32 rows (MG = 2 row groups of 16);
+// up to 16 rows take the LDS-staged form further down.
 // v_mfma_i32_16x16x64_i8 with the WEIGHTS as the 16-row operand: lane (g = lane / 16, i = lane % 16) supplies 16
 // contiguous K bytes of weight row i (K offset 16 g inside the 64-byte step) and the same 16 K bytes of activation row
 // i (zero for i >= M); the result register r of that lane is output (channel 4 g + r, activation row i).
@@ -541,6 +545,233 @@ static int launch_mfma(const GemvArgs &g, int m, const RequantParams &rq, hipStr
   return MI_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// 2 to 16 activation rows (one group of 16 for the matrix cores) with the activations staged through LDS.
+// In the form above a wave's activation fetch asks, per instruction, for 64 bytes of each of up to 16 rows: four lanes
+// per row, so every group of four neighbouring lanes touches four different cache lines, and the address unit looks a
+// line up per lane group rather than per instruction.  Here a wave fetches its K slice of the rows with lanes along K
+// (the MR x D x 64 bytes of a pass as MR runs of whole cache lines), writes them to a private LDS area one row after
+// the other (row stride D x 64 + 16 bytes, so that the 16 rows of a fragment read fall on different banks) and reads
+// the matrix-core fragments back from there.  Row MR of the area stays zero: lanes whose row does not exist read it.
+// The area is private to the wave (LDS operations of one wave execute in order), so staging needs no barrier.
+// Both operands are fetched through buffer descriptors, so a fetch that has nothing to fetch returns zeros without a
+// memory access and without a mask on the data.
+// The waves' partial sums meet in LDS accumulators (atomic adds), and after one barrier every wave finishes one
+// (row group, result register) pair, one output per lane: the barrier and what follows it is what a launch with one
+// workgroup per CU cannot overlap with anything, so it is kept short (measured on the decode matrices at 8 rows:
+// 0.1-0.3 us per launch against eight partial reads per output by the first waves only).
+// RG row groups per workgroup: activation bytes per weight byte are M / (16 RG); three where there are channels
+// enough (a 12288 x 4096 matrix is then 256 workgroups, one per CU, all resident at once), D weight steps in flight
+// per wave and row group.  MR = the number of rows rounded up to 2, 4, 8 or 16 (the number of fetch instructions is a
+// compile-time constant).
+// ---------------------------------------------------------------------------------------------------------------------
+template <int WAVES, int RG, int D, int MR>
+__device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
+  constexpr int ROWB = D * 64;                       // activation bytes per row and pass
+  constexpr int STRIDE = ROWB + 16;                  // LDS row stride
+  constexpr int LPR = ROWB / 16;                     // 16-byte chunks of one row in a pass
+  constexpr int NLD = (MR * LPR + 63) / 64;          // fetch instructions per pass
+  constexpr int AREA = (MR + 1) * STRIDE;            // per wave
+  __shared__ int sums[(4 * RG + 1) * 64];
+  __shared__ __attribute__((aligned(16))) char lds[WAVES * AREA];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane >> 4, idx = lane & 15;
+  const int n0 = block * (RG * 16);
+  const int k_bytes = g.kchunks * 16;
+  const int total = g.k_pad >> 6;  // 64-byte steps in a (zero padded) weight row
+  const int spw = (total + WAVES - 1) / WAVES;
+  const int s0 = wave * spw;
+  char *area = lds + wave * AREA;
+  const int n_pad = (g.n + 255) & ~255;            // rows of the packed weights and of the parameter arrays
+  const int rg_live = (n_pad - n0) >> 4;           // row groups of this workgroup that exist (RG need not divide 16)
+
+  // Both operands come through buffer descriptors: a load whose lane offset is kOutOfRange returns zero without touching
+  // memory, so loads that have nothing to fetch (a step past the wave's slice or past the row, a row group or an
+  // activation row that does not exist, bytes past K) need neither a substitute address nor a mask on the data, and a
+  // load's address is one lane offset plus a scalar.
+  constexpr int kOutOfRange = (int)0x80000000u;
+  const int sw0 = __builtin_amdgcn_readfirstlane(s0);
+  const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<int8_t *>(g.w) + (int64_t)(n0 >> 4) * total * 1024, (short)0,
+      (rg_live < RG ? rg_live : RG) * total * 1024, 0x00020000);
+  const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<int8_t *>(g.a), (short)0, (int)((m_rows - 1) * g.lda) + k_bytes, 0x00020000);
+  // fetch geometry: the MR x LPR chunks of a pass in row-major order, 64 per instruction
+  int a_off[NLD], a_chunk[NLD], a_dst[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) {
+    const int c = i * 64 + lane, row = c / LPR, chunk = c % LPR;
+    a_chunk[i] = chunk;
+    a_off[i] = row < m_rows ? row * (int)g.lda + chunk * 16 : kOutOfRange;
+    a_dst[i] = row < MR ? row * STRIDE + chunk * 16 : -1;
+  }
+  auto load_a = [&](int base, int i) -> v4i {
+    const int step = base + (a_chunk[i] >> 2);
+    const int kb = (sw0 + base) * 64;
+    const bool any = base < spw && sw0 + base < total && kb < k_bytes;  // (wave-uniform)
+    const bool live = step < spw && sw0 + step < total && kb + a_chunk[i] * 16 < k_bytes;
+    return __builtin_bit_cast(
+        v4i, __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, live ? a_off[i] : kOutOfRange, any ? kb : 0, 0));
+  };
+  auto store_a = [&](int base, int i, v4i v) {
+    if (a_dst[i] >= 0) *reinterpret_cast<v4i *>(area + a_dst[i]) = v;
+  };
+  auto load_w = [&](int j, int rg) -> v4i {
+    const int s = sw0 + j;
+    const bool live = j < spw && s < total && rg < rg_live;  // (wave-uniform)
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, live ? lane * 16 : kOutOfRange,
+                                                                         live ? (rg * total + s) * 1024 : 0, 2));
+  };
+
+  // activations first: they return first, and the rows can be in LDS while the weights are still on their way
+  v4i abuf[NLD];
+#pragma unroll
+  for (int i = 0; i < NLD; ++i) abuf[i] = load_a(0, i);
+  v4i wbuf[D][RG];
+#pragma unroll
+  for (int j = 0; j < D; ++j)
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(j, rg);
+  for (int c = lane; c < STRIDE / 16; c += 64) *reinterpret_cast<v4i *>(area + MR * STRIDE + c * 16) = v4i{0, 0, 0, 0};
+  for (int c = tid; c < (4 * RG + 1) * 64; c += WAVES * 64) sums[c] = 0;
+  __syncthreads();  // (every wave gets here right after it has issued its loads)
+
+  // after the reduction, (row group, result register) pair q = wave + 8 t is finished by this wave: one output per
+  // lane and pair
+  constexpr int NQ = (4 * RG + WAVES - 1) / WAVES;
+  int32_t p_mult[NQ], p_e[NQ], p_ls[NQ], p_bias2[NQ], p_zw[NQ];
+#pragma unroll
+  for (int t = 0; t < NQ; ++t) {
+    const int q = wave + WAVES * t;
+    const int n = q < 4 * RG && (q >> 2) < rg_live ? n0 + (q >> 2) * 16 + 4 * grp + (q & 3) : n0;
+    p_mult[t] = rq.mult[n];
+    p_e[t] = rq.rshift[n];
+    p_ls[t] = rq.lshift[n];
+    p_bias2[t] = rq.bias2[n];
+    p_zw[t] = rq.zw[n];
+  }
+
+  v4i acc[RG], asum = {0, 0, 0, 0};
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg) acc[rg] = v4i{0, 0, 0, 0};
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  const char *frag = area + (idx < m_rows ? idx : MR) * STRIDE + grp * 16;
+
+  auto pass = [&](int base, auto refill) {
+#pragma unroll
+    for (int i = 0; i < NLD; ++i) store_a(base, i, abuf[i]);
+    if (decltype(refill)::value) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) abuf[i] = load_a(base + D, i);
+    }
+#pragma unroll
+    for (int j = 0; j < D; ++j) {
+      const v4i x = *reinterpret_cast<const v4i *>(frag + j * 64);
+      v4i w[RG];
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];
+      if (decltype(refill)::value) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(base + D + j, rg);
+      }
+#pragma unroll
+      for (int rg = 0; rg < RG; ++rg) acc[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x, acc[rg], 0, 0, 0);
+      if (rq.has_zw) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x, asum, 0, 0, 0);
+    }
+  };
+  int base = 0;
+  for (; base + D < spw; base += D) pass(base, std::true_type());
+  pass(base, std::false_type());
+
+  // the partial sums meet in LDS accumulators (LDS atomic adds without a return value; the accumulators were zeroed
+  // before the first barrier): register r of row group rg at sums[(4 rg + r) * 64 + lane], the row sum behind them
+#pragma unroll
+  for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      __hip_atomic_fetch_add(&sums[(4 * rg + r) * 64 + lane], acc[rg][r], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_WORKGROUP);
+  if (rq.has_zw)
+    __hip_atomic_fetch_add(&sums[4 * RG * 64 + lane], asum[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < NQ; ++t) {
+    const int q = wave + WAVES * t;
+    const int f_rg = q >> 2, f_r = q & 3;
+    const int f_n = n0 + f_rg * 16 + 4 * grp + f_r;
+    if (q < 4 * RG && idx < m_rows && f_n < g.n) {
+      uint32_t v = (uint32_t)sums[q * 64 + lane];
+      if (rq.has_zw) v -= (uint32_t)sums[4 * RG * 64 + lane] * (uint32_t)p_zw[t];
+      v += (uint32_t)p_bias2[t];
+      int32_t y;
+      if (rq.fast) {
+        y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[t]), p_e[t], (1 << p_e[t]) >> 1);
+      } else {
+        y = rdiv_pot(srdhm((int32_t)(v << p_ls[t]), p_mult[t]), p_e[t]);
+      }
+      y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+      y = y < rq.amax ? y : rq.amax;
+      y = y > rq.amin ? y : rq.amin;
+      g.c[(int64_t)idx * g.ldc + f_n] = (int8_t)y;
+    }
+  }
+}
+
+template <int WAVES, int RG, int D, int MR>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_kernel(GemvArgs g, int m_rows, RequantParams rq) {
+  gemv_mfma_lds_body<WAVES, RG, D, MR>(g, m_rows, rq, (int)blockIdx.x);
+}
+
+template <int WAVES, int RG, int D, int MR>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_group_kernel(GemvGroup grp, int m_rows) {
+  GemvArgs g;
+  RequantParams rq;
+  int block;
+  pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
+  gemv_mfma_lds_body<WAVES, RG, D, MR>(g, m_rows, rq, block);
+}
+
+template <int WAVES, int D, typename F>
+static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8 or 16
+  using std::integral_constant;
+  if (m <= 2) return f(integral_constant<int, 2>());
+  if (m <= 4) return f(integral_constant<int, 4>());
+  if (m <= 8) return f(integral_constant<int, 8>());
+  if constexpr (WAVES * 17 * (D * 64 + 16) <= 160 * 1024) {
+    return f(integral_constant<int, 16>());
+  } else {
+    set_error("gemv: %d rows do not fit the staging area of this configuration", m);
+    return MI_PARAM_INVALID;
+  }
+}
+
+template <int WAVES, int RG, int D>
+static int launch_group_mfma_lds(GemvGroup &grp, int m, hipStream_t stream) {
+  int blocks = 0;
+  for (int i = 0; i < grp.count; ++i) {
+    blocks += (grp.g[i].n + RG * 16 - 1) / (RG * 16);
+    grp.block_end[i] = blocks;
+  }
+  return with_row_class<WAVES, D>(m, [&](auto mr) {
+    hipLaunchKernelGGL((gemv_mfma_lds_group_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks), dim3(WAVES * 64),
+                       0, stream, grp, m);
+    MI_HIP_CHECK(hipGetLastError());
+    return (int)MI_OK;
+  });
+}
+
+template <int WAVES, int RG, int D>
+static int launch_mfma_lds(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  return with_row_class<WAVES, D>(m, [&](auto mr) {
+    hipLaunchKernelGGL((gemv_mfma_lds_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks), dim3(WAVES * 64), 0,
+                       stream, g, m, rq);
+    MI_HIP_CHECK(hipGetLastError());
+    return (int)MI_OK;
+  });
+}
+
+
 __global__ __launch_bounds__(256) void block_weights_kernel(const int8_t *__restrict__ w, int ldw, int kblocks,
                                                             int64_t chunks, int8_t *__restrict__ blocked) {
   // one 16-byte chunk per thread; destination order, so the stores coalesce
@@ -576,6 +807,7 @@ static int check_gemv_operands(const int8_t *a, int64_t lda, int m, int k, const
   if (m < 1 || m > kGemvMaxRows || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
       wv.k_pad % kKPad != 0 || wv.k_pad < k || wv.ldw < wv.k_pad || (wv.ldw & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
+      (int64_t)(m - 1) * lda + k >= (int64_t)1 << 30 || wv.k_pad > 1 << 20 ||  // (32-bit buffer offsets)
       (m <= kGemvDotRows && (int64_t)m * round_up(k, 1024) > 160 * 1024 - 1024)) {
     set_error("gemv: unsupported operand geometry m=%d n=%d k=%d lda=%lld", m, n, k, (long long)lda);
     return MI_PARAM_INVALID;
@@ -610,7 +842,7 @@ int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, con
     for (int i = 0; i < count; ++i) grp.g[i].w = wv[i].blocked;
     const bool wide = n_max >= 8192 && k_pad_max <= 4096;
     if (m > 16) return wide ? launch_group_mfma<2, 4, 2>(grp, m, stream) : launch_group_mfma<1, 8, 2>(grp, m, stream);
-    return wide ? launch_group_mfma<2, 4>(grp, m, stream) : launch_group_mfma<1, 8>(grp, m, stream);
+    return wide ? launch_group_mfma_lds<8, 2, 4>(grp, m, stream) : launch_group_mfma_lds<8, 1, 8>(grp, m, stream);
   }
   return m == 1 ? launch_group_m<1>(grp, stream) : launch_group_m<2>(grp, stream);
 }
@@ -630,8 +862,8 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
       if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4, 2>(g, m, rq, stream);
       return launch_mfma<1, 8, 2>(g, m, rq, stream);
     }
-    if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4>(g, m, rq, stream);
-    return launch_mfma<1, 8>(g, m, rq, stream);
+    if (n >= 8192 && k_pad <= 4096) return launch_mfma_lds<8, 3, 4>(g, m, rq, stream);
+    return launch_mfma_lds<8, 1, 8>(g, m, rq, stream);
   }
   return m == 1 ? launch_m<1>(g, rq, stream) : launch_m<2>(g, rq, stream);
 }

@@ -69,13 +69,15 @@ def test_matmul_shapes(orc, m, n, k):
 
 @pytest.mark.parametrize("n,k", [(40, 2048), (24, 4000), (16, 5008), (9, 13008), (8200, 1040), (8196, 208),
                                  (21, 2800), (18, 6144), (13, 7008), (11, 8192), (7, 9232), (10, 10240), (6, 11008),
-                                 (5, 12288)])
+                                 (5, 12288), (11008, 528), (8250, 80)])
 def test_decode_rows_every_stream_shape(orc, n, k):
     """1..32 activation rows (v_dot4 kernel for one row, and for two on a handle without the blocked copy; matrix-core
     kernel otherwise: one group of 16 rows up to 16, two
     groups up to 32) and the first row counts of the GEMM path, against every weight-stream shape the
     skinny path distinguishes: rows of one to six 1 KiB segments (whole rows per wave), seven to twelve (two waves
-    per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels."""
+    per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels
+    (from 8192 channels on a workgroup of the matrix-core kernel owns three groups of 16 channels: 11008 channels end
+    in a workgroup with one live group, 8250 in one whose live group is ragged)."""
     rng = np.random.default_rng(n * 131 + k)
     orc.set_threads(16)
     for m in list(range(1, 19)) + [23, 31, 32, 33, 40]:
