@@ -350,221 +350,37 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 
 // =====================================================================================================================
 // 2 <= M <= 32 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
-// This form (activation fragments fetched straight from global memory) serves 17..32 rows (MG = 2 row groups of 16);
-// up to 16 rows take the LDS-staged form further down.
 // v_mfma_i32_16x16x64_i8 with the WEIGHTS as the 16-row operand: lane (g = lane / 16, i = lane % 16) supplies 16
 // contiguous K bytes of weight row i (K offset 16 g inside the 64-byte step) and the same 16 K bytes of activation row
-// i (zero for i >= M); the result register r of that lane is output (channel 4 g + r, activation row i).
+// i (zero for i >= M; rows 16..31 are a second fragment against the same weight fragment); the result register r of
+// that lane is output (channel 4 g + r, activation row i).
 // The weights come from the blocked copy: 1 KiB blocks [row / 16][k / 64], inside a block the 16-byte chunks in lane
 // order ([(k % 64) / 16][row % 16]), so a wave instruction fetches 64 consecutive chunks -- eight whole cache lines --
 // and a wave's consecutive steps walk consecutive KiB.  (With the chunks in row order the same KiB cost four times
 // the cache-line lookups, and the decode matrices ran 10-20 % slower.)
 // A workgroup of 8 waves owns RG x 16 channels; the waves split K into contiguous slices, each wave keeps D steps
-// (D x RG KiB of weights) in flight, and the partial sums meet in LDS.
-// =====================================================================================================================
-template <int RG, int D, int MG>
-__device__ __forceinline__ void gemv_mfma_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
-  constexpr int WAVES = 8;
-  __shared__ v4i red[WAVES][(RG + 1) * MG][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int grp = lane >> 4, idx = lane & 15;
-  const int n0 = block * (RG * 16);
-  const int k_bytes = g.kchunks * 16;
-  const int total = g.k_pad >> 6;  // 64-byte steps in a (zero padded) weight row
-  const int spw = (total + WAVES - 1) / WAVES;
-  const int s0 = wave * spw;
-  // blocked weights: 1 KiB block (row group, step) = 16 rows x 64 bytes, chunk of lane (grp, idx) = row idx, K chunk
-  // grp at position lane
-  const int8_t *wbase = g.w + (int64_t)(n0 >> 4) * total * 1024 + lane * 16;
-  // activation rows of this lane: idx + 16 * mg (a row past the last one re-reads the last and is zeroed)
-  const int8_t *abase[MG];
-#pragma unroll
-  for (int mg = 0; mg < MG; ++mg) {
-    const int row = idx + 16 * mg;
-    abase[mg] = g.a + (int64_t)(row < m_rows ? row : m_rows - 1) * g.lda;
-  }
-
-  // the finishing lanes (first RG waves) fetch their channels' parameters while the weights stream
-  int32_t p_mult[4], p_e[4], p_ls[4], p_bias2[4], p_zw[4];
-  if (wave < RG) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int n = n0 + wave * 16 + 4 * grp + r;
-      p_mult[r] = rq.mult[n];
-      p_e[r] = rq.rshift[n];
-      p_ls[r] = rq.lshift[n];
-      p_bias2[r] = rq.bias2[n];
-      p_zw[r] = rq.zw[n];
-    }
-  }
-
-  // (a step past this wave's slice or past the row asks for the first 16 bytes of an activation row, which are in
-  //  the nearest cache, instead of weight bytes that another wave streams or that do not exist)
-  auto load_w = [&](int j, int rg) -> v4i {
-    const int s = s0 + j;
-    const bool live = j < spw && s < total;
-    const int8_t *p = live ? wbase + ((int64_t)rg * total + s) * 1024 : abase[0];
-    return __builtin_nontemporal_load(reinterpret_cast<const v4i *>(p));
-  };
-  auto load_x = [&](int j, int mg) -> v4i {
-    int off = (s0 + j) * 64 + grp * 16;
-    off = off < k_bytes ? off : k_bytes - 16;
-    return *reinterpret_cast<const v4i *>(abase[mg] + off);
-  };
-  v4i wbuf[D][RG], xbuf[D][MG];
-#pragma unroll
-  for (int j = 0; j < D; ++j) {
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(j, rg);
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) xbuf[j][mg] = load_x(j, mg);
-  }
-
-  v4i acc[RG][MG], asum[MG];
-#pragma unroll
-  for (int mg = 0; mg < MG; ++mg) {
-    asum[mg] = v4i{0, 0, 0, 0};
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg) acc[rg][mg] = v4i{0, 0, 0, 0};
-  }
-  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-
-  auto pass = [&](int base, auto refill) {
-#pragma unroll
-    for (int j = 0; j < D; ++j) {
-      const int jj = base + j;
-      const bool in_k = jj < spw && s0 + jj < total && (s0 + jj) * 64 + grp * 16 < k_bytes;
-      v4i x[MG];
-#pragma unroll
-      for (int mg = 0; mg < MG; ++mg) {
-        const bool live = in_k && idx + 16 * mg < m_rows;
-        x[mg] = xbuf[j][mg];
-        x[mg].x = live ? x[mg].x : 0;
-        x[mg].y = live ? x[mg].y : 0;
-        x[mg].z = live ? x[mg].z : 0;
-        x[mg].w = live ? x[mg].w : 0;
-      }
-      v4i w[RG];
-#pragma unroll
-      for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];
-      if (decltype(refill)::value) {
-#pragma unroll
-        for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(jj + D, rg);
-#pragma unroll
-        for (int mg = 0; mg < MG; ++mg) xbuf[j][mg] = load_x(jj + D, mg);
-      }
-#pragma unroll
-      for (int mg = 0; mg < MG; ++mg) {
-#pragma unroll
-        for (int rg = 0; rg < RG; ++rg)
-          acc[rg][mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x[mg], acc[rg][mg], 0, 0, 0);
-        if (rq.has_zw) asum[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x[mg], asum[mg], 0, 0, 0);
-      }
-    }
-  };
-  int base = 0;
-  for (; base + D < spw; base += D) pass(base, std::true_type());
-  pass(base, std::false_type());
-
-#pragma unroll
-  for (int mg = 0; mg < MG; ++mg) {
-#pragma unroll
-    for (int rg = 0; rg < RG; ++rg) red[wave][mg * (RG + 1) + rg][lane] = acc[rg][mg];
-    red[wave][mg * (RG + 1) + RG][lane] = asum[mg];
-  }
-  __syncthreads();
-  if (wave < RG) {
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) {
-      v4i tot = {0, 0, 0, 0}, xs = {0, 0, 0, 0};
-#pragma unroll
-      for (int w = 0; w < WAVES; ++w) {
-        tot += red[w][mg * (RG + 1) + wave][lane];
-        xs += red[w][mg * (RG + 1) + RG][lane];
-      }
-      const int row = idx + 16 * mg;
-      if (row < m_rows) {
-        const int nb = n0 + wave * 16 + 4 * grp;
-        int8_t outv[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          uint32_t v = (uint32_t)tot[r];
-          if (rq.has_zw) v -= (uint32_t)xs[0] * (uint32_t)p_zw[r];
-          v += (uint32_t)p_bias2[r];
-          int32_t y;
-          if (rq.fast) {
-            y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[r]), p_e[r], (1 << p_e[r]) >> 1);
-          } else {
-            y = rdiv_pot(srdhm((int32_t)(v << p_ls[r]), p_mult[r]), p_e[r]);
-          }
-          y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
-          y = y < rq.amax ? y : rq.amax;
-          y = y > rq.amin ? y : rq.amin;
-          outv[r] = (int8_t)y;
-        }
-        int8_t *dst = g.c + (int64_t)row * g.ldc + nb;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (nb + r < g.n) dst[r] = outv[r];
-      }
-    }
-  }
-}
-
-template <int RG, int D, int MG>
-__global__ __launch_bounds__(512) void gemv_mfma_kernel(GemvArgs g, int m_rows, RequantParams rq) {
-  gemv_mfma_body<RG, D, MG>(g, m_rows, rq, (int)blockIdx.x);
-}
-
-template <int RG, int D, int MG>
-__global__ __launch_bounds__(512) void gemv_mfma_group_kernel(GemvGroup grp, int m_rows) {
-  GemvArgs g;
-  RequantParams rq;
-  int block;
-  pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
-  gemv_mfma_body<RG, D, MG>(g, m_rows, rq, block);
-}
-
-template <int RG, int D, int MG = 1>
-static int launch_group_mfma(GemvGroup &grp, int m, hipStream_t stream) {
-  int blocks = 0;
-  for (int i = 0; i < grp.count; ++i) {
-    blocks += (grp.g[i].n + RG * 16 - 1) / (RG * 16);
-    grp.block_end[i] = blocks;
-  }
-  hipLaunchKernelGGL((gemv_mfma_group_kernel<RG, D, MG>), dim3(blocks), dim3(512), 0, stream, grp, m);
-  MI_HIP_CHECK(hipGetLastError());
-  return MI_OK;
-}
-
-template <int RG, int D, int MG = 1>
-static int launch_mfma(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
-  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
-  hipLaunchKernelGGL((gemv_mfma_kernel<RG, D, MG>), dim3(blocks), dim3(512), 0, stream, g, m, rq);
-  MI_HIP_CHECK(hipGetLastError());
-  return MI_OK;
-}
-
-// ---------------------------------------------------------------------------------------------------------------------
-// 2 to 16 activation rows (one group of 16 for the matrix cores) with the activations staged through LDS.
-// In the form above a wave's activation fetch asks, per instruction, for 64 bytes of each of up to 16 rows: four lanes
-// per row, so every group of four neighbouring lanes touches four different cache lines, and the address unit looks a
-// line up per lane group rather than per instruction.  Here a wave fetches its K slice of the rows with lanes along K
-// (the MR x D x 64 bytes of a pass as MR runs of whole cache lines), writes them to a private LDS area one row after
-// the other (row stride D x 64 + 16 bytes, so that the 16 rows of a fragment read fall on different banks) and reads
-// the matrix-core fragments back from there.  Row MR of the area stays zero: lanes whose row does not exist read it.
-// The area is private to the wave (LDS operations of one wave execute in order), so staging needs no barrier.
+// (D x RG KiB of weights) in flight.
+//
+// The activation rows go through LDS.  Fetched straight into fragments, an instruction asks for 64 bytes of each of
+// up to 16 rows: four lanes per row, so every group of four neighbouring lanes touches four different cache lines, and
+// the address unit looks a line up per lane group rather than per instruction.  Instead a wave fetches its K slice of
+// the rows with lanes along K (the MR x D x 64 bytes of a pass as MR runs of whole cache lines), writes them to a
+// private LDS area one row after the other (row stride D x 64 + 16 bytes, so that the 16 rows of a fragment read fall
+// on different banks) and reads the fragments back from there.  Row MR of the area stays zero: lanes whose row does
+// not exist read it.  The area is private to the wave (LDS operations of one wave execute in order), so staging needs
+// no barrier.
 // Both operands are fetched through buffer descriptors, so a fetch that has nothing to fetch returns zeros without a
 // memory access and without a mask on the data.
 // The waves' partial sums meet in LDS accumulators (atomic adds), and after one barrier every wave finishes one
-// (row group, result register) pair, one output per lane: the barrier and what follows it is what a launch with one
-// workgroup per CU cannot overlap with anything, so it is kept short (measured on the decode matrices at 8 rows:
-// 0.1-0.3 us per launch against eight partial reads per output by the first waves only).
-// RG row groups per workgroup: activation bytes per weight byte are M / (16 RG); three where there are channels
-// enough (a 12288 x 4096 matrix is then 256 workgroups, one per CU, all resident at once), D weight steps in flight
-// per wave and row group.  MR = the number of rows rounded up to 2, 4, 8 or 16 (the number of fetch instructions is a
-// compile-time constant).
-// ---------------------------------------------------------------------------------------------------------------------
+// (activation row group, channel group, result register) triple, one output per lane: the barrier and what follows it
+// is what a launch with one workgroup per CU cannot overlap with anything, so it is kept short (measured on the decode
+// matrices at 8 rows: 0.1-0.3 us per launch against eight partial reads per output by the first waves only).
+// RG channel groups per workgroup: activation bytes per weight byte are M / (16 RG); three where there are channels
+// enough (a 12288 x 4096 matrix is then 256 workgroups, one per CU, all resident at once).  MR = the number of rows
+// rounded up to 2, 4, 8, 16 or 32 (the number of fetch instructions is a compile-time constant).
+// Measured over a decoder layer against fragments fetched from global memory, eight partial reads per output and two
+// channel groups: 8 rows 4.57 -> 4.95 TB/s, 16 rows 3.95 -> 4.58, 32 rows 2.67 -> 3.66.
+// =====================================================================================================================
 template <int WAVES, int RG, int D, int MR>
 __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
   constexpr int ROWB = D * 64;                       // activation bytes per row and pass
@@ -572,7 +388,9 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   constexpr int LPR = ROWB / 16;                     // 16-byte chunks of one row in a pass
   constexpr int NLD = (MR * LPR + 63) / 64;          // fetch instructions per pass
   constexpr int AREA = (MR + 1) * STRIDE;            // per wave
-  __shared__ int sums[(4 * RG + 1) * 64];
+  constexpr int MG = MR > 16 ? 2 : 1;                // groups of 16 activation rows
+  constexpr int NSUM = (4 * RG + 1) * MG;            // accumulators per lane: 4 RG results + the row sum, per row group
+  __shared__ int sums[NSUM * 64];
   __shared__ __attribute__((aligned(16))) char lds[WAVES * AREA];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane >> 4, idx = lane & 15;
@@ -633,17 +451,17 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(j, rg);
   for (int c = lane; c < STRIDE / 16; c += 64) *reinterpret_cast<v4i *>(area + MR * STRIDE + c * 16) = v4i{0, 0, 0, 0};
-  for (int c = tid; c < (4 * RG + 1) * 64; c += WAVES * 64) sums[c] = 0;
+  for (int c = tid; c < NSUM * 64; c += WAVES * 64) sums[c] = 0;
   __syncthreads();  // (every wave gets here right after it has issued its loads)
 
-  // after the reduction, (row group, result register) pair q = wave + 8 t is finished by this wave: one output per
-  // lane and pair
-  constexpr int NQ = (4 * RG + WAVES - 1) / WAVES;
+  // after the reduction, (activation row group, channel group, result register) triple q = wave + 8 t is finished by
+  // this wave: one output per lane and triple
+  constexpr int NQ = (4 * RG * MG + WAVES - 1) / WAVES;
   int32_t p_mult[NQ], p_e[NQ], p_ls[NQ], p_bias2[NQ], p_zw[NQ];
 #pragma unroll
   for (int t = 0; t < NQ; ++t) {
-    const int q = wave + WAVES * t;
-    const int n = q < 4 * RG && (q >> 2) < rg_live ? n0 + (q >> 2) * 16 + 4 * grp + (q & 3) : n0;
+    const int q = (wave + WAVES * t) % (4 * RG);  // (the channel does not depend on the activation row group)
+    const int n = (q >> 2) < rg_live ? n0 + (q >> 2) * 16 + 4 * grp + (q & 3) : n0;
     p_mult[t] = rq.mult[n];
     p_e[t] = rq.rshift[n];
     p_ls[t] = rq.lshift[n];
@@ -651,11 +469,17 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
     p_zw[t] = rq.zw[n];
   }
 
-  v4i acc[RG], asum = {0, 0, 0, 0};
+  v4i acc[MG][RG], asum[MG];
 #pragma unroll
-  for (int rg = 0; rg < RG; ++rg) acc[rg] = v4i{0, 0, 0, 0};
+  for (int mg = 0; mg < MG; ++mg) {
+    asum[mg] = v4i{0, 0, 0, 0};
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) acc[mg][rg] = v4i{0, 0, 0, 0};
+  }
   const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
-  const char *frag = area + (idx < m_rows ? idx : MR) * STRIDE + grp * 16;
+  const char *frag[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) frag[mg] = area + (idx + 16 * mg < m_rows ? idx + 16 * mg : MR) * STRIDE + grp * 16;
 
   auto pass = [&](int base, auto refill) {
 #pragma unroll
@@ -666,7 +490,9 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
     }
 #pragma unroll
     for (int j = 0; j < D; ++j) {
-      const v4i x = *reinterpret_cast<const v4i *>(frag + j * 64);
+      v4i x[MG];
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) x[mg] = *reinterpret_cast<const v4i *>(frag[mg] + j * 64);
       v4i w[RG];
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];
@@ -675,8 +501,12 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
         for (int rg = 0; rg < RG; ++rg) wbuf[j][rg] = load_w(base + D + j, rg);
       }
 #pragma unroll
-      for (int rg = 0; rg < RG; ++rg) acc[rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x, acc[rg], 0, 0, 0);
-      if (rq.has_zw) asum = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x, asum, 0, 0, 0);
+      for (int mg = 0; mg < MG; ++mg) {
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg)
+          acc[mg][rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x[mg], acc[mg][rg], 0, 0, 0);
+        if (rq.has_zw) asum[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x[mg], asum[mg], 0, 0, 0);
+      }
     }
   };
   int base = 0;
@@ -684,24 +514,30 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   pass(base, std::false_type());
 
   // the partial sums meet in LDS accumulators (LDS atomic adds without a return value; the accumulators were zeroed
-  // before the first barrier): register r of row group rg at sums[(4 rg + r) * 64 + lane], the row sum behind them
+  // before the first barrier): for activation row group mg, register r of channel group rg at
+  // sums[((4 RG + 1) mg + 4 rg + r) * 64 + lane], the row sum behind them
 #pragma unroll
-  for (int rg = 0; rg < RG; ++rg)
+  for (int mg = 0; mg < MG; ++mg) {
+    int *dst = sums + (4 * RG + 1) * mg * 64 + lane;
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      __hip_atomic_fetch_add(&sums[(4 * rg + r) * 64 + lane], acc[rg][r], __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_WORKGROUP);
-  if (rq.has_zw)
-    __hip_atomic_fetch_add(&sums[4 * RG * 64 + lane], asum[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        __hip_atomic_fetch_add(dst + (4 * rg + r) * 64, acc[mg][rg][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (rq.has_zw)
+      __hip_atomic_fetch_add(dst + 4 * RG * 64, asum[mg][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
   __syncthreads();
 #pragma unroll
   for (int t = 0; t < NQ; ++t) {
-    const int q = wave + WAVES * t;
-    const int f_rg = q >> 2, f_r = q & 3;
-    const int f_n = n0 + f_rg * 16 + 4 * grp + f_r;
-    if (q < 4 * RG && idx < m_rows && f_n < g.n) {
-      uint32_t v = (uint32_t)sums[q * 64 + lane];
-      if (rq.has_zw) v -= (uint32_t)sums[4 * RG * 64 + lane] * (uint32_t)p_zw[t];
+    const int qq = wave + WAVES * t;
+    const int mg = qq / (4 * RG), q = qq % (4 * RG);
+    const int f_n = n0 + (q >> 2) * 16 + 4 * grp + (q & 3);
+    const int row = idx + 16 * mg;
+    if (qq < 4 * RG * MG && row < m_rows && f_n < g.n) {
+      const int *src = sums + (4 * RG + 1) * mg * 64 + lane;
+      uint32_t v = (uint32_t)src[q * 64];
+      if (rq.has_zw) v -= (uint32_t)src[4 * RG * 64] * (uint32_t)p_zw[t];
       v += (uint32_t)p_bias2[t];
       int32_t y;
       if (rq.fast) {
@@ -712,7 +548,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
       y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
       y = y < rq.amax ? y : rq.amax;
       y = y > rq.amin ? y : rq.amin;
-      g.c[(int64_t)idx * g.ldc + f_n] = (int8_t)y;
+      g.c[(int64_t)row * g.ldc + f_n] = (int8_t)y;
     }
   }
 }
@@ -732,17 +568,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_group_kernel(GemvGro
 }
 
 template <int WAVES, int D, typename F>
-static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8 or 16
+static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 32
   using std::integral_constant;
   if (m <= 2) return f(integral_constant<int, 2>());
   if (m <= 4) return f(integral_constant<int, 4>());
   if (m <= 8) return f(integral_constant<int, 8>());
-  if constexpr (WAVES * 17 * (D * 64 + 16) <= 160 * 1024) {
-    return f(integral_constant<int, 16>());
-  } else {
-    set_error("gemv: %d rows do not fit the staging area of this configuration", m);
-    return MI_PARAM_INVALID;
-  }
+  if (m <= 16) return f(integral_constant<int, 16>());
+  return f(integral_constant<int, 32>());
 }
 
 template <int WAVES, int RG, int D>
@@ -841,7 +673,8 @@ int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, con
   if (mfma) {  // the same choices as for a single matrix, made for the group's largest member
     for (int i = 0; i < count; ++i) grp.g[i].w = wv[i].blocked;
     const bool wide = n_max >= 8192 && k_pad_max <= 4096;
-    if (m > 16) return wide ? launch_group_mfma<2, 4, 2>(grp, m, stream) : launch_group_mfma<1, 8, 2>(grp, m, stream);
+    // (17..32 rows stage twice the rows: four steps per pass keep the staging areas of two workgroups in a CU's LDS)
+    if (m > 16) return wide ? launch_group_mfma_lds<8, 2, 4>(grp, m, stream) : launch_group_mfma_lds<8, 1, 4>(grp, m, stream);
     return wide ? launch_group_mfma_lds<8, 2, 4>(grp, m, stream) : launch_group_mfma_lds<8, 1, 8>(grp, m, stream);
   }
   return m == 1 ? launch_group_m<1>(grp, stream) : launch_group_m<2>(grp, stream);
@@ -856,12 +689,9 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
   GemvArgs g{a, lda, k / 16, w, wv.ldw, k_pad, n, c, ldc};
   if (prefers_mfma(m, wv)) {
     g.w = wv.blocked;
-    // two 16-channel groups per workgroup (half the activation traffic) once there are enough channels to fill the
-    // device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
-    if (m > 16) {  // two groups of 16 activation rows against every weight fragment
-      if (n >= 8192 && k_pad <= 4096) return launch_mfma<2, 4, 2>(g, m, rq, stream);
-      return launch_mfma<1, 8, 2>(g, m, rq, stream);
-    }
+    // three 16-channel groups per workgroup (a third of the activation traffic) once there are enough channels to
+    // fill the device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (m > 16 && !(n >= 8192 && k_pad <= 4096)) return launch_mfma_lds<8, 1, 4>(g, m, rq, stream);
     if (n >= 8192 && k_pad <= 4096) return launch_mfma_lds<8, 3, 4>(g, m, rq, stream);
     return launch_mfma_lds<8, 1, 8>(g, m, rq, stream);
   }
