@@ -493,6 +493,9 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
       v4i x[MG];
 #pragma unroll
       for (int mg = 0; mg < MG; ++mg) x[mg] = *reinterpret_cast<const v4i *>(frag[mg] + j * 64);
+      // (the slot is refilled before the products that read its old contents: the new fetch gets registers of its
+      //  own and does not have to wait for the old data, so a wave has up to two passes in flight; refilling after
+      //  the products saves a third of the registers and costs 5 % of the decode rate)
       v4i w[RG];
 #pragma unroll
       for (int rg = 0; rg < RG; ++rg) w[rg] = wbuf[j][rg];

@@ -36,6 +36,33 @@ def test_random_matmul(orc, seed):
         assert np.array_equal(got, want), (seed, it, m, n, k, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("seed", [11])
+def test_random_decode_rows_against_wide_matrices(orc, seed):
+    """2..32 activation rows against 8192 channels and more with K up to 4096: the matrix-core decode kernel with three
+    channel groups per workgroup (ragged last workgroups, ragged K, zero points, every activation), singly and as a
+    group launch of two members."""
+    import torch
+    rng = np.random.default_rng(seed)
+    orc.set_threads(16)
+    for it in range(36):
+        m = int(rng.integers(2, 33))
+        n = _pick(rng, [8192, 8193, 8200, 8250, 9001, 11008, 12288]) if it % 3 else int(rng.integers(8192, 9400))
+        k = _pick(rng, [64, 80, 1000, 1024, 2048, 3000, 4096]) if it % 2 else int(rng.integers(16, 4097))
+        case = T._mm_case(rng, m, n, k, _flag(rng), _flag(rng), True, _pick(rng, [0, 1, 3]), _flag(rng))
+        got, kern = T._gpu_matmul(case, device_tensors=True)
+        want = orc.matmul_int8(**case)
+        assert np.array_equal(got, want), (seed, it, m, n, k, int((got != want).sum()))
+        if it % 4 == 0:  # the same handle and a narrower one as one launch
+            c2 = T._mm_case(rng, m, int(rng.integers(16, 600)), k, True, _flag(rng), True, 0)
+            c2.update(a=case["a"], sx=case["sx"], zx=case["zx"])
+            k2 = K.MatmulInt8Kernel(c2["w"], c2["bias"], K.QuantParam(c2["sx"], c2["zx"]), T._qps(c2["sw"], c2["zw"]),
+                                    K.QuantParam(c2["so"], c2["zo"]), c2["b_transpose"], c2["act"])
+            outs = K.matmul_run_group([kern, k2], torch.from_numpy(case["a"]).cuda())
+            torch.cuda.synchronize()
+            assert np.array_equal(outs[0].cpu().numpy(), want), (seed, it, "group member 0")
+            assert np.array_equal(outs[1].cpu().numpy(), orc.matmul_int8(**c2)), (seed, it, "group member 1")
+
+
 @pytest.mark.parametrize("seed", [3])
 def test_random_dynamic_matmul(orc, seed):
     rng = np.random.default_rng(seed)
