@@ -14,6 +14,7 @@
 #include "quant_math.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 
@@ -381,7 +382,9 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 // Measured over a decoder layer against fragments fetched from global memory, eight partial reads per output and two
 // channel groups: 8 rows 4.57 -> 4.95 TB/s, 16 rows 3.95 -> 4.58, 32 rows 2.67 -> 3.66.
 // =====================================================================================================================
-template <int WAVES, int RG, int D, int MR>
+// DIAG: timing what-ifs (wrong results, see gemv_diag()): bit 0 = no activation fetches, bit 1 = no barrier before the
+// final sum.
+template <int WAVES, int RG, int D, int MR, int DIAG = 0>
 __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
   constexpr int ROWB = D * 64;                       // activation bytes per row and pass
   constexpr int STRIDE = ROWB + 16;                  // LDS row stride
@@ -442,9 +445,10 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   };
 
   // activations first: they return first, and the rows can be in LDS while the weights are still on their way
+  constexpr bool kFetchA = (DIAG & 1) == 0, kMeet = (DIAG & 2) == 0;
   v4i abuf[NLD];
 #pragma unroll
-  for (int i = 0; i < NLD; ++i) abuf[i] = load_a(0, i);
+  for (int i = 0; i < NLD; ++i) abuf[i] = kFetchA ? load_a(0, i) : v4i{lane, 1, 2, 3};
   v4i wbuf[D][RG];
 #pragma unroll
   for (int j = 0; j < D; ++j)
@@ -484,7 +488,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   auto pass = [&](int base, auto refill) {
 #pragma unroll
     for (int i = 0; i < NLD; ++i) store_a(base, i, abuf[i]);
-    if (decltype(refill)::value) {
+    if (decltype(refill)::value && kFetchA) {
 #pragma unroll
       for (int i = 0; i < NLD; ++i) abuf[i] = load_a(base + D, i);
     }
@@ -530,7 +534,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
     if (rq.has_zw)
       __hip_atomic_fetch_add(dst + 4 * RG * 64, asum[mg][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
-  __syncthreads();
+  if (kMeet) __syncthreads();
 #pragma unroll
   for (int t = 0; t < NQ; ++t) {
     const int qq = wave + WAVES * t;
@@ -556,9 +560,9 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   }
 }
 
-template <int WAVES, int RG, int D, int MR>
+template <int WAVES, int RG, int D, int MR, int DIAG = 0>
 __global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_kernel(GemvArgs g, int m_rows, RequantParams rq) {
-  gemv_mfma_lds_body<WAVES, RG, D, MR>(g, m_rows, rq, (int)blockIdx.x);
+  gemv_mfma_lds_body<WAVES, RG, D, MR, DIAG>(g, m_rows, rq, (int)blockIdx.x);
 }
 
 template <int WAVES, int RG, int D, int MR>
@@ -624,6 +628,30 @@ int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t 
   const int64_t want = (chunks + 255) / 256;
   hipLaunchKernelGGL(block_weights_kernel, dim3((unsigned)(want > 65536 ? 65536 : want)), dim3(256), 0, stream, w, ldw,
                      k_pad / 64, chunks, blocked);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+// Measurement aid, off unless the environment says MI355X_DIAG_GEMV=1, 2 or 3 when the library is first used: a
+// single-matrix launch with 5..8 activation rows then runs a build of the matrix-core kernel without its activation
+// fetches (1), without the barrier before the final sum (2) or without both (3).  The results are wrong; the launch
+// times show what each of the two costs.
+static int gemv_diag() {
+  static const int v = [] {
+    const char *e = getenv("MI355X_DIAG_GEMV");
+    return e != nullptr ? atoi(e) & 3 : 0;
+  }();
+  return v;
+}
+
+template <int RG, int D>
+static int launch_mfma_lds_diag(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  switch (gemv_diag()) {
+    case 1: hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, RG, D, 8, 1>), dim3(blocks), dim3(512), 0, stream, g, m, rq); break;
+    case 2: hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, RG, D, 8, 2>), dim3(blocks), dim3(512), 0, stream, g, m, rq); break;
+    default: hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, RG, D, 8, 3>), dim3(blocks), dim3(512), 0, stream, g, m, rq); break;
+  }
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -694,6 +722,10 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
     g.w = wv.blocked;
     // three 16-channel groups per workgroup (a third of the activation traffic) once there are enough channels to
     // fill the device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (gemv_diag() != 0 && m > 4 && m <= 8) {
+      return n >= 8192 && k_pad <= 4096 ? launch_mfma_lds_diag<3, 4>(g, m, rq, stream)
+                                        : launch_mfma_lds_diag<1, 8>(g, m, rq, stream);
+    }
     if (m > 16 && !(n >= 8192 && k_pad <= 4096)) return launch_mfma_lds<8, 1, 4>(g, m, rq, stream);
     if (n >= 8192 && k_pad <= 4096) return launch_mfma_lds<8, 3, 4>(g, m, rq, stream);
     return launch_mfma_lds<8, 1, 8>(g, m, rq, stream);
