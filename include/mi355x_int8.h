@@ -269,7 +269,7 @@ typedef struct mi_dynmm_desc {
   int32_t filter_quant_num; /* 1 or col; the zero point used is always filter_zps[0] (matmul_dynamic_int8.cc:52) */
   const double *filter_scales;
   const int32_t *filter_zps;
-  int32_t flags;               /* 0 or MI_DYNMM_WEIGHT_PACKED_SDOT */
+  int32_t flags;               /* 0 or MI_DYNMM_WEIGHT_PACKED_SDOT | MI_DYNMM_NO_DECODE_PACK */
   const int32_t *weight_sums;  /* with MI_DYNMM_WEIGHT_PACKED_SDOT: the model's weight-sums tensor
                                   [round_up(col, 16)], or NULL to have the sums computed from the weight */
 } mi_dynmm_desc;
@@ -284,6 +284,10 @@ typedef struct mi_dynmm_desc {
  * mindspore/lite/src/litert/runtime_packed_node_pass.cc:158-192), repacks it into its own layout and uses the given
  * sums.  b_transpose is ignored with this flag. */
 #define MI_DYNMM_WEIGHT_PACKED_SDOT 1
+/* Like mi_matmul, a dynamic MatMul handle holds a second, blocked form of its weights (deep x col bytes more) that
+ * serves 1..32 activation rows (decode) with the matrix-core weight-streaming kernel; MI_DYNMM_NO_DECODE_PACK skips it
+ * for handles that will only see larger row counts (few rows then run on the GEMM tiles, same results). */
+#define MI_DYNMM_NO_DECODE_PACK 2
 /* The unpacking by itself (host arithmetic, no GPU needed): packed -> weight_nk [col][deep] row-major. */
 int mi_unpack_weight_4x16(const int8_t *packed, int32_t col, int32_t deep, int8_t *weight_nk);
 

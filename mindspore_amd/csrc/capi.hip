@@ -470,6 +470,7 @@ struct mi_dynmm {
   int32_t zw0 = 0;
   bool has_bias = false;
   DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out, h_params;
+  DevBuf w_blocked;  // the weights in 1 KiB matrix-core blocks for 1..32 activation rows; built in create or absent
 };
 
 // No C++ exception may cross the C ABI: host allocations in the create calls can throw.
@@ -1240,7 +1241,7 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
     set_error("mi_dynmm_create: bad shape/activation");
     return MI_PARAM_INVALID;
   }
-  if ((d->flags & ~MI_DYNMM_WEIGHT_PACKED_SDOT) != 0) {
+  if ((d->flags & ~(MI_DYNMM_WEIGHT_PACKED_SDOT | MI_DYNMM_NO_DECODE_PACK)) != 0) {
     set_error("mi_dynmm_create: unknown flags 0x%x", d->flags);
     return MI_PARAM_INVALID;
   }
@@ -1279,6 +1280,20 @@ static int mi_dynmm_create_impl(const mi_dynmm_desc *d, const int8_t *weight_hos
   if (rc == MI_OK && h->has_bias) rc = upload(&h->bias, bs);
   if (rc != MI_OK) {
     return rc;
+  }
+  if ((d->flags & MI_DYNMM_NO_DECODE_PACK) == 0) {
+    // as for mi_matmul: an optimisation for few activation rows (decode), not a requirement -- without it those row
+    // counts run on the GEMM tiles, and a device without room for the copy still gets a working handle
+    rc = h->w_blocked.ensure((size_t)h->n_pad * h->k_pad);
+    if (rc == MI_OK)
+      rc = launch_block_weights(static_cast<const int8_t *>(h->w.p), h->n_pad, h->k_pad, h->ldw,
+                                static_cast<int8_t *>(h->w_blocked.p), nullptr);
+    if (rc == MI_OK && hipStreamSynchronize(nullptr) != hipSuccess) rc = MI_ERROR;
+    if (rc != MI_OK) {
+      (void)hipGetLastError();
+      h->w_blocked.release();
+      set_error("");
+    }
   }
   *out = owner.release();
   return MI_OK;
@@ -1323,7 +1338,13 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   dq.per_row = per_row ? 1 : 0;
   dq.deep = h->k;
   dq.act = h->act;
-  const WeightView w{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw, nullptr};
+  const WeightView w{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw,
+                     static_cast<const int8_t *>(h->w_blocked.p)};
+  // decode-sized runs: the matrix-core decode kernel streams the blocked weights once (any N, any output alignment)
+  // (one row runs on the row-major weights and needs no blocked copy, as long as the row fits the kernel's LDS form)
+  if (rows <= kGemvMaxRows && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024) &&
+      (rows == 1 || (w.blocked != nullptr && h->k_pad <= 1 << 20)))
+    return launch_gemv_dequant(a, lda, rows, k16, w, h->n, dq, c_dev, h->n, s);
   if ((h->n & 3) == 0 && (reinterpret_cast<uintptr_t>(c_dev) & 15) == 0)
     return launch_gemm_dequant(a, lda, rows, k16, w, h->n, dq, c_dev, h->n, s);
   const int n4 = round_up(h->n, 4);

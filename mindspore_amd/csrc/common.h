@@ -96,6 +96,10 @@ constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel can run (it doe
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
 
+// 1..32 rows of the dynamic-quant MatMul (fp32 out) on the blocked weight copy (w.blocked must be there).
+int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
+                        const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
+
 // Up to four weight matrices with the same K against the same activation rows, as one launch (the grid is the
 // concatenation of the members' grids); member i writes c[i] with row stride n[i].
 int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *w, const int *n,

@@ -62,8 +62,11 @@ struct GemvArgs {
 // last chunk; both meet a zero activation fragment or are not accumulated.
 // KS = 2: two neighbouring waves share their R rows, each walks one half of K (long rows: twice the waves, each with
 // half the registers, so that more of them are resident), and the even wave adds the odd wave's sums through LDS.
-template <int M, int R, int D, bool DIRECT, int KS>
-__device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantParams &rq, int block) {
+// DEQ: the fp32 epilogue of the dynamic-quant MatMul (see gemv_mfma_lds_body) instead of the requantising one.
+template <int M, int R, int D, bool DIRECT, int KS, bool DEQ = false>
+__device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantParams &rq, const DequantParams &dq,
+                                             int block) {
+  const bool has_zw = DEQ ? dq.zw0 != 0 : rq.has_zw != 0;
   static_assert(D % R == 0, "the slot -> row mapping must be static");
   static_assert(KS == 1 || KS == 2, "one or two waves per row group");
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -97,8 +100,21 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
   // behind the weight stream (the parameter arrays are padded to a multiple of 256 channels)
   const int my_rr = lane / M, my_m = lane - my_rr * M;
   const int my_n = n_base + (lane < R * M ? my_rr : 0);
-  const int32_t p_mult = rq.mult[my_n], p_e = rq.rshift[my_n], p_ls = rq.lshift[my_n], p_bias2 = rq.bias2[my_n];
-  const int32_t p_zw = rq.zw[my_n];
+  int32_t p_mult = 0, p_e = 0, p_ls = 0, p_bias2 = 0, p_zw = 0, d_wsum = 0, d_zx = 0;
+  float d_ws = 0.0f, d_bias = 0.0f, d_sx = 0.0f;
+  if (DEQ) {
+    d_ws = dq.wscale[my_n];
+    d_wsum = dq.wsum[my_n];
+    d_bias = dq.bias != nullptr ? dq.bias[my_n] : 0.0f;
+    d_sx = dq.qp_dev != nullptr ? dq.qp_dev[dq.per_row && lane < R * M ? my_m : 0].scale_f : dq.sx;
+    d_zx = dq.qp_dev != nullptr ? dq.qp_dev->zero_point : dq.zx;
+  } else {
+    p_mult = rq.mult[my_n];
+    p_e = rq.rshift[my_n];
+    p_ls = rq.lshift[my_n];
+    p_bias2 = rq.bias2[my_n];
+    p_zw = rq.zw[my_n];
+  }
 
   // DIRECT (the whole share of the wave is in flight, total <= D): every wave fetches its own activation fragments
   // straight into registers -- no LDS, no workgroup barrier.  Otherwise the workgroup stages the activations in LDS
@@ -157,7 +173,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
           } else {
             af[m] = seg < nseg ? sa[m * kc_pad + (seg0 + seg) * 64 + lane] : z;
           }
-          if (rq.has_zw) {
+          if (has_zw) {
             v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
             asum[m] = dot16(af[m], ones, asum[m]);
           }
@@ -176,7 +192,7 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
 #pragma unroll
   for (int m = 0; m < M; ++m) {
     int s = 0;
-    if (rq.has_zw) s = wave_sum(asum[m]);
+    if (has_zw) s = wave_sum(asum[m]);
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
       const int t = wave_sum(acc[rr][m]);
@@ -199,9 +215,21 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
   }
   if (lane < R * M) {
     const int m = my_m, n = my_n;
-    if (n < g.n) {
+    if (n < g.n && DEQ) {
       uint32_t v = (uint32_t)mine;
-      if (rq.has_zw) v -= (uint32_t)my_asum * (uint32_t)p_zw;
+      v += (uint32_t)dq.deep * (uint32_t)d_zx * (uint32_t)dq.zw0 - (uint32_t)d_zx * (uint32_t)d_wsum;
+      if (has_zw) v -= (uint32_t)dq.zw0 * (uint32_t)my_asum;
+      float d = __fmul_rn(__fmul_rn(d_sx, d_ws), (float)(int32_t)v);
+      if (dq.bias != nullptr) d = __fadd_rn(d, d_bias);
+      const bool with_act = dq.act == MI_ACT_RELU || dq.act == MI_ACT_RELU6;
+      const float act_lo = with_act ? 0.0f : -__builtin_inff();
+      const float act_hi = dq.act == MI_ACT_RELU6 ? 6.0f : __builtin_inff();
+      d = (act_lo > d) ? act_lo : d;
+      d = (act_hi < d) ? act_hi : d;
+      reinterpret_cast<float *>(g.c)[(int64_t)m * g.ldc + n] = d;
+    } else if (n < g.n) {
+      uint32_t v = (uint32_t)mine;
+      if (has_zw) v -= (uint32_t)my_asum * (uint32_t)p_zw;
       v += (uint32_t)p_bias2;
       const int32_t mult = p_mult, e = p_e;
       int32_t y;
@@ -220,7 +248,12 @@ __device__ __forceinline__ void gemv_i8_body(const GemvArgs &g, const RequantPar
 
 template <int M, int R, int D, bool DIRECT, int KS>
 __global__ __launch_bounds__(256) void gemv_i8_kernel(GemvArgs g, RequantParams rq) {
-  gemv_i8_body<M, R, D, DIRECT, KS>(g, rq, (int)blockIdx.x);
+  gemv_i8_body<M, R, D, DIRECT, KS, false>(g, rq, DequantParams{}, (int)blockIdx.x);
+}
+
+template <int M, int R, int D, bool DIRECT, int KS>
+__global__ __launch_bounds__(256) void gemv_i8_deq_kernel(GemvArgs g, DequantParams dq) {
+  gemv_i8_body<M, R, D, DIRECT, KS, true>(g, RequantParams{}, dq, (int)blockIdx.x);
 }
 
 // Several weight matrices against the same activation rows in one launch (MatMuls that share their input, e.g. the
@@ -260,7 +293,7 @@ __global__ __launch_bounds__(256) void gemv_i8_group_kernel(GemvGroup grp) {
   RequantParams rq;
   int block;
   pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
-  gemv_i8_body<M, R, D, DIRECT, KS>(g, rq, block);
+  gemv_i8_body<M, R, D, DIRECT, KS, false>(g, rq, DequantParams{}, block);
 }
 
 template <int M, int R, int D, bool DIRECT, int KS>
@@ -271,6 +304,16 @@ static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t s
   const int rows_per_block = 4 / KS * R;
   const int blocks = (g.n + rows_per_block - 1) / rows_per_block;
   hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), lds_bytes, stream, g, rq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <int M, int R, int D, bool DIRECT, int KS>
+static int launch_mrdx_deq(const GemvArgs &g, const DequantParams &dq, hipStream_t stream) {
+  const int lds_bytes = DIRECT ? 0 : M * ((g.kchunks + 63) / 64) * 1024;
+  const int rows_per_block = 4 / KS * R;
+  const int blocks = (g.n + rows_per_block - 1) / rows_per_block;
+  hipLaunchKernelGGL((gemv_i8_deq_kernel<M, R, D, DIRECT, KS>), dim3(blocks), dim3(256), lds_bytes, stream, g, dq);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -295,6 +338,9 @@ static int allow_big_lds() {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_kernel<M, 1, 12, false, 1>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  if (M == 1)
+    MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_deq_kernel<1, 1, 12, false, 1>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   return MI_OK;
 }
 
@@ -384,8 +430,14 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 // =====================================================================================================================
 // DIAG: timing what-ifs (wrong results, see gemv_diag()): bit 0 = no activation fetches, bit 1 = no barrier before the
 // final sum.
-template <int WAVES, int RG, int D, int MR, int DIAG = 0>
-__device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows, const RequantParams &rq, int block) {
+// DEQ: the fp32 epilogue of the dynamic-quant MatMul (DynamicMatmul4x16x4AIWI,
+// mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/dynamic_matmul_int8.c:99-143) instead of the requantising one:
+// value = sum - zx * sum_k w - zw * sum_k a + K * zx * zw, out = (sx[row] * sw[c]) * (float)value (+ bias) (activation);
+// g.c then points at floats.
+template <int WAVES, int RG, int D, int MR, int DIAG = 0, bool DEQ = false>
+__device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows, const RequantParams &rq,
+                                                   const DequantParams &dq, int block) {
+  const bool has_zw = DEQ ? dq.zw0 != 0 : rq.has_zw != 0;
   constexpr int ROWB = D * 64;                       // activation bytes per row and pass
   constexpr int STRIDE = ROWB + 16;                  // LDS row stride
   constexpr int LPR = ROWB / 16;                     // 16-byte chunks of one row in a pass
@@ -462,16 +514,29 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   // this wave: one output per lane and triple
   constexpr int NQ = (4 * RG * MG + WAVES - 1) / WAVES;
   int32_t p_mult[NQ], p_e[NQ], p_ls[NQ], p_bias2[NQ], p_zw[NQ];
+  float d_ws[NQ], d_bias[NQ], d_sx[NQ];  // DEQ: weight scale, fp32 bias, input scale of the lane's row
+  int32_t d_wsum[NQ], d_zx = 0;
 #pragma unroll
   for (int t = 0; t < NQ; ++t) {
-    const int q = (wave + WAVES * t) % (4 * RG);  // (the channel does not depend on the activation row group)
+    const int qq = wave + WAVES * t;
+    const int q = qq % (4 * RG);  // (the channel does not depend on the activation row group)
     const int n = (q >> 2) < rg_live ? n0 + (q >> 2) * 16 + 4 * grp + (q & 3) : n0;
-    p_mult[t] = rq.mult[n];
-    p_e[t] = rq.rshift[n];
-    p_ls[t] = rq.lshift[n];
-    p_bias2[t] = rq.bias2[n];
-    p_zw[t] = rq.zw[n];
+    if (DEQ) {
+      d_ws[t] = dq.wscale[n];
+      d_wsum[t] = dq.wsum[n];
+      d_bias[t] = dq.bias != nullptr ? dq.bias[n] : 0.0f;
+      int row = idx + 16 * (qq / (4 * RG));
+      row = row < m_rows ? row : m_rows - 1;
+      d_sx[t] = dq.qp_dev != nullptr ? dq.qp_dev[dq.per_row ? row : 0].scale_f : dq.sx;
+    } else {
+      p_mult[t] = rq.mult[n];
+      p_e[t] = rq.rshift[n];
+      p_ls[t] = rq.lshift[n];
+      p_bias2[t] = rq.bias2[n];
+      p_zw[t] = rq.zw[n];
+    }
   }
+  if (DEQ) d_zx = dq.qp_dev != nullptr ? dq.qp_dev->zero_point : dq.zx;
 
   v4i acc[MG][RG], asum[MG];
 #pragma unroll
@@ -512,7 +577,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
 #pragma unroll
         for (int rg = 0; rg < RG; ++rg)
           acc[mg][rg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[rg], x[mg], acc[mg][rg], 0, 0, 0);
-        if (rq.has_zw) asum[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x[mg], asum[mg], 0, 0, 0);
+        if (has_zw) asum[mg] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, x[mg], asum[mg], 0, 0, 0);
       }
     }
   };
@@ -531,7 +596,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         __hip_atomic_fetch_add(dst + (4 * rg + r) * 64, acc[mg][rg][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (rq.has_zw)
+    if (has_zw)
       __hip_atomic_fetch_add(dst + 4 * RG * 64, asum[mg][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   if (kMeet) __syncthreads();
@@ -544,25 +609,45 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
     if (qq < 4 * RG * MG && row < m_rows && f_n < g.n) {
       const int *src = sums + (4 * RG + 1) * mg * 64 + lane;
       uint32_t v = (uint32_t)src[q * 64];
-      if (rq.has_zw) v -= (uint32_t)src[4 * RG * 64] * (uint32_t)p_zw[t];
-      v += (uint32_t)p_bias2[t];
-      int32_t y;
-      if (rq.fast) {
-        y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[t]), p_e[t], (1 << p_e[t]) >> 1);
+      if (DEQ) {
+        // the steps of the reference, separately rounded: int -> float, the scale product, the product, the bias
+        v += (uint32_t)dq.deep * (uint32_t)d_zx * (uint32_t)dq.zw0 - (uint32_t)d_zx * (uint32_t)d_wsum[t];
+        if (has_zw) v -= (uint32_t)dq.zw0 * (uint32_t)src[4 * RG * 64];
+        float d = __fmul_rn(__fmul_rn(d_sx[t], d_ws[t]), (float)(int32_t)v);
+        if (dq.bias != nullptr) d = __fadd_rn(d, d_bias[t]);
+        // (bounds that are infinite where the reference makes no comparison: false for every d, NaN included)
+        const bool with_act = dq.act == MI_ACT_RELU || dq.act == MI_ACT_RELU6;
+        const float act_lo = with_act ? 0.0f : -__builtin_inff();
+        const float act_hi = dq.act == MI_ACT_RELU6 ? 6.0f : __builtin_inff();
+        d = (act_lo > d) ? act_lo : d;
+        d = (act_hi < d) ? act_hi : d;
+        reinterpret_cast<float *>(g.c)[(int64_t)row * g.ldc + f_n] = d;
       } else {
-        y = rdiv_pot(srdhm((int32_t)(v << p_ls[t]), p_mult[t]), p_e[t]);
+        if (has_zw) v -= (uint32_t)src[4 * RG * 64] * (uint32_t)p_zw[t];
+        v += (uint32_t)p_bias2[t];
+        int32_t y;
+        if (rq.fast) {
+          y = rdiv_pot_fast(srdhm_nosat((int32_t)v, p_mult[t]), p_e[t], (1 << p_e[t]) >> 1);
+        } else {
+          y = rdiv_pot(srdhm((int32_t)(v << p_ls[t]), p_mult[t]), p_e[t]);
+        }
+        y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
+        y = y < rq.amax ? y : rq.amax;
+        y = y > rq.amin ? y : rq.amin;
+        g.c[(int64_t)row * g.ldc + f_n] = (int8_t)y;
       }
-      y = (int32_t)((uint32_t)y + (uint32_t)rq.zo);
-      y = y < rq.amax ? y : rq.amax;
-      y = y > rq.amin ? y : rq.amin;
-      g.c[(int64_t)row * g.ldc + f_n] = (int8_t)y;
     }
   }
 }
 
 template <int WAVES, int RG, int D, int MR, int DIAG = 0>
 __global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_kernel(GemvArgs g, int m_rows, RequantParams rq) {
-  gemv_mfma_lds_body<WAVES, RG, D, MR, DIAG>(g, m_rows, rq, (int)blockIdx.x);
+  gemv_mfma_lds_body<WAVES, RG, D, MR, DIAG, false>(g, m_rows, rq, DequantParams{}, (int)blockIdx.x);
+}
+
+template <int WAVES, int RG, int D, int MR>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_deq_kernel(GemvArgs g, int m_rows, DequantParams dq) {
+  gemv_mfma_lds_body<WAVES, RG, D, MR, 0, true>(g, m_rows, RequantParams{}, dq, (int)blockIdx.x);
 }
 
 template <int WAVES, int RG, int D, int MR>
@@ -571,7 +656,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_group_kernel(GemvGro
   RequantParams rq;
   int block;
   pick_member(grp, (int)blockIdx.x, &g, &rq, &block);
-  gemv_mfma_lds_body<WAVES, RG, D, MR>(g, m_rows, rq, block);
+  gemv_mfma_lds_body<WAVES, RG, D, MR, 0, false>(g, m_rows, rq, DequantParams{}, block);
 }
 
 template <int WAVES, int D, typename F>
@@ -630,6 +715,17 @@ int launch_block_weights(const int8_t *w, int n_pad, int k_pad, int ldw, int8_t 
                      k_pad / 64, chunks, blocked);
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
+}
+
+template <int WAVES, int RG, int D>
+static int launch_mfma_lds_deq(const GemvArgs &g, int m, const DequantParams &dq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  return with_row_class<WAVES, D>(m, [&](auto mr) {
+    hipLaunchKernelGGL((gemv_mfma_lds_deq_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks), dim3(WAVES * 64),
+                       0, stream, g, m, dq);
+    MI_HIP_CHECK(hipGetLastError());
+    return (int)MI_OK;
+  });
 }
 
 // Measurement aid, off unless the environment says MI355X_DIAG_GEMV=1, 2 or 3 when the library is first used: a
@@ -731,6 +827,29 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
     return launch_mfma_lds<8, 1, 8>(g, m, rq, stream);
   }
   return m == 1 ? launch_m<1>(g, rq, stream) : launch_m<2>(g, rq, stream);
+}
+
+// The dynamic-quant MatMul at 1..32 rows: the matrix-core decode kernel on the blocked weight copy with the fp32
+// epilogue; the same configurations as for the requantising form.
+int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n,
+                        const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream) {
+  const int rc = check_gemv_operands(a, lda, m, k, wv, n, reinterpret_cast<const int8_t *>(c));
+  if (rc != MI_OK) return rc;
+  if (m == 1) {  // one row: the v_dot4 kernel on the row-major weights, as for the requantising MatMul
+    const GemvArgs g1{a, lda, k / 16, wv.w, wv.ldw, wv.k_pad, n, reinterpret_cast<int8_t *>(c), ldc};
+    return with_config<1>((g1.kchunks + 63) >> 6, [&](auto r, auto d, auto direct, auto ks) {
+      return launch_mrdx_deq<1, decltype(r)::value, decltype(d)::value, decltype(direct)::value, decltype(ks)::value>(
+          g1, dq, stream);
+    });
+  }
+  if (wv.blocked == nullptr) {
+    set_error("gemv: the blocked weight copy is missing");
+    return MI_NULL_PTR;
+  }
+  GemvArgs g{a, lda, k / 16, wv.blocked, wv.ldw, wv.k_pad, n, reinterpret_cast<int8_t *>(c), ldc};
+  const bool wide = n >= 8192 && wv.k_pad <= 4096;
+  if (wide) return launch_mfma_lds_deq<8, 3, 4>(g, m, dq, stream);
+  return m > 16 ? launch_mfma_lds_deq<8, 1, 4>(g, m, dq, stream) : launch_mfma_lds_deq<8, 1, 8>(g, m, dq, stream);
 }
 
 }  // namespace mi

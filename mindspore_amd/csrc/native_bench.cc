@@ -330,6 +330,74 @@ static int run_dynmm(int rows, int n, int k, int steps, int warmup) {
   return 0;
 }
 
+// The decoder layer of run_decode as dynamic-quant MatMuls (int8 activations with a run-time scale, fp32 out): three
+// layers' worth of distinct weights cycled, one launch per matrix.  no_pack = 1 creates the handles without the
+// blocked weight copy, so that the same rows run on the GEMM tiles (what they did before the decode kernel had the
+// fp32 epilogue).
+static int run_dyndecode(int rows, int layers, int steps, int warmup, int no_pack) {
+  struct DynMatrix {
+    mi_dynmm *h;
+    int8_t *act;
+    float *out;
+  };
+  std::vector<DynMatrix> ms;
+  double bytes = 0;
+  Rng rng{4321};
+  for (int l = 0; l < layers; ++l) {
+    for (int s = 0; s < 5; ++s) {
+      const int n = kDecode[s].n, k = kDecode[s].k;
+      std::vector<int8_t> w((size_t)n * k);
+      for (auto &x : w) x = normal_weight(&rng);
+      std::vector<double> scales(n);
+      std::vector<int32_t> zps(n, 0);
+      for (int c = 0; c < n; ++c) scales[c] = 0.001 + 0.009 * rng.uniform();
+      mi_dynmm_desc d{};
+      d.deep = k;
+      d.col = n;
+      d.b_transpose = 1;
+      d.act_type = MI_ACT_NONE;
+      d.filter_quant_num = n;
+      d.filter_scales = scales.data();
+      d.filter_zps = zps.data();
+      d.flags = no_pack ? MI_DYNMM_NO_DECODE_PACK : 0;
+      DynMatrix m{};
+      CHECK_MI(mi_dynmm_create(&d, w.data(), nullptr, &m.h));
+      std::vector<int8_t> a((size_t)rows * k);
+      for (auto &x : a) x = (int8_t)(rng.next() & 0xff);
+      CHECK_HIP(hipMalloc(&m.act, a.size()));
+      CHECK_HIP(hipMalloc(&m.out, (size_t)rows * n * 4));
+      CHECK_HIP(hipMemcpy(m.act, a.data(), a.size(), hipMemcpyHostToDevice));
+      ms.push_back(m);
+      bytes += (double)n * k + (double)rows * k + 4.0 * rows * n + 12.0 * n;
+    }
+  }
+  hipStream_t st;
+  CHECK_HIP(hipStreamCreate(&st));
+  hipEvent_t e0, e1;
+  CHECK_HIP(hipEventCreate(&e0));
+  CHECK_HIP(hipEventCreate(&e1));
+  auto step = [&]() -> int {
+    for (auto &m : ms) CHECK_MI(mi_dynmm_run(m.h, m.act, rows, 0.031, -3, m.out, st));
+    return 0;
+  };
+  for (int i = 0; i < warmup; ++i)
+    if (step()) return 1;
+  CHECK_HIP(hipStreamSynchronize(st));
+  CHECK_HIP(hipEventRecord(e0, st));
+  for (int i = 0; i < steps; ++i)
+    if (step()) return 1;
+  CHECK_HIP(hipEventRecord(e1, st));
+  CHECK_HIP(hipEventSynchronize(e1));
+  float t = 0;
+  CHECK_HIP(hipEventElapsedTime(&t, e0, e1));
+  const double ms_step = t / steps;
+  printf("{\"mode\": \"dyndecode\", \"m\": %d, \"blocked_copy\": %d, \"launches_per_step\": %zu, \"ms_per_step\": %.6f, "
+         "\"us_per_launch\": %.3f, \"bytes_per_step\": %.0f, \"gbps\": %.1f}\n",
+         rows, no_pack ? 0 : 1, ms.size(), ms_step, ms_step * 1e3 / ms.size(), bytes, bytes / (ms_step * 1e-3) / 1e9);
+  for (auto &m : ms) mi_dynmm_destroy(m.h);
+  return 0;
+}
+
 static int run_gemm(int rows, int n, int k, int steps, int warmup) {
   const Shape sh{"gemm", n, k};
   Matrix m;
@@ -407,13 +475,15 @@ static int run_dw(int ih, int iw, int c, int steps, int warmup) {
 
 int main(int argc, char **argv) {
   if (argc < 2) {
-    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup> | shape <n> <k> <rows> <steps> <warmup> | bert <steps> <warmup> | dynmm <rows> <n> <k> <steps> <warmup> | gemm <rows> <n> <k> <steps> <warmup> | dw <h> <w> <c> <steps> <warmup>\n");
+    fprintf(stderr, "usage: native_bench decode <rows> <layers> <steps> <warmup> | warm <rows> <steps> <warmup> | read <mib> <steps> <warmup> | shape <n> <k> <rows> <steps> <warmup> | dyndecode <rows> <layers> <steps> <warmup> [no_pack] | bert <steps> <warmup> | dynmm <rows> <n> <k> <steps> <warmup> | gemm <rows> <n> <k> <steps> <warmup> | dw <h> <w> <c> <steps> <warmup>\n");
     return 2;
   }
   CHECK_MI(mi_init(0));
   if (strcmp(argv[1], "shape") == 0 && argc >= 7) return run_shape(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
   if (strcmp(argv[1], "decode") == 0 && argc >= 6) return run_decode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]));
   if (strcmp(argv[1], "warm") == 0 && argc >= 5) return run_warm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]));
+  if (strcmp(argv[1], "dyndecode") == 0 && argc >= 6)
+    return run_dyndecode(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argc >= 7 ? atoi(argv[6]) : 0);
   if (strcmp(argv[1], "bert") == 0 && argc >= 4) return run_bert(atoi(argv[2]), atoi(argv[3]));
   if (strcmp(argv[1], "dynmm") == 0 && argc >= 7) return run_dynmm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));
   if (strcmp(argv[1], "gemm") == 0 && argc >= 7) return run_gemm(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]));

@@ -320,10 +320,11 @@ class MatmulDynamicInt8Kernel(_Handle):
     _destroy = "mi_dynmm_destroy"
 
     def __init__(self, weight, bias, weight_quant, transpose_b=True, act=ACT_NONE, device=0, packed_sdot=None,
-                 weight_sums=None):
+                 weight_sums=None, decode_pack=True):
         """packed_sdot=(N, K): `weight` is the flat byte string a model converted for the ARM dot-product kernel
         carries (blocks of 16 channels x 4 K-bytes, RowMajor2Row4x16MajorInt8 / RowMajor2Col4x16MajorInt8) and
-        weight_sums, if given, its int32 weight-sums tensor [round_up(N, 16)]."""
+        weight_sums, if given, its int32 weight-sums tensor [round_up(N, 16)].  decode_pack=False skips the blocked
+        second copy of the weights that serves 1..32 rows (MI_DYNMM_NO_DECODE_PACK)."""
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)
@@ -348,7 +349,8 @@ class MatmulDynamicInt8Kernel(_Handle):
                 raise ValueError("weight_sums goes with a packed weight and holds at least N entries")
             sums = weight_sums.ctypes.data_as(C.POINTER(C.c_int32))
         d = _lib.DynmmDesc(self.k, self.n, 1 if transpose_b else 0, act, nq, scales, zps,
-                           _lib.DYNMM_WEIGHT_PACKED_SDOT if packed_sdot is not None else 0, sums)
+                           (_lib.DYNMM_WEIGHT_PACKED_SDOT if packed_sdot is not None else 0)
+                           | (0 if decode_pack else _lib.DYNMM_NO_DECODE_PACK), sums)
         _lib.check(L.mi_dynmm_create(C.byref(d), weight.ctypes.data, None if bias is None else bias.ctypes.data,
                                      C.byref(self._h)), "mi_dynmm_create")
 

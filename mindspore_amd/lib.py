@@ -58,6 +58,7 @@ class DynmmDesc(C.Structure):
 
 
 DYNMM_WEIGHT_PACKED_SDOT = 1
+DYNMM_NO_DECODE_PACK = 2
 
 
 class ConvInfer(C.Structure):

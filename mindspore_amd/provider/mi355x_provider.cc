@@ -404,20 +404,21 @@ class MatmulKernel : public kernel::Kernel {
     std::vector<int32_t> zps;
     FilterQuant(w, &scales, &zps);
     const void *bias = inputs_.size() > kBiasIndex ? inputs_[kBiasIndex].Data().get() : nullptr;
+    // The second packed form of the weights serves up to 32 activation rows; a node whose inferred output already has
+    // more rows than that does without it (half the device memory per weight).  Should the model later be resized
+    // to a few rows, they run on the GEMM tiles.
+    const auto oshape = outputs_[0].Shape();
+    bool rows_known = !oshape.empty();
+    for (int64_t e : oshape) rows_known = rows_known && e >= 0;
+    const int64_t rows_now = batched_ && oshape.size() >= 2 ? oshape[oshape.size() - 2] : RowsOfOutput(outputs_[0]);
+    const bool no_decode_pack = rows_known && rows_now > kSiblingMaxRows;
     if (outputs_[0].DataType() == DataType::kNumberTypeInt8) {
       const auto iq = inputs_[0].QuantParams().front();
       const auto oq = outputs_[0].QuantParams().front();
       mi_matmul_desc d{k, n, b_transpose_ ? 1 : 0, act_, iq.scale, iq.zero_point, oq.scale, oq.zero_point,
                        static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
       d.b_batch = static_cast<int32_t>(b_batch);
-      // The second packed form of the weights serves 2..32 activation rows; a node whose inferred output already has
-      // more rows than that does without it (half the device memory per weight).  Should the model later be resized
-      // to a few rows, they run on the GEMM tiles.
-      const auto oshape = outputs_[0].Shape();
-      bool rows_known = !oshape.empty();
-      for (int64_t e : oshape) rows_known = rows_known && e >= 0;
-      const int64_t rows_now = batched_ && oshape.size() >= 2 ? oshape[oshape.size() - 2] : RowsOfOutput(outputs_[0]);
-      if (rows_known && rows_now > kSiblingMaxRows) d.flags |= MI_MATMUL_NO_DECODE_PACK;
+      if (no_decode_pack) d.flags |= MI_MATMUL_NO_DECODE_PACK;
       const int rc = mi_matmul_create(&d, static_cast<const int8_t *>(w.Data().get()),
                                       static_cast<const int32_t *>(bias), &full_);
       // (a session that runs its nodes in parallel gives no order to lean on: no groups there)
@@ -429,6 +430,7 @@ class MatmulKernel : public kernel::Kernel {
     }
     if (batched_) return kLiteError;  // (the creator declines batched weights for the dynamic MatMul)
     mi_dynmm_desc d{k, n, b_transpose_ ? 1 : 0, act_, static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
+    if (no_decode_pack) d.flags |= MI_DYNMM_NO_DECODE_PACK;
     return ToStatus(
       mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_));
   }

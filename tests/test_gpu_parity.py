@@ -452,6 +452,39 @@ def test_dynamic_matmul(orc):
         assert np.array_equal(got2.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("n,k", [(4096, 4096), (8200, 1040), (11008, 528), (300, 11008), (21, 2800), (7, 100),
+                                 (8250, 80), (515, 3000)])
+def test_dynamic_matmul_decode_rows(orc, n, k):
+    """1..32 rows of the dynamic-quant MatMul take the matrix-core decode kernel with the fp32 epilogue (one and three
+    channel groups per workgroup, ragged channels and K, one and two groups of activation rows); 33 rows and a handle
+    without the blocked weight copy take the GEMM tiles.  Per-tensor and per-channel weight scales, a weight zero
+    point, bias, every activation; input parameters by value, from device memory, and one scale per row."""
+    import torch
+    rng = np.random.default_rng(n * 7 + k)
+    orc.set_threads(16)
+    w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+    for it, m in enumerate([1, 2, 3, 5, 8, 16, 17, 31, 32, 33]):
+        a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+        nf = n if it & 1 else 1
+        sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+        zw = np.full(nf, 0 if it & 2 else int(rng.integers(-5, 6)), np.int32)
+        bias = rng.standard_normal(n).astype(np.float32) if it % 3 else None
+        sx, zx, act = float(rng.uniform(0.01, 0.1)), int(rng.integers(-128, 128)), [0, 1, 3][it % 3]
+        kern = K.MatmulDynamicInt8Kernel(w, bias, _qps(sw, zw), True, act)
+        want = orc.dynamic_matmul(a, w, bias, sx, zx, sw, zw, act, True)
+        got = kern.run(torch.from_numpy(a).cuda(), QP(sx, zx)).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (m, n, k, "by value")
+        if it % 4 == 0:  # the same through a handle without the blocked copy
+            plain = K.MatmulDynamicInt8Kernel(w, bias, _qps(sw, zw), True, act, decode_pack=False)
+            got = plain.run(torch.from_numpy(a).cuda(), QP(sx, zx)).cpu().numpy()
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (m, n, k, "no blocked copy")
+        if it % 2 == 0:  # one input scale per row (the zero point is that of the first row, as in the reference)
+            sxr = rng.uniform(0.01, 0.1, m).astype(np.float32)
+            want_r = orc.dynamic_matmul_rows(a, w, bias, sxr, zx, sw, zw, act)
+            got_r = kern.run(a, [QP(float(s), zx) for s in sxr])
+            assert np.array_equal(got_r.view(np.uint32), want_r.view(np.uint32)), (m, n, k, "per row")
+
+
 def test_dynamic_quant_chained_into_matmul(orc):
     """DynamicQuant -> dynamic MatMul with the scale / zero point handed over in device memory."""
     import torch
