@@ -404,6 +404,10 @@ def _dq_inputs():
     sp[5], sp[77], sp[900] = np.nan, 12.5, -13.25
     xs.append(sp)
     xs.append(np.array([np.inf, -np.inf, 1.0, -2.0, 3e38, -3e38, np.nan, 0.0] * 9, np.float32))
+    # both sides of the size up to which one workgroup does the whole tensor in one launch, and a few decode rows
+    xs += [rng.standard_normal(24576).astype(np.float32), rng.standard_normal(24577).astype(np.float32) * 2 - 1,
+           rng.standard_normal((2, 11008)).astype(np.float32), rng.standard_normal(24575).astype(np.float32),
+           rng.standard_normal(3).astype(np.float32), rng.standard_normal((8, 4096)).astype(np.float32)]
     return xs
 
 
