@@ -307,6 +307,14 @@ int mi_dynmm_run_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, double in
  * quantisation.  row_params_dev is what mi_dynquant_run_segments wrote. */
 int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_dq_params *row_params_dev,
                       float *c_dev, void *stream);
+/* Dynamic MatMuls that read the same activation rows (q / k / v, gate / up of a dynamic-quant transformer), as
+ * mi_matmul_run_group does for the full-quant MatMul: up to four handles with the same deep at up to 32 rows run as
+ * one launch, anything else member by member.  The input's scale and zero point come by value (params_dev NULL), from
+ * the block a DynamicQuant run left on the device (params_dev, per_row 0) or as one scale per row (per_row 1);
+ * member i writes c_dev[i], fp32 [rows, col_i].  No counterpart in the reference, which runs one node at a time. */
+int mi_dynmm_run_group(mi_dynmm *const *handles, int32_t count, const int8_t *a_dev, int32_t rows, double in_scale,
+                       int32_t in_zp, const mi_dq_params *params_dev, int32_t per_row, float *const *c_dev,
+                       void *stream);
 int mi_dynmm_run_rows_host(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,
                            float *c_host);
 /* As mi_matmul_reserve (the buffers of MatmulDynamicBaseInt8CPUKernel::ReSize, LK/int8/matmul_dynamic_base_int8.cc:

@@ -1313,6 +1313,21 @@ int mi_dynmm_create(const mi_dynmm_desc *d, const int8_t *weight_host, const flo
   return guarded("mi_dynmm_create", [&] { return mi_dynmm_create_impl(d, weight_host, bias_host, out); });
 }
 
+static DequantParams dequant_params(const mi_dynmm *h, float sx, int32_t zx, const mi_dq_params *qp_dev, bool per_row) {
+  DequantParams dq;
+  dq.wscale = static_cast<const float *>(h->wscale.p);
+  dq.bias = h->has_bias ? static_cast<const float *>(h->bias.p) : nullptr;
+  dq.wsum = static_cast<const int32_t *>(h->wsum.p);
+  dq.qp_dev = qp_dev;
+  dq.sx = sx;
+  dq.zx = zx;
+  dq.zw0 = h->zw0;
+  dq.per_row = per_row ? 1 : 0;
+  dq.deep = h->k;
+  dq.act = h->act;
+  return dq;
+}
+
 static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float sx, int32_t zx,
                           const mi_dq_params *qp_dev, float *c_dev, hipStream_t s, bool per_row = false) {
   if (h == nullptr || a_dev == nullptr || c_dev == nullptr) {
@@ -1327,17 +1342,7 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
   int64_t lda = 0;
   int k16 = 0;
   if ((rc = prepare_rows(a_dev, rows, h->k, Workspace::growable(&h->a_ws), s, &a, &lda, &k16)) != MI_OK) return rc;
-  DequantParams dq;
-  dq.wscale = static_cast<const float *>(h->wscale.p);
-  dq.bias = h->has_bias ? static_cast<const float *>(h->bias.p) : nullptr;
-  dq.wsum = static_cast<const int32_t *>(h->wsum.p);
-  dq.qp_dev = qp_dev;
-  dq.sx = sx;
-  dq.zx = zx;
-  dq.zw0 = h->zw0;
-  dq.per_row = per_row ? 1 : 0;
-  dq.deep = h->k;
-  dq.act = h->act;
+  const DequantParams dq = dequant_params(h, sx, zx, qp_dev, per_row);
   const WeightView w{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw,
                      static_cast<const int8_t *>(h->w_blocked.p)};
   // decode-sized runs: the matrix-core decode kernel streams the blocked weights once (any N, any output alignment)
@@ -1384,6 +1389,61 @@ int mi_dynmm_run_rows(mi_dynmm *h, const int8_t *a_dev, int32_t rows, const mi_d
     return MI_NULL_PTR;
   }
   return dynmm_run_impl(h, a_dev, rows, 0.0f, 0, row_params_dev, c_dev, static_cast<hipStream_t>(stream), true);
+}
+
+int mi_dynmm_run_group(mi_dynmm *const *handles, int32_t count, const int8_t *a_dev, int32_t rows, double in_scale,
+                       int32_t in_zp, const mi_dq_params *params_dev, int32_t per_row, float *const *c_dev,
+                       void *stream) {
+  if (handles == nullptr || a_dev == nullptr || c_dev == nullptr) {
+    set_error("mi_dynmm_run_group: null argument");
+    return MI_NULL_PTR;
+  }
+  if (count < 1 || rows < 0 || (per_row != 0 && params_dev == nullptr)) {
+    set_error("mi_dynmm_run_group: count=%d rows=%d per_row=%d", count, rows, per_row);
+    return MI_PARAM_INVALID;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (handles[i] == nullptr || c_dev[i] == nullptr) {
+      set_error("mi_dynmm_run_group: member %d is null", i);
+      return MI_NULL_PTR;
+    }
+    if (handles[i]->k != handles[0]->k) {
+      set_error("mi_dynmm_run_group: member %d has deep=%d, member 0 has %d", i, handles[i]->k, handles[0]->k);
+      return MI_PARAM_INVALID;
+    }
+  }
+  if (rows == 0) return MI_OK;
+  int rc = ensure_device();
+  if (rc != MI_OK) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int8_t *a = nullptr;
+  int64_t lda = 0;
+  int k16 = 0;
+  // the activation rows are brought into the kernels' form once, for all members
+  if ((rc = prepare_rows(a_dev, rows, handles[0]->k, Workspace::growable(&handles[0]->a_ws), s, &a, &lda, &k16)) != MI_OK)
+    return rc;
+  // decode-sized runs of up to four members go out as one launch; anything else runs member by member
+  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvMaxRows &&
+                    (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024);
+  for (int i = 0; i < count && one_launch; ++i)
+    one_launch = rows == 1 || (handles[i]->w_blocked.p != nullptr && handles[i]->k_pad <= 1 << 20);
+  if (one_launch) {
+    WeightView wv[4];
+    DequantParams dq[4];
+    int n[4];
+    for (int i = 0; i < count; ++i) {
+      const mi_dynmm *h = handles[i];
+      wv[i] = WeightView{static_cast<const int8_t *>(h->w.p), h->k_pad, h->ldw, static_cast<const int8_t *>(h->w_blocked.p)};
+      dq[i] = dequant_params(h, (float)in_scale, in_zp, params_dev, per_row != 0);
+      n[i] = h->n;
+    }
+    return launch_gemv_group_dequant(a, lda, rows, k16, count, wv, n, dq, c_dev, s);
+  }
+  for (int i = 0; i < count; ++i) {
+    if ((rc = dynmm_run_impl(handles[i], a_dev, rows, (float)in_scale, in_zp, params_dev, c_dev[i], s, per_row != 0)) != MI_OK)
+      return rc;
+  }
+  return MI_OK;
 }
 
 static int mi_dynmm_run_rows_host_impl(mi_dynmm *h, const int8_t *a_host, int32_t rows, const double *in_scales, int32_t in_zp,

@@ -100,6 +100,11 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
 int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
 
+// Up to four dynamic-quant MatMuls with the same K against the same activation rows, as one launch; member i writes
+// c[i] (fp32) with row stride n[i].  For more than one row every member needs w.blocked.
+int launch_gemv_group_dequant(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *w, const int *n,
+                              const DequantParams *dq, float *const *c, hipStream_t stream);
+
 // Up to four weight matrices with the same K against the same activation rows, as one launch (the grid is the
 // concatenation of the members' grids); member i writes c[i] with row stride n[i].
 int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *w, const int *n,

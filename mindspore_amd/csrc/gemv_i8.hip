@@ -261,14 +261,18 @@ __global__ __launch_bounds__(256) void gemv_i8_deq_kernel(GemvArgs g, DequantPar
 // first finds the member it belongs to.  Every field is picked with selects over constant indices, which keeps the
 // table in scalar registers (a dynamically indexed kernel argument would be copied to scratch memory).
 constexpr int kGemvGroupMax = 4;
-struct GemvGroup {
+template <typename P>  // P: the members' epilogue parameters (RequantParams or DequantParams)
+struct GemvGroupT {
   int count;
   int block_end[kGemvGroupMax];  // exclusive prefix sums of the members' workgroup counts
   GemvArgs g[kGemvGroupMax];
-  RequantParams rq[kGemvGroupMax];
+  P rq[kGemvGroupMax];
 };
+typedef GemvGroupT<RequantParams> GemvGroup;
+typedef GemvGroupT<DequantParams> GemvGroupDeq;
 
-__device__ __forceinline__ void pick_member(const GemvGroup &grp, int block, GemvArgs *g, RequantParams *rq,
+template <typename P>
+__device__ __forceinline__ void pick_member(const GemvGroupT<P> &grp, int block, GemvArgs *g, P *rq,
                                             int *local_block) {
   int member = 0;
 #pragma unroll
@@ -297,6 +301,15 @@ __global__ __launch_bounds__(256) void gemv_i8_group_kernel(GemvGroup grp) {
 }
 
 template <int M, int R, int D, bool DIRECT, int KS>
+__global__ __launch_bounds__(256) void gemv_i8_group_deq_kernel(GemvGroupDeq grp) {
+  GemvArgs g;
+  DequantParams dq;
+  int block;
+  pick_member(grp, (int)blockIdx.x, &g, &dq, &block);
+  gemv_i8_body<M, R, D, DIRECT, KS, true>(g, RequantParams{}, dq, block);
+}
+
+template <int M, int R, int D, bool DIRECT, int KS>
 static int launch_mrdx(const GemvArgs &g, const RequantParams &rq, hipStream_t stream) {
   auto kern = gemv_i8_kernel<M, R, D, DIRECT, KS>;
   // (more than 64 KiB of dynamic LDS needs the attribute that gemv_prepare_device set when the library was initialised)
@@ -318,15 +331,19 @@ static int launch_mrdx_deq(const GemvArgs &g, const DequantParams &dq, hipStream
   return MI_OK;
 }
 
-template <int M, int R, int D, bool DIRECT, int KS>
-static int launch_group_mrdx(GemvGroup &grp, hipStream_t stream) {
+template <int M, int R, int D, bool DIRECT, int KS, typename P>
+static int launch_group_mrdx(GemvGroupT<P> &grp, hipStream_t stream) {
   const int lds_bytes = DIRECT ? 0 : M * ((grp.g[0].kchunks + 63) / 64) * 1024;
   int blocks = 0;
   for (int i = 0; i < grp.count; ++i) {
     blocks += (grp.g[i].n + 4 / KS * R - 1) / (4 / KS * R);
     grp.block_end[i] = blocks;
   }
-  hipLaunchKernelGGL((gemv_i8_group_kernel<M, R, D, DIRECT, KS>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
+  if constexpr (std::is_same<P, DequantParams>::value) {
+    hipLaunchKernelGGL((gemv_i8_group_deq_kernel<M, R, D, DIRECT, KS>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
+  } else {
+    hipLaunchKernelGGL((gemv_i8_group_kernel<M, R, D, DIRECT, KS>), dim3(blocks), dim3(256), lds_bytes, stream, grp);
+  }
   MI_HIP_CHECK(hipGetLastError());
   return MI_OK;
 }
@@ -338,9 +355,12 @@ static int allow_big_lds() {
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_kernel<M, 1, 12, false, 1>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-  if (M == 1)
+  if (M == 1) {
     MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_deq_kernel<1, 1, 12, false, 1>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    MI_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(gemv_i8_group_deq_kernel<1, 1, 12, false, 1>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  }
   return MI_OK;
 }
 
@@ -379,8 +399,8 @@ static int with_config(int nseg, F &&f) {
   }
 }
 
-template <int M>
-static int launch_group_m(GemvGroup &grp, hipStream_t stream) {  // the choice depends on K only
+template <int M, typename P>
+static int launch_group_m(GemvGroupT<P> &grp, hipStream_t stream) {  // the choice depends on K only
   return with_config<M>((grp.g[0].kchunks + 63) >> 6, [&](auto r, auto d, auto direct, auto ks) {
     return launch_group_mrdx<M, decltype(r)::value, decltype(d)::value, decltype(direct)::value, decltype(ks)::value>(
         grp, stream);
@@ -659,6 +679,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_group_kernel(GemvGro
   gemv_mfma_lds_body<WAVES, RG, D, MR, 0, false>(g, m_rows, rq, DequantParams{}, block);
 }
 
+template <int WAVES, int RG, int D, int MR>
+__global__ __launch_bounds__(WAVES * 64) void gemv_mfma_lds_group_deq_kernel(GemvGroupDeq grp, int m_rows) {
+  GemvArgs g;
+  DequantParams dq;
+  int block;
+  pick_member(grp, (int)blockIdx.x, &g, &dq, &block);
+  gemv_mfma_lds_body<WAVES, RG, D, MR, 0, true>(g, m_rows, RequantParams{}, dq, block);
+}
+
 template <int WAVES, int D, typename F>
 static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 32
   using std::integral_constant;
@@ -669,16 +698,21 @@ static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 
   return f(integral_constant<int, 32>());
 }
 
-template <int WAVES, int RG, int D>
-static int launch_group_mfma_lds(GemvGroup &grp, int m, hipStream_t stream) {
+template <int WAVES, int RG, int D, typename P>
+static int launch_group_mfma_lds(GemvGroupT<P> &grp, int m, hipStream_t stream) {
   int blocks = 0;
   for (int i = 0; i < grp.count; ++i) {
     blocks += (grp.g[i].n + RG * 16 - 1) / (RG * 16);
     grp.block_end[i] = blocks;
   }
   return with_row_class<WAVES, D>(m, [&](auto mr) {
-    hipLaunchKernelGGL((gemv_mfma_lds_group_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks), dim3(WAVES * 64),
-                       0, stream, grp, m);
+    if constexpr (std::is_same<P, DequantParams>::value) {
+      hipLaunchKernelGGL((gemv_mfma_lds_group_deq_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks),
+                         dim3(WAVES * 64), 0, stream, grp, m);
+    } else {
+      hipLaunchKernelGGL((gemv_mfma_lds_group_kernel<WAVES, RG, D, decltype(mr)::value>), dim3(blocks),
+                         dim3(WAVES * 64), 0, stream, grp, m);
+    }
     MI_HIP_CHECK(hipGetLastError());
     return (int)MI_OK;
   });
@@ -850,6 +884,36 @@ int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
   const bool wide = n >= 8192 && wv.k_pad <= 4096;
   if (wide) return launch_mfma_lds_deq<8, 3, 4>(g, m, dq, stream);
   return m > 16 ? launch_mfma_lds_deq<8, 1, 4>(g, m, dq, stream) : launch_mfma_lds_deq<8, 1, 8>(g, m, dq, stream);
+}
+
+// The dynamic-quant MatMuls that share their input, as one launch (mi_dynmm_run_group): one row on the dot kernel,
+// 2..32 rows on the matrix-core kernel (every member then needs its blocked weight copy).
+int launch_gemv_group_dequant(const int8_t *a, int64_t lda, int m, int k, int count, const WeightView *wv, const int *n,
+                              const DequantParams *dq, float *const *c, hipStream_t stream) {
+  if (count < 1 || count > kGemvGroupMax) {
+    set_error("gemv group: %d members (1..%d)", count, kGemvGroupMax);
+    return MI_PARAM_INVALID;
+  }
+  GemvGroupDeq grp{};
+  grp.count = count;
+  int n_max = 0, k_pad_max = 0;
+  for (int i = 0; i < count; ++i) {
+    const int rc = check_gemv_operands(a, lda, m, k, wv[i], n[i], reinterpret_cast<const int8_t *>(c[i]));
+    if (rc != MI_OK) return rc;
+    if (m > 1 && wv[i].blocked == nullptr) {
+      set_error("gemv group: the blocked weight copy is missing");
+      return MI_NULL_PTR;
+    }
+    grp.g[i] = GemvArgs{a, lda, k / 16, m == 1 ? wv[i].w : wv[i].blocked, wv[i].ldw, wv[i].k_pad, n[i],
+                        reinterpret_cast<int8_t *>(c[i]), n[i]};
+    grp.rq[i] = dq[i];
+    n_max = std::max(n_max, n[i]);
+    k_pad_max = std::max(k_pad_max, wv[i].k_pad);
+  }
+  if (m == 1) return launch_group_m<1>(grp, stream);
+  const bool wide = n_max >= 8192 && k_pad_max <= 4096;
+  if (m > 16) return wide ? launch_group_mfma_lds<8, 2, 4>(grp, m, stream) : launch_group_mfma_lds<8, 1, 4>(grp, m, stream);
+  return wide ? launch_group_mfma_lds<8, 2, 4>(grp, m, stream) : launch_group_mfma_lds<8, 1, 8>(grp, m, stream);
 }
 
 }  // namespace mi

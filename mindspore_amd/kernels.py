@@ -184,6 +184,33 @@ def matmul_run_group(kernels, a, outs=None):
     return outs
 
 
+def dynmm_run_group(kernels, a, in_quant=None, params_dev=None, row_params=None, outs=None):
+    """Runs several MatmulDynamicInt8Kernel objects that share the input `a` (a contiguous CUDA int8 tensor [..., K])
+    as mi_dynmm_run_group does: decode-sized inputs go out as one launch.  The input's quantisation comes as one
+    QuantParam (in_quant), as the address of the block a DynamicQuantKernel.run left on the device (params_dev) or as
+    the tensor DynamicQuantKernel.run_rows returned (row_params).  Returns the list of fp32 outputs."""
+    import torch
+    L = _lib.load()
+    k = kernels[0].k
+    if a.dtype != torch.int8 or not a.is_cuda or not a.is_contiguous() or a.shape[-1] != k:
+        raise ValueError("expected a contiguous CUDA int8 tensor [..., %d]" % k)
+    rows = a.numel() // k
+    if outs is None:
+        outs = [torch.empty(a.shape[:-1] + (kn.n,), dtype=torch.float32, device=a.device) for kn in kernels]
+    hs = (C.c_void_p * len(kernels))(*[kn._h.value for kn in kernels])
+    cs = (C.c_void_p * len(kernels))(*[o.data_ptr() for o in outs])
+    scale, zp, dev, per_row = 0.0, 0, None, 0
+    if row_params is not None:
+        dev, per_row = row_params.data_ptr(), 1
+    elif params_dev is not None:
+        dev = params_dev
+    else:
+        scale, zp = float(in_quant.scale), int(in_quant.zero_point)
+    _lib.check(L.mi_dynmm_run_group(hs, len(kernels), a.data_ptr(), rows, scale, zp, dev, per_row, cs, _stream()),
+               "mi_dynmm_run_group")
+    return outs
+
+
 class ConvolutionInt8Kernel(_Handle):
     """Conv2DFusion int8, NHWC.  weight [OC, KH, KW, IC] (group 1) or [C, KH, KW] (depthwise, group == C).
     pad = (up, down, left, right).  Raises MiError with code MI_NOT_SUPPORT for the cases a provider must decline.

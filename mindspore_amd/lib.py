@@ -18,7 +18,7 @@ EXPORTS = [
     "mi_conv_create", "mi_conv_out_shape", "mi_conv_same_pad", "mi_conv_run", "mi_conv_run_host", "mi_conv_reserve", "mi_conv_destroy",
     "mi_dynquant_create", "mi_dynquant_run", "mi_dynquant_get_params", "mi_dynquant_device_params",
     "mi_dynquant_run_host", "mi_dynquant_run_segments", "mi_dynquant_run_segments_host", "mi_dynquant_destroy",
-    "mi_unpack_weight_4x16", "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
+    "mi_unpack_weight_4x16", "mi_dynmm_create", "mi_dynmm_run", "mi_dynmm_run_chained", "mi_dynmm_run_host", "mi_dynmm_run_rows", "mi_dynmm_run_group", "mi_dynmm_run_rows_host", "mi_dynmm_reserve",
     "mi_dynmm_destroy",
     "mi_infer_matmul", "mi_infer_fullconnection", "mi_infer_conv2d",
     "mi_device_malloc", "mi_device_free", "mi_copy_to_device", "mi_copy_to_host", "mi_copy_to_host_async", "mi_stream_synchronize", "mi_stream_create", "mi_stream_destroy",
@@ -144,6 +144,7 @@ def load():
     L.mi_dynmm_run_chained.argtypes = [vp, vp, i32, vp, vp, vp]
     L.mi_dynmm_run_host.argtypes = [vp, vp, i32, dbl, i32, vp]
     L.mi_dynmm_run_rows.argtypes = [vp, vp, i32, vp, vp, vp]
+    L.mi_dynmm_run_group.argtypes = [C.POINTER(vp), i32, vp, i32, C.c_double, i32, vp, i32, C.POINTER(vp), vp]
     L.mi_dynmm_run_rows_host.argtypes = [vp, vp, i32, C.POINTER(dbl), i32, vp]
     L.mi_dynmm_reserve.argtypes = [vp, i32]
     L.mi_dynmm_destroy.argtypes = [vp]

@@ -431,8 +431,14 @@ class MatmulKernel : public kernel::Kernel {
     if (batched_) return kLiteError;  // (the creator declines batched weights for the dynamic MatMul)
     mi_dynmm_desc d{k, n, b_transpose_ ? 1 : 0, act_, static_cast<int32_t>(scales.size()), scales.data(), zps.data()};
     if (no_decode_pack) d.flags |= MI_DYNMM_NO_DECODE_PACK;
-    return ToStatus(
-      mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_));
+    const int rc =
+      mi_dynmm_create(&d, static_cast<const int8_t *>(w.Data().get()), static_cast<const float *>(bias), &dyn_);
+    // dynamic MatMuls that read the same DynamicQuant output (q / k / v, gate / up) form groups like the full-quant ones
+    if (rc == MI_OK && !inputs_[0].IsConst() && context_ != nullptr && !context_->GetEnableParallel() &&
+        getenv("MI355X_NO_SIBLING_GROUPS") == nullptr) {
+      group_ = SiblingGroup::Join(context_, inputs_[0], k, this);
+    }
+    return ToStatus(rc);
   }
 
   int ReSize() override {  // the row count is read from the input tensor at every Execute
@@ -457,7 +463,7 @@ class MatmulKernel : public kernel::Kernel {
         return io_.Deliver(&outputs_[0]);
       }
     }
-    if (full_ != nullptr && group_ != nullptr && rows <= kSiblingMaxRows) {
+    if (group_ != nullptr && rows <= kSiblingMaxRows) {
       const int rc = ExecuteWithSiblings(rows);
       if (rc != kNotGrouped) return rc;
     }
@@ -507,26 +513,45 @@ class MatmulKernel : public kernel::Kernel {
   int ExecuteWithSiblings(int32_t rows) {
     std::vector<MatmulKernel *> run;
     run.push_back(this);
+    const bool dynamic = dyn_ != nullptr;
     for (MatmulKernel *m : group_->Members()) {
-      if (m == this || m->full_ == nullptr) continue;
+      if (m == this || (dynamic ? m->dyn_ == nullptr : m->full_ == nullptr)) continue;
       if (RowsOfOutput(m->outputs_[0]) != rows || m->inputs_[0].ElementNum() != static_cast<int64_t>(rows) * k_) continue;
       run.push_back(m);
     }
     if (run.size() < 2) return kNotGrouped;
+    // a dynamic MatMul reads its input's scale and zero point at every run: where DynamicQuant left them on the
+    // device, or one pair from the tensor; one pair per row on the host keeps the members apart (each uploads its own)
+    QuantOnDevice on_dev;
+    const bool quant_on_device = dynamic && inputs_[0].GetDeviceData() != nullptr &&
+                                 Published::Quant(inputs_[0].GetDeviceData(), &on_dev) &&
+                                 (!on_dev.per_row || on_dev.rows == rows);
+    const auto iqs = dynamic && !quant_on_device ? inputs_[0].QuantParams() : std::vector<QuantParam>();
+    if (dynamic && !quant_on_device && iqs.size() != 1) return kNotGrouped;
     const auto *a = static_cast<const int8_t *>(io_.Input(&inputs_[0]));
     if (a == nullptr) return kLiteNullptr;
-    std::vector<mi_matmul *> handles;
-    std::vector<int8_t *> outs;
+    if (dynamic && quant_on_device && a != inputs_[0].GetDeviceData()) return kNotGrouped;
+    std::vector<void *> outs;
     for (MatmulKernel *m : run) {
       void *c = m->io_.Output(m->outputs_[0].DataSize());
       if (c == nullptr) return kLiteNullptr;
-      handles.push_back(m->full_);
-      outs.push_back(static_cast<int8_t *>(c));
+      outs.push_back(c);
     }
-    if (mi_matmul_run_group(handles.data(), static_cast<int32_t>(handles.size()), a, rows, outs.data(),
-                            io_.stream()) != MI_OK) {
-      return kLiteError;
+    int rc = MI_ERROR;
+    if (dynamic) {
+      std::vector<mi_dynmm *> handles;
+      for (MatmulKernel *m : run) handles.push_back(m->dyn_);
+      rc = mi_dynmm_run_group(handles.data(), static_cast<int32_t>(handles.size()), a, rows,
+                              quant_on_device ? 0.0 : iqs[0].scale, quant_on_device ? 0 : iqs[0].zero_point,
+                              quant_on_device ? on_dev.params : nullptr, quant_on_device && on_dev.per_row ? 1 : 0,
+                              reinterpret_cast<float *const *>(outs.data()), io_.stream());
+    } else {
+      std::vector<mi_matmul *> handles;
+      for (MatmulKernel *m : run) handles.push_back(m->full_);
+      rc = mi_matmul_run_group(handles.data(), static_cast<int32_t>(handles.size()), a, rows,
+                               reinterpret_cast<int8_t *const *>(outs.data()), io_.stream());
     }
+    if (rc != MI_OK) return kLiteError;
     g_group_launches.fetch_add(1, std::memory_order_relaxed);
     for (MatmulKernel *m : run) {
       if (m == this) continue;

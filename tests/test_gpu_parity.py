@@ -489,6 +489,54 @@ def test_dynamic_matmul_decode_rows(orc, n, k):
             assert np.array_equal(got_r.view(np.uint32), want_r.view(np.uint32)), (m, n, k, "per row")
 
 
+@pytest.mark.parametrize("rows,k,ns", [(1, 4096, (1100, 900)), (2, 1040, (64, 260, 36)), (1, 144, (8, 4, 12, 20)),
+                                       (5, 4096, (256, 8200)), (8, 1040, (48, 16, 100)), (17, 2048, (40, 520)),
+                                       (32, 400, (33, 31, 64, 5)), (40, 528, (96, 100)), (3, 64, (8, 8, 8, 8, 8))])
+def test_dynamic_matmul_group_equals_member_by_member(orc, rows, k, ns):
+    """mi_dynmm_run_group: dynamic MatMuls that share their input run as one launch (up to 32 rows, two to four
+    members) or one after the other (more rows, five members); every member's fp32 output is compared with the oracle,
+    for an input scale given by value, read from the block DynamicQuant left on the device, and one scale per row."""
+    import torch
+    rng = np.random.default_rng(rows * 137 + k + sum(ns))
+    orc.set_threads(16)
+    x = (rng.standard_normal((rows, k)) * 2).astype(np.float32)
+    cases, kerns = [], []
+    for i, n in enumerate(ns):
+        w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+        nf = n if i & 1 else 1
+        sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+        zw = np.full(nf, 0 if i % 3 else int(rng.integers(-5, 6)), np.int32)
+        bias = rng.standard_normal(n).astype(np.float32) if i != 1 else None
+        act = [0, 1, 3, 0][i % 4]
+        cases.append((w, bias, sw, zw, act))
+        kerns.append(K.MatmulDynamicInt8Kernel(w, bias, _qps(sw, zw), True, act))
+    # by value
+    a = rng.integers(-128, 128, (rows, k), dtype=np.int8)
+    sx, zx = float(rng.uniform(0.01, 0.1)), int(rng.integers(-128, 128))
+    outs = K.dynmm_run_group(kerns, torch.from_numpy(a).cuda(), in_quant=QP(sx, zx))
+    torch.cuda.synchronize()
+    for i, (w, bias, sw, zw, act) in enumerate(cases):
+        want = orc.dynamic_matmul(a, w, bias, sx, zx, sw, zw, act, True)
+        assert np.array_equal(outs[i].cpu().numpy().view(np.uint32), want.view(np.uint32)), (rows, k, ns, i, "by value")
+    # chained behind DynamicQuant, per tensor and per row
+    dq = K.DynamicQuantKernel(False)
+    q, _ = dq.run(torch.from_numpy(x).cuda(), fetch_params=False)
+    outs = K.dynmm_run_group(kerns, q, params_dev=dq.device_params())
+    torch.cuda.synchronize()
+    q_ref, s_ref, z_ref = orc.dynamic_quant(x)
+    for i, (w, bias, sw, zw, act) in enumerate(cases):
+        want = orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw, act, True)
+        assert np.array_equal(outs[i].cpu().numpy().view(np.uint32), want.view(np.uint32)), (rows, k, ns, i, "chained")
+    dqr = K.DynamicQuantKernel(True)
+    qr, row_params = dqr.run_rows(torch.from_numpy(x).cuda())
+    outs = K.dynmm_run_group(kerns, qr, row_params=row_params)
+    torch.cuda.synchronize()
+    qr_ref, sr_ref, zr_ref = orc.dynamic_quant_segments(x, True)
+    for i, (w, bias, sw, zw, act) in enumerate(cases):
+        want = orc.dynamic_matmul_rows(qr_ref, w, bias, sr_ref.astype(np.float32), int(zr_ref[0]), sw, zw, act)
+        assert np.array_equal(outs[i].cpu().numpy().view(np.uint32), want.view(np.uint32)), (rows, k, ns, i, "per row")
+
+
 def test_dynamic_quant_chained_into_matmul(orc):
     """DynamicQuant -> dynamic MatMul with the scale / zero point handed over in device memory."""
     import torch

@@ -706,6 +706,52 @@ def test_dynamic_quant_feeds_the_dynamic_matmul_on_the_device(H, orc):
 
 
 @pytest.mark.gpu
+def test_sibling_dynamic_matmuls_run_as_one_launch(H, orc):
+    """DynamicQuant feeding three dynamic MatMuls (q / k / v): at up to 32 rows the first MatMul executed runs all three
+    as one launch, reading the scale where DynamicQuant left it on the device (one for the tensor, or one per row), and
+    the others deliver what it left; beyond 32 rows every node runs by itself.  Every output equals the oracle's."""
+    rng = np.random.default_rng(31)
+    k = 256
+    for per_row in (False, True):
+        dq_op = op(DYNQUANT, symmetric=1, n_prefer_axes=1, prefer_axes=(0,)) if per_row else op(DYNQUANT)
+        dq = Node(H, dq_op, [tensor(F32, (4, k), None)], I8, out_name=b"q")
+        assert dq.stage == OK, (dq.stage, dq.code)
+        sibs = []
+        for n in (96, 320, 48):
+            w = rng.integers(-127, 128, (n, k), dtype=np.int8)
+            sw = rng.uniform(1e-3, 1e-2, n).astype(np.float32).astype(np.float64)
+            bias = rng.standard_normal(n).astype(np.float32)
+            mm = Node(H, op(MATMUL, transpose_b=1),
+                      [tensor(I8, (4, k), None), tensor(I8, w.shape, w, True, [(s, 0) for s in sw]),
+                       tensor(F32, (n,), bias, True)], F32, producer=dq)
+            assert mm.stage == OK, (mm.stage, mm.code)
+            sibs.append((mm, w, sw, bias))
+        before = H.mi355x_provider_group_launches()
+        runs = 0
+        for rows in (4, 1, 9, 40):
+            x = (rng.standard_normal((rows, k)) * 3).astype(np.float32)
+            dq.run(x)
+            for mm, *_ in sibs:
+                mm.resize_linked()
+            if per_row:
+                q_ref, scales_ref, _ = orc.dynamic_quant_segments(x, True)
+            else:
+                q_ref, s_ref, z_ref = orc.dynamic_quant(x, False)
+            for mm, w, sw, bias in sibs:
+                mm.run_linked()
+                y, _ = mm.output()
+                zw = np.zeros(w.shape[0], np.int32)
+                ref = orc.dynamic_matmul_rows(q_ref, w, bias, scales_ref, 0, sw, zw) if per_row else \
+                    orc.dynamic_matmul(q_ref, w, bias, s_ref, z_ref, sw, zw)
+                assert y.shape == ref.shape and np.array_equal(y.view(np.uint32), ref.view(np.uint32)), (per_row, rows)
+            runs += 1 if rows <= 32 else 0
+        assert H.mi355x_provider_group_launches() - before == runs, (per_row, runs)
+        for mm, *_ in reversed(sibs):
+            mm.close()
+        dq.close()
+
+
+@pytest.mark.gpu
 def test_time_of_dynamic_quant_into_the_qkv_matmul(H, orc):
     """Per-layer host time of DynamicQuant (4096 x 768) -> QKV dynamic MatMul (2304 channels) through the provider:
     with every tensor handed over on the host, with the int8 tensor device-only, and with both outputs device-only
