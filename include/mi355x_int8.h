@@ -110,9 +110,9 @@ typedef struct mi_matmul_desc {
 
 /* All weight packing happens in mi_matmul_create (the role of TransferB, LK/int8/matmul_base_int8.cc:360-384: pack
  * once at Prepare).  Two packed forms are kept: K-contiguous rows (GEMM tiles; one activation row) and 1 KiB
- * blocks of 16 channels x 64 K-bytes in matrix-core operand order (2..32 activation rows, the batched decode
+ * blocks of 16 channels x 64 K-bytes in matrix-core operand order (2..64 activation rows, the batched decode
  * kernel).  MI_MATMUL_NO_DECODE_PACK skips the second form (deep x col bytes of device memory less) for callers
- * that know they never run with 2..32 rows; such a handle still accepts those row counts and runs two rows on the
+ * that know they never run with 2..64 rows; such a handle still accepts those row counts and runs two rows on the
  * one-row kernel's two-row form and the others on the GEMM tiles.  mi_matmul_run never packs, allocates for packing or waits. */
 #define MI_MATMUL_NO_DECODE_PACK 1
 
@@ -285,7 +285,7 @@ typedef struct mi_dynmm_desc {
  * sums.  b_transpose is ignored with this flag. */
 #define MI_DYNMM_WEIGHT_PACKED_SDOT 1
 /* Like mi_matmul, a dynamic MatMul handle holds a second, blocked form of its weights (deep x col bytes more) that
- * serves 1..32 activation rows (decode) with the matrix-core weight-streaming kernel; MI_DYNMM_NO_DECODE_PACK skips it
+ * serves 1..64 activation rows (decode) with the matrix-core weight-streaming kernel; MI_DYNMM_NO_DECODE_PACK skips it
  * for handles that will only see larger row counts (few rows then run on the GEMM tiles, same results). */
 #define MI_DYNMM_NO_DECODE_PACK 2
 /* The unpacking by itself (host arithmetic, no GPU needed): packed -> weight_nk [col][deep] row-major. */

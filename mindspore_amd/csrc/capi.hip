@@ -419,8 +419,8 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
                             const Workspace &c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
-  // one row: the dot kernel on the row-major weights; 2..32 rows: the matrix-core decode kernel on the blocked copy
-  // made at create time -- a handle without it runs two rows on the dot kernel and 3..32 on the GEMM tiles
+  // one row: the dot kernel on the row-major weights; 2..64 rows: the matrix-core decode kernel on the blocked copy
+  // made at create time -- a handle without it runs two rows on the dot kernel and 3..64 on the GEMM tiles
   const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
                                            : rows <= kGemvMaxRows && st.w_blocked.p != nullptr && st.k_pad <= 1 << 20;
   if (skinny) {
@@ -815,7 +815,7 @@ int mi_matmul_run_group(mi_matmul *const *handles, int32_t count, const int8_t *
   if ((rc = prepare_rows(a_dev, rows, handles[0]->st.k, Workspace::growable(&handles[0]->a_ws), s, &a, &lda, &k16)) != MI_OK)
     return rc;
   // decode-sized runs of up to four members go out as one launch; anything else runs member by member
-  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvMaxRows;
+  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvGroupMaxRows;
   for (int i = 0; i < count && one_launch; ++i)
     one_launch = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
                                       : handles[i]->st.w_blocked.p != nullptr && handles[i]->st.k_pad <= 1 << 20;
@@ -1423,7 +1423,7 @@ int mi_dynmm_run_group(mi_dynmm *const *handles, int32_t count, const int8_t *a_
   if ((rc = prepare_rows(a_dev, rows, handles[0]->k, Workspace::growable(&handles[0]->a_ws), s, &a, &lda, &k16)) != MI_OK)
     return rc;
   // decode-sized runs of up to four members go out as one launch; anything else runs member by member
-  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvMaxRows &&
+  bool one_launch = count >= 2 && count <= 4 && rows <= kGemvGroupMaxRows &&
                     (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024);
   for (int i = 0; i < count && one_launch; ++i)
     one_launch = rows == 1 || (handles[i]->w_blocked.p != nullptr && handles[i]->k_pad <= 1 << 20);

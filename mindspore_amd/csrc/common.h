@@ -74,7 +74,7 @@ struct WeightView {
   const int8_t *w;
   int k_pad;
   int ldw;
-  // Second copy for the matrix-core decode kernel (2..32 activation rows), or nullptr: the same bytes regrouped into
+  // Second copy for the matrix-core decode kernel (2..64 activation rows), or nullptr: the same bytes regrouped into
   // 1 KiB blocks [row / 16][k / 64], the 64 16-byte chunks of a block in the order the lanes of the MFMA operand take
   // them ([(k % 64) / 16][row % 16]), so that a wave instruction fetches 1 KiB front to back.  Built on the device
   // when the handle is created (launch_block_weights).
@@ -91,12 +91,13 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
 
 // Skinny-M path (m <= kGemvMaxRows): streams the weights once with 16-byte coalesced loads.
-constexpr int kGemvMaxRows = 32;
+constexpr int kGemvMaxRows = 64;
+constexpr int kGemvGroupMaxRows = 32;  // the group launches (several matrices, one launch) stop here
 constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel can run (it does for one row, and for two when the handle has no blocked copy), above it the MFMA kernel
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);
 
-// 1..32 rows of the dynamic-quant MatMul (fp32 out) on the blocked weight copy (w.blocked must be there).
+// 1..64 rows of the dynamic-quant MatMul (fp32 out) on the blocked weight copy (w.blocked must be there).
 int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream);
 

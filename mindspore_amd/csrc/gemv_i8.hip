@@ -1,6 +1,6 @@
-// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 32 activation rows
+// Skinny-M (decode) int8 GEMV with the requantising epilogue of the full-quant MatMul: M <= 64 activation rows
 // against the packed int8 weight matrix (n_pad rows of k_pad bytes, row stride ldw): a v_dot4 kernel for one row (and
-// for two on a handle without the blocked weight copy), matrix-core kernels on the blocked copy for 2 <= M <= 32.
+// for two on a handle without the blocked weight copy), matrix-core kernels on the blocked copy for 2 <= M <= 64.
 // The kernels are HBM-bound on the weight stream, so the design goal is "every weight byte crosses HBM once, in 1 KiB
 // coalesced wave loads, with enough loads in flight":
 //   - v_dot4 kernel: a wave owns R consecutive output channels and walks K in 1 KiB segments (64 lanes x 16 bytes),
@@ -8,7 +8,7 @@
 //     once at the end;
 //   - matrix-core kernels: a workgroup of eight waves owns RG x 16 channels, the waves split K, the weights are the
 //     16-row operand of v_mfma_i32_16x16x64_i8 and are read from 1 KiB blocks laid out in lane order; the activation
-//     rows go through LDS (up to 16 rows) or straight into fragments (17..32 rows).
+//     rows go through LDS.
 // Arithmetic reference: MatmulInt8Opt, mindspore/ccsrc/plugin/device/cpu/kernel/nnacl/int8/matmul_int8.c:296-331.
 #include "common.h"
 #include "quant_math.h"
@@ -416,10 +416,10 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 }
 
 // =====================================================================================================================
-// 2 <= M <= 32 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
+// 2 <= M <= 64 activation rows: the matrix cores do the products, so the arithmetic cost does not grow with M.
 // v_mfma_i32_16x16x64_i8 with the WEIGHTS as the 16-row operand: lane (g = lane / 16, i = lane % 16) supplies 16
 // contiguous K bytes of weight row i (K offset 16 g inside the 64-byte step) and the same 16 K bytes of activation row
-// i (zero for i >= M; rows 16..31 are a second fragment against the same weight fragment); the result register r of
+// i (zero for i >= M; rows 16..31, 32..47 and 48..63 are further fragments against the same weight fragment); the result register r of
 // that lane is output (channel 4 g + r, activation row i).
 // The weights come from the blocked copy: 1 KiB blocks [row / 16][k / 64], inside a block the 16-byte chunks in lane
 // order ([(k % 64) / 16][row % 16]), so a wave instruction fetches 64 consecutive chunks -- eight whole cache lines --
@@ -444,7 +444,7 @@ static int launch_m(const GemvArgs &g, const RequantParams &rq, hipStream_t stre
 // matrices at 8 rows: 0.1-0.3 us per launch against eight partial reads per output by the first waves only).
 // RG channel groups per workgroup: activation bytes per weight byte are M / (16 RG); three where there are channels
 // enough (a 12288 x 4096 matrix is then 256 workgroups, one per CU, all resident at once).  MR = the number of rows
-// rounded up to 2, 4, 8, 16 or 32 (the number of fetch instructions is a compile-time constant).
+// rounded up to 2, 4, 8, 16, 32 or 64 (the number of fetch instructions is a compile-time constant).
 // Measured over a decoder layer against fragments fetched from global memory, eight partial reads per output and two
 // channel groups: 8 rows 4.57 -> 4.95 TB/s, 16 rows 3.95 -> 4.58, 32 rows 2.67 -> 3.66.
 // =====================================================================================================================
@@ -463,7 +463,7 @@ __device__ __forceinline__ void gemv_mfma_lds_body(const GemvArgs &g, int m_rows
   constexpr int LPR = ROWB / 16;                     // 16-byte chunks of one row in a pass
   constexpr int NLD = (MR * LPR + 63) / 64;          // fetch instructions per pass
   constexpr int AREA = (MR + 1) * STRIDE;            // per wave
-  constexpr int MG = MR > 16 ? 2 : 1;                // groups of 16 activation rows
+  constexpr int MG = MR > 16 ? MR / 16 : 1;          // groups of 16 activation rows
   constexpr int NSUM = (4 * RG + 1) * MG;            // accumulators per lane: 4 RG results + the row sum, per row group
   __shared__ int sums[NSUM * 64];
   __shared__ __attribute__((aligned(16))) char lds[WAVES * AREA];
@@ -698,6 +698,26 @@ static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 
   return f(integral_constant<int, 32>());
 }
 
+// 33..64 rows: four groups of 16 activation rows against every weight fragment, two steps per pass (the staging
+// area of 64 rows and the accumulators leave room for no more).  Measured against the 64 x 64 GEMM tiles these row
+// counts ran on before (us per launch at 64 rows): 12288 x 4096 17.9 -> 14.9, 4096 x 4096 15.8 -> 8.9,
+// 4096 x 11008 34.9 -> 18.7.
+template <int RG>
+static int launch_mfma_lds_64(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, RG, 2, 64>), dim3(blocks), dim3(512), 0, stream, g, m, rq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+template <int RG>
+static int launch_mfma_lds_deq_64(const GemvArgs &g, int m, const DequantParams &dq, hipStream_t stream) {
+  const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
+  hipLaunchKernelGGL((gemv_mfma_lds_deq_kernel<8, RG, 2, 64>), dim3(blocks), dim3(512), 0, stream, g, m, dq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 template <int WAVES, int RG, int D, typename P>
 static int launch_group_mfma_lds(GemvGroupT<P> &grp, int m, hipStream_t stream) {
   int blocks = 0;
@@ -818,6 +838,10 @@ int launch_gemv_group(const int8_t *a, int64_t lda, int m, int k, int count, con
     set_error("gemv group: %d members (1..%d)", count, kGemvGroupMax);
     return MI_PARAM_INVALID;
   }
+  if (m > kGemvGroupMaxRows) {
+    set_error("gemv group: %d rows (1..%d)", m, kGemvGroupMaxRows);
+    return MI_PARAM_INVALID;
+  }
   GemvGroup grp{};
   grp.count = count;
   int n_max = 0, k_pad_max = 0;
@@ -852,6 +876,9 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
     g.w = wv.blocked;
     // three 16-channel groups per workgroup (a third of the activation traffic) once there are enough channels to
     // fill the device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (m > 32) {
+      return n >= 8192 && k_pad <= 4096 ? launch_mfma_lds_64<3>(g, m, rq, stream) : launch_mfma_lds_64<1>(g, m, rq, stream);
+    }
     if (gemv_diag() != 0 && m > 4 && m <= 8) {
       return n >= 8192 && k_pad <= 4096 ? launch_mfma_lds_diag<3, 4>(g, m, rq, stream)
                                         : launch_mfma_lds_diag<1, 8>(g, m, rq, stream);
@@ -863,7 +890,7 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
   return m == 1 ? launch_m<1>(g, rq, stream) : launch_m<2>(g, rq, stream);
 }
 
-// The dynamic-quant MatMul at 1..32 rows: the matrix-core decode kernel on the blocked weight copy with the fp32
+// The dynamic-quant MatMul at 1..64 rows: the matrix-core decode kernel on the blocked weight copy with the fp32
 // epilogue; the same configurations as for the requantising form.
 int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const WeightView &wv, int n,
                         const DequantParams &dq, float *c, int64_t ldc, hipStream_t stream) {
@@ -882,6 +909,7 @@ int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
   }
   GemvArgs g{a, lda, k / 16, wv.blocked, wv.ldw, wv.k_pad, n, reinterpret_cast<int8_t *>(c), ldc};
   const bool wide = n >= 8192 && wv.k_pad <= 4096;
+  if (m > 32) return wide ? launch_mfma_lds_deq_64<3>(g, m, dq, stream) : launch_mfma_lds_deq_64<1>(g, m, dq, stream);
   if (wide) return launch_mfma_lds_deq<8, 3, 4>(g, m, dq, stream);
   return m > 16 ? launch_mfma_lds_deq<8, 1, 4>(g, m, dq, stream) : launch_mfma_lds_deq<8, 1, 8>(g, m, dq, stream);
 }
@@ -892,6 +920,10 @@ int launch_gemv_group_dequant(const int8_t *a, int64_t lda, int m, int k, int co
                               const DequantParams *dq, float *const *c, hipStream_t stream) {
   if (count < 1 || count > kGemvGroupMax) {
     set_error("gemv group: %d members (1..%d)", count, kGemvGroupMax);
+    return MI_PARAM_INVALID;
+  }
+  if (m > kGemvGroupMaxRows) {
+    set_error("gemv group: %d rows (1..%d)", m, kGemvGroupMaxRows);
     return MI_PARAM_INVALID;
   }
   GemvGroupDeq grp{};

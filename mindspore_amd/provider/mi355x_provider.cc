@@ -404,14 +404,14 @@ class MatmulKernel : public kernel::Kernel {
     std::vector<int32_t> zps;
     FilterQuant(w, &scales, &zps);
     const void *bias = inputs_.size() > kBiasIndex ? inputs_[kBiasIndex].Data().get() : nullptr;
-    // The second packed form of the weights serves up to 32 activation rows; a node whose inferred output already has
+    // The second packed form of the weights serves up to 64 activation rows; a node whose inferred output already has
     // more rows than that does without it (half the device memory per weight).  Should the model later be resized
     // to a few rows, they run on the GEMM tiles.
     const auto oshape = outputs_[0].Shape();
     bool rows_known = !oshape.empty();
     for (int64_t e : oshape) rows_known = rows_known && e >= 0;
     const int64_t rows_now = batched_ && oshape.size() >= 2 ? oshape[oshape.size() - 2] : RowsOfOutput(outputs_[0]);
-    const bool no_decode_pack = rows_known && rows_now > kSiblingMaxRows;
+    const bool no_decode_pack = rows_known && rows_now > kDecodeMaxRows;
     if (outputs_[0].DataType() == DataType::kNumberTypeInt8) {
       const auto iq = inputs_[0].QuantParams().front();
       const auto oq = outputs_[0].QuantParams().front();
@@ -506,6 +506,7 @@ class MatmulKernel : public kernel::Kernel {
 
  private:
   static constexpr int32_t kSiblingMaxRows = 32;  // the row counts that mi_matmul_run_group runs as one launch
+  static constexpr int32_t kDecodeMaxRows = 64;   // the row counts that the blocked second copy of the weights serves
   static constexpr int kNotGrouped = -1000;
 
   // Runs this kernel and every sibling that is ready for the same rows as one launch.  kNotGrouped: nothing was
