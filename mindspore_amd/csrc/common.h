@@ -93,6 +93,13 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
 // Skinny-M path (m <= kGemvMaxRows): streams the weights once with 16-byte coalesced loads.
 constexpr int kGemvMaxRows = 64;
 constexpr int kGemvGroupMaxRows = 32;  // the group launches (several matrices, one launch) stop here
+// Matrices with fewer than 8192 channels keep the matrix-core decode kernel up to 128 rows: the GEMM's weight-stream
+// tiles (64 channels each) would occupy a quarter of the CUs there.
+constexpr int kGemvNarrowMaxRows = 128;
+constexpr int kGemvNarrowChannels = 8192;
+inline bool gemv_takes_rows(int rows, int n) {
+  return rows <= kGemvMaxRows || (rows <= kGemvNarrowMaxRows && n < kGemvNarrowChannels);
+}
 constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel can run (it does for one row, and for two when the handle has no blocked copy), above it the MFMA kernel
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,
                         const RequantParams &rq, int8_t *c, int64_t ldc, hipStream_t stream);

@@ -702,6 +702,23 @@ static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 
 // area of 64 rows and the accumulators leave room for no more).  Measured against the 64 x 64 GEMM tiles these row
 // counts ran on before (us per launch at 64 rows): 12288 x 4096 17.9 -> 14.9, 4096 x 4096 15.8 -> 8.9,
 // 4096 x 11008 34.9 -> 18.7.
+// 65..128 rows against fewer than 8192 channels: eight fragments per weight fragment, one channel group per workgroup
+// (the staging area of 128 rows takes the LDS of a CU).  Every workgroup re-reads M / 16 = 8 activation bytes per
+// weight byte from the L2s, which is what bounds it; the GEMM's weight-stream tiles of 64 channels, the alternative,
+// occupy at most N / 64 CUs (us per launch at 128 rows: 4096 x 4096 22.6 -> 13.7, 4096 x 11008 52.7 -> 29.6; a matrix
+// of 12288 channels is faster on the tiles, 24 against 37).
+static int launch_mfma_lds_128(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
+  hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, 1, 2, 128>), dim3((g.n + 15) / 16), dim3(512), 0, stream, g, m, rq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
+static int launch_mfma_lds_deq_128(const GemvArgs &g, int m, const DequantParams &dq, hipStream_t stream) {
+  hipLaunchKernelGGL((gemv_mfma_lds_deq_kernel<8, 1, 2, 128>), dim3((g.n + 15) / 16), dim3(512), 0, stream, g, m, dq);
+  MI_HIP_CHECK(hipGetLastError());
+  return MI_OK;
+}
+
 template <int RG>
 static int launch_mfma_lds_64(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
   const int blocks = (g.n + RG * 16 - 1) / (RG * 16);
@@ -817,7 +834,7 @@ static int check_gemv_operands(const int8_t *a, int64_t lda, int m, int k, const
     set_error("gemv: null pointer");
     return MI_NULL_PTR;
   }
-  if (m < 1 || m > kGemvMaxRows || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
+  if (m < 1 || !gemv_takes_rows(m, n) || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
       wv.k_pad % kKPad != 0 || wv.k_pad < k || wv.ldw < wv.k_pad || (wv.ldw & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
       (int64_t)(m - 1) * lda + k >= (int64_t)1 << 30 || wv.k_pad > 1 << 20 ||  // (32-bit buffer offsets)
@@ -876,6 +893,7 @@ int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const Weight
     g.w = wv.blocked;
     // three 16-channel groups per workgroup (a third of the activation traffic) once there are enough channels to
     // fill the device with 8-wave workgroups and the rows are short enough for a wave's share to be in flight at once
+    if (m > 64) return launch_mfma_lds_128(g, m, rq, stream);
     if (m > 32) {
       return n >= 8192 && k_pad <= 4096 ? launch_mfma_lds_64<3>(g, m, rq, stream) : launch_mfma_lds_64<1>(g, m, rq, stream);
     }
@@ -909,6 +927,7 @@ int launch_gemv_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
   }
   GemvArgs g{a, lda, k / 16, wv.blocked, wv.ldw, wv.k_pad, n, reinterpret_cast<int8_t *>(c), ldc};
   const bool wide = n >= 8192 && wv.k_pad <= 4096;
+  if (m > 64) return launch_mfma_lds_deq_128(g, m, dq, stream);
   if (m > 32) return wide ? launch_mfma_lds_deq_64<3>(g, m, dq, stream) : launch_mfma_lds_deq_64<1>(g, m, dq, stream);
   if (wide) return launch_mfma_lds_deq<8, 3, 4>(g, m, dq, stream);
   return m > 16 ? launch_mfma_lds_deq<8, 1, 4>(g, m, dq, stream) : launch_mfma_lds_deq<8, 1, 8>(g, m, dq, stream);

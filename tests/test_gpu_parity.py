@@ -73,14 +73,15 @@ def test_matmul_shapes(orc, m, n, k):
 def test_decode_rows_every_stream_shape(orc, n, k):
     """1..64 activation rows (v_dot4 kernel for one row, and for two on a handle without the blocked copy; matrix-core
     kernel otherwise: one group of 16 rows up to 16, two
-    groups up to 32, four up to 64) and the first row counts of the GEMM path, against every weight-stream shape the
+    groups up to 32, four up to 64, eight up to 128 against fewer than 8192 channels) and the first row counts of
+    the GEMM path, against every weight-stream shape the
     skinny path distinguishes: rows of one to six 1 KiB segments (whole rows per wave), seven to twelve (two waves
     per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels
     (from 8192 channels on a workgroup of the matrix-core kernel owns three groups of 16 channels: 11008 channels end
     in a workgroup with one live group, 8250 in one whose live group is ragged)."""
     rng = np.random.default_rng(n * 131 + k)
     orc.set_threads(16)
-    for m in list(range(1, 19)) + [23, 31, 32, 33, 40, 48, 63, 64, 65]:
+    for m in list(range(1, 19)) + [23, 31, 32, 33, 40, 48, 63, 64, 65, 96, 127, 128, 129]:
         case = _mm_case(rng, m, n, k, bool(m & 1), bool(m & 2), m != 4, [0, 1, 3][m % 3])
         got, _ = _gpu_matmul(case, device_tensors=bool(m & 4))
         want = orc.matmul_int8(**case)
@@ -467,7 +468,7 @@ def test_dynamic_matmul_decode_rows(orc, n, k):
     rng = np.random.default_rng(n * 7 + k)
     orc.set_threads(16)
     w = rng.integers(-128, 128, (n, k), dtype=np.int8)
-    for it, m in enumerate([1, 2, 3, 5, 8, 16, 17, 31, 32, 33, 48, 64, 65]):
+    for it, m in enumerate([1, 2, 3, 5, 8, 16, 17, 31, 32, 33, 48, 64, 65, 100, 128, 129]):
         a = rng.integers(-128, 128, (m, k), dtype=np.int8)
         nf = n if it & 1 else 1
         sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
