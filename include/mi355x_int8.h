@@ -110,8 +110,8 @@ typedef struct mi_matmul_desc {
 
 /* All weight packing happens in mi_matmul_create (the role of TransferB, LK/int8/matmul_base_int8.cc:360-384: pack
  * once at Prepare).  Two packed forms are kept: K-contiguous rows (GEMM tiles; one activation row) and 1 KiB
- * blocks of 16 channels x 64 K-bytes in matrix-core operand order (2..64 activation rows, 2..128 against fewer
- * than 8192 channels: the batched decode kernel).  MI_MATMUL_NO_DECODE_PACK skips the second form (deep x col bytes of device memory less) for callers
+ * blocks of 16 channels x 64 K-bytes in matrix-core operand order (2..64 activation rows, 2..128 against at most
+ * 4096 channels with deep >= 1024: the batched decode kernel).  MI_MATMUL_NO_DECODE_PACK skips the second form (deep x col bytes of device memory less) for callers
  * that know they never run with 2..64 rows; such a handle still accepts those row counts and runs two rows on the
  * one-row kernel's two-row form and the others on the GEMM tiles.  mi_matmul_run never packs, allocates for packing or waits. */
 #define MI_MATMUL_NO_DECODE_PACK 1

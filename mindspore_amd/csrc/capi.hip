@@ -419,10 +419,10 @@ static int run_requant_gemm(RequantState &st, const int8_t *a, int64_t lda, int 
                             const Workspace &c_ws, hipStream_t stream) {
   const RequantParams rq = st.params();
   WeightView w{static_cast<const int8_t *>(st.w.p), st.k_pad, st.ldw, nullptr};
-  // one row: the dot kernel on the row-major weights; 2..64 rows (..128 against fewer than 8192 channels): the matrix-core decode kernel on the blocked copy
+  // one row: the dot kernel on the row-major weights; 2..64 rows (..128 against at most 4096 channels and K >= 1024): the matrix-core decode kernel on the blocked copy
   // made at create time -- a handle without it runs two rows on the dot kernel and 3..64 on the GEMM tiles
   const bool skinny = rows <= kGemvDotRows ? (int64_t)rows * k16 <= 150 * 1024
-                                           : gemv_takes_rows(rows, st.n) && st.w_blocked.p != nullptr && st.k_pad <= 1 << 20;
+                                           : gemv_takes_rows(rows, st.n, st.k_pad) && st.w_blocked.p != nullptr && st.k_pad <= 1 << 20;
   if (skinny) {
     if (rows >= 2) w.blocked = static_cast<const int8_t *>(st.w_blocked.p);  // (may be absent: two rows then take the v_dot4 kernel)
     return launch_gemv_requant(a, lda, rows, k16, w, st.n, rq, c, st.n, stream);
@@ -1347,7 +1347,7 @@ static int dynmm_run_impl(mi_dynmm *h, const int8_t *a_dev, int32_t rows, float 
                      static_cast<const int8_t *>(h->w_blocked.p)};
   // decode-sized runs: the matrix-core decode kernel streams the blocked weights once (any N, any output alignment)
   // (one row runs on the row-major weights and needs no blocked copy, as long as the row fits the kernel's LDS form)
-  if (gemv_takes_rows(rows, h->n) && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024) &&
+  if (gemv_takes_rows(rows, h->n, h->k_pad) && (rows > kGemvDotRows || (int64_t)rows * k16 <= 150 * 1024) &&
       (rows == 1 || (w.blocked != nullptr && h->k_pad <= 1 << 20)))
     return launch_gemv_dequant(a, lda, rows, k16, w, h->n, dq, c_dev, h->n, s);
   if ((h->n & 3) == 0 && (reinterpret_cast<uintptr_t>(c_dev) & 15) == 0)

@@ -93,12 +93,16 @@ int launch_gemm_dequant(const int8_t *a, int64_t lda, int m, int k, const Weight
 // Skinny-M path (m <= kGemvMaxRows): streams the weights once with 16-byte coalesced loads.
 constexpr int kGemvMaxRows = 64;
 constexpr int kGemvGroupMaxRows = 32;  // the group launches (several matrices, one launch) stop here
-// Matrices with fewer than 8192 channels keep the matrix-core decode kernel up to 128 rows: the GEMM's weight-stream
-// tiles (64 channels each) would occupy a quarter of the CUs there.
+// 65..128 rows keep the matrix-core decode kernel only where it has at most one workgroup per CU (16 channels each,
+// so at most 4096 channels) and a reduction long enough to pay for its set-up.  Measured against the GEMM's
+// weight-stream tiles at 128 rows, weights not cache-resident (us per launch): 4096 x 4096 14.5 against 22.6,
+// 4096 x 11008 31.5 against 52.7, 1024 x 4096 12.7 against 22.5, 4096 x 1024 6.8 against 8.8, 2048 x 768 7.1 against
+// 6.7; 6144 x 4096 25.0 against 22.9, 8192 x 4096 26.6 against 23.1.
 constexpr int kGemvNarrowMaxRows = 128;
-constexpr int kGemvNarrowChannels = 8192;
-inline bool gemv_takes_rows(int rows, int n) {
-  return rows <= kGemvMaxRows || (rows <= kGemvNarrowMaxRows && n < kGemvNarrowChannels);
+constexpr int kGemvNarrowChannels = 4096;  // at most this many
+constexpr int kGemvNarrowMinK = 1024;      // padded reduction length from which those rows come here
+inline bool gemv_takes_rows(int rows, int n, int k_pad) {
+  return rows <= kGemvMaxRows || (rows <= kGemvNarrowMaxRows && n <= kGemvNarrowChannels && k_pad >= kGemvNarrowMinK);
 }
 constexpr int kGemvDotRows = 2;  // up to here the v_dot4 kernel can run (it does for one row, and for two when the handle has no blocked copy), above it the MFMA kernel
 int launch_gemv_requant(const int8_t *a, int64_t lda, int m, int k, const WeightView &w, int n,

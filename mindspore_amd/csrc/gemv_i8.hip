@@ -702,11 +702,14 @@ static int with_row_class(int m, F &&f) {  // rows rounded up to 2, 4, 8, 16 or 
 // area of 64 rows and the accumulators leave room for no more).  Measured against the 64 x 64 GEMM tiles these row
 // counts ran on before (us per launch at 64 rows): 12288 x 4096 17.9 -> 14.9, 4096 x 4096 15.8 -> 8.9,
 // 4096 x 11008 34.9 -> 18.7.
-// 65..128 rows against fewer than 8192 channels: eight fragments per weight fragment, one channel group per workgroup
-// (the staging area of 128 rows takes the LDS of a CU).  Every workgroup re-reads M / 16 = 8 activation bytes per
-// weight byte from the L2s, which is what bounds it; the GEMM's weight-stream tiles of 64 channels, the alternative,
-// occupy at most N / 64 CUs (us per launch at 128 rows: 4096 x 4096 22.6 -> 13.7, 4096 x 11008 52.7 -> 29.6; a matrix
-// of 12288 channels is faster on the tiles, 24 against 37).
+// 65..128 rows against at most 4096 channels with K >= 1024: eight fragments per weight fragment, one channel group
+// per workgroup (the staging area of 128 rows takes the LDS of a CU, so more than 4096 channels would need a second
+// round of workgroups, and shorter reductions do not pay for the set-up).  Every workgroup re-reads M / 16 = 8
+// activation bytes per weight byte from the L2s, which is what bounds it; the GEMM's weight-stream tiles of 64
+// channels, the alternative, occupy at most N / 64 CUs (us per launch at 128 rows, weights not cache-resident:
+// 4096 x 4096 22.6 -> 14.5, 4096 x 11008 52.7 -> 31.5; with the weights in the caches the two are level at
+// 4096 x 4096, 13.3 against 13.5).  Two channel groups per workgroup with one step per pass (what the LDS then has
+// room for) were 10-15 % ahead of the tiles between 4096 and 8192 channels and behind them above, and were not kept.
 static int launch_mfma_lds_128(const GemvArgs &g, int m, const RequantParams &rq, hipStream_t stream) {
   hipLaunchKernelGGL((gemv_mfma_lds_kernel<8, 1, 2, 128>), dim3((g.n + 15) / 16), dim3(512), 0, stream, g, m, rq);
   MI_HIP_CHECK(hipGetLastError());
@@ -834,7 +837,7 @@ static int check_gemv_operands(const int8_t *a, int64_t lda, int m, int k, const
     set_error("gemv: null pointer");
     return MI_NULL_PTR;
   }
-  if (m < 1 || !gemv_takes_rows(m, n) || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
+  if (m < 1 || !gemv_takes_rows(m, n, wv.k_pad) || n <= 0 || k <= 0 || (k & 15) != 0 || (lda & 15) != 0 || lda < k ||
       wv.k_pad % kKPad != 0 || wv.k_pad < k || wv.ldw < wv.k_pad || (wv.ldw & 15) != 0 ||
       (reinterpret_cast<uintptr_t>(a) & 15) != 0 ||
       (int64_t)(m - 1) * lda + k >= (int64_t)1 << 30 || wv.k_pad > 1 << 20 ||  // (32-bit buffer offsets)

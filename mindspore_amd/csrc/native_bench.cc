@@ -99,6 +99,8 @@ static int make_matrix(const Shape &shape, int rows, Rng *rng, Matrix *m) {
   d.filter_quant_num = n;
   d.filter_scales = scales.data();
   d.filter_zps = zps.data();
+  // NATIVE_BENCH_NO_DECODE_PACK=1: handles without the blocked weight copy (2 rows and more then run on the GEMM tiles)
+  if (getenv("NATIVE_BENCH_NO_DECODE_PACK") != nullptr) d.flags |= MI_MATMUL_NO_DECODE_PACK;
   CHECK_MI(mi_matmul_create(&d, w.data(), bias.data(), &m->h));
   std::vector<int8_t> a((size_t)rows * k);
   for (auto &x : a) x = (int8_t)(rng->next() & 0xff);

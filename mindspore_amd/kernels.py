@@ -68,7 +68,7 @@ class _Handle:
 
 class MatmulInt8Kernel(_Handle):
     """Full-quant int8 MatMul: C = requant(A x W^T).  weight is [N, K] when transpose_b else [K, N]; bias int32 [N].
-    decode_pack=False skips the second packed form of the weights (the one runs with 2..32 rows use); such rows then
+    decode_pack=False skips the second packed form of the weights (the one runs with 2..64 rows use, 2..128 against at most 4096 channels with K >= 1024); such rows then
     run on the GEMM tiles."""
     _destroy = "mi_matmul_destroy"
 
@@ -351,7 +351,7 @@ class MatmulDynamicInt8Kernel(_Handle):
         """packed_sdot=(N, K): `weight` is the flat byte string a model converted for the ARM dot-product kernel
         carries (blocks of 16 channels x 4 K-bytes, RowMajor2Row4x16MajorInt8 / RowMajor2Col4x16MajorInt8) and
         weight_sums, if given, its int32 weight-sums tensor [round_up(N, 16)].  decode_pack=False skips the blocked
-        second copy of the weights that serves 1..32 rows (MI_DYNMM_NO_DECODE_PACK)."""
+        second copy of the weights that serves 2..64 rows, and 65..128 against at most 4096 channels with K >= 1024 (MI_DYNMM_NO_DECODE_PACK)."""
         super().__init__()
         L = _lib.init(device)
         weight = _host_i8(weight)

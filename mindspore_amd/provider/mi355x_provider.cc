@@ -411,7 +411,7 @@ class MatmulKernel : public kernel::Kernel {
     bool rows_known = !oshape.empty();
     for (int64_t e : oshape) rows_known = rows_known && e >= 0;
     const int64_t rows_now = batched_ && oshape.size() >= 2 ? oshape[oshape.size() - 2] : RowsOfOutput(outputs_[0]);
-    const bool no_decode_pack = rows_known && rows_now > (n < 8192 ? 2 * kDecodeMaxRows : kDecodeMaxRows);
+    const bool no_decode_pack = rows_known && rows_now > (n <= 4096 && k >= 1024 ? 2 * kDecodeMaxRows : kDecodeMaxRows);
     if (outputs_[0].DataType() == DataType::kNumberTypeInt8) {
       const auto iq = inputs_[0].QuantParams().front();
       const auto oq = outputs_[0].QuantParams().front();
@@ -507,7 +507,7 @@ class MatmulKernel : public kernel::Kernel {
  private:
   static constexpr int32_t kSiblingMaxRows = 32;  // the row counts that mi_matmul_run_group runs as one launch
   static constexpr int32_t kDecodeMaxRows = 64;   // the row counts that the blocked second copy of the weights serves
-                                                  // (twice as many against fewer than 8192 channels)
+                                                  // (twice as many against at most 4096 channels with K >= 1024)
   static constexpr int kNotGrouped = -1000;
 
   // Runs this kernel and every sibling that is ready for the same rows as one launch.  kNotGrouped: nothing was

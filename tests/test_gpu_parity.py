@@ -73,7 +73,7 @@ def test_matmul_shapes(orc, m, n, k):
 def test_decode_rows_every_stream_shape(orc, n, k):
     """1..64 activation rows (v_dot4 kernel for one row, and for two on a handle without the blocked copy; matrix-core
     kernel otherwise: one group of 16 rows up to 16, two
-    groups up to 32, four up to 64, eight up to 128 against fewer than 8192 channels) and the first row counts of
+    groups up to 32, four up to 64, eight up to 128 against at most 4096 channels with K >= 1024) and the first row counts of
     the GEMM path, against every weight-stream shape the
     skinny path distinguishes: rows of one to six 1 KiB segments (whole rows per wave), seven to twelve (two waves
     per row, even and odd segment counts), a stream longer than the in-flight queue, few and many output channels
@@ -461,8 +461,8 @@ def test_dynamic_matmul(orc):
                                  (8250, 80), (515, 3000)])
 def test_dynamic_matmul_decode_rows(orc, n, k):
     """1..64 rows of the dynamic-quant MatMul take the decode kernels with the fp32 epilogue (one and three
-    channel groups per workgroup, ragged channels and K, one, two and four groups of activation rows); 65 rows and a
-    handle without the blocked weight copy take the GEMM tiles.  Per-tensor and per-channel weight scales, a weight zero
+    channel groups per workgroup, ragged channels and K, one, two, four and eight groups of activation rows); 129
+    rows, 65..128 against many channels or a short K, and a handle without the blocked weight copy take the GEMM tiles.  Per-tensor and per-channel weight scales, a weight zero
     point, bias, every activation; input parameters by value, from device memory, and one scale per row."""
     import torch
     rng = np.random.default_rng(n * 7 + k)
