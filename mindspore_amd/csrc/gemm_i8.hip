@@ -1149,6 +1149,13 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   if (EPI == EPI_DEQUANT && tiles_m >= 128 && tiles_m < 256 && g.k <= 1024)
     return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 4, 3>(g, rq, dq, stream);
   if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 4, 2>(g, rq, dq, stream);
+  // What is left has few tiles, so a workgroup walks its whole K alone: with a long K and weights that are not
+  // cache-resident, three 64-byte steps in flight leave it waiting on memory.  Eight stages, two workgroups per CU
+  // (us per launch, weights streamed from HBM): 256 x 4096 x 4096 23.2 -> 15.3, 256 x 4096 x 11008 55.0 -> 34.8,
+  // 384 x 4096 x 4096 42.8 -> 26.1 (384 tiles: one round instead of two); with the weights in the L2s
+  // 300 x 4096 x 2048 16.4 -> 11.0, 640 x 2048 x 1024 8.5 -> 6.9, and 5 % slower where fewer than a hundred tiles
+  // find them there (512 x 768 x 3072: 8.5 -> 9.0).  Sixteen stages are no better than eight.
+  if (g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 8, 2>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }
 

@@ -51,6 +51,8 @@ MM_SHAPES = [(1, 1, 1), (1, 64, 16), (2, 5, 7), (3, 100, 15), (4, 256, 128), (5,
              # few rows against long weight rows: the deep-prefetch tile configuration (16 LDS stages)
              (17, 100, 1024), (33, 260, 2048), (64, 512, 4096), (40, 64, 1280), (20, 36, 5120),
              (65, 100, 1024), (128, 260, 2048), (100, 64, 1280),
+             # more than 128 rows, few tiles and a long K: the 64 x 64 tiles on eight stages, two workgroups per CU
+             (129, 260, 2048), (300, 500, 1040), (200, 4100, 1024), (384, 333, 4112),
              # a few hundred rows against many channels: the 256-channel x 128-row tile; two workgroups per CU on the
              # 128 x 128 tile (4224 x 2100 gives 33 x 17 of them)
              (300, 11008, 80), (512, 8196, 272), (129, 32772, 48), (4224, 2100, 144)]
@@ -439,7 +441,9 @@ def test_dynamic_matmul(orc):
                                     (700, 300, 129), (64, 2304, 768), (4100, 4096, 400), (4097, 4100, 208),
                                     # fp32 output on the 128-tile K-block loop: at most one tile per CU, K >= 2048,
                                     # 768 tiles and more; and 306 tiles, which stay on the 64-byte-step loop
-                                    (1500, 1420, 144), (1300, 1290, 2064), (4100, 3000, 144), (2100, 2304, 208)]):
+                                    (1500, 1420, 144), (1300, 1290, 2064), (4100, 3000, 144), (2100, 2304, 208),
+                                    # few tiles and a long K: 64 x 64 tiles on eight stages
+                                    (260, 516, 1100), (129, 100, 2048)]):
         a = rng.integers(-128, 128, (m, k), dtype=np.int8)
         w = rng.integers(-128, 128, (n, k), dtype=np.int8)
         nf = n if it & 1 else 1
