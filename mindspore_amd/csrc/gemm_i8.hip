@@ -1116,6 +1116,24 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   // a few activation rows against a big weight matrix: one row of 64 x 64 tiles, deep prefetch (HBM-bound)
   if (g.m <= 64 && g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 16>(g, rq, dq, stream);
   if (g.m <= 128 && g.k_pad >= 1024) return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
+  // Few tiles and a long K: every workgroup walks its whole K alone at the pace of its own loop (a 64 x 64 tile takes
+  // about 0.2 us per 64 bytes of K, a 64 x 128 tile 0.3, a 128 x 128 tile 0.6 per 128 bytes, whatever the number of
+  // workgroups up to one per CU), so the smallest tile that still fits the device in one round wins, on eight stages
+  // (three steps in flight leave a lone workgroup waiting on memory).  Measured with the weights streamed from HBM
+  // (us per launch): 256 x 4096 x 4096 23.2 -> 15.6, 256 x 4096 x 11008 55.0 -> 35.7, 384 x 4096 x 4096 42.8 -> 19.5,
+  // 512 x 4096 x 4096 22.2 -> 19.3, 512 x 3072 x 4096 41.2 -> 19.1, 2048 x 768 x 3072 31.8 -> 14.0,
+  // 256 x 8192 x 2048 13.6 -> 12.5; with the weights in the L2s 300 x 4096 x 2048 16.4 -> 11.0,
+  // 640 x 2048 x 1024 8.5 -> 6.9, and 5 % slower where fewer than a hundred tiles find them there
+  // (512 x 768 x 3072: 8.5 -> 9.0).  Sixteen stages are no better than eight.
+  if (g.k_pad >= 1024) {
+    const int64_t cols64 = (g.n + 63) / 64;
+    if ((int64_t)((g.m + 63) / 64) * cols64 <= 256) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 8, 2>(g, rq, dq, stream);
+    // (against the 128 x 128 K-block tiles at K = 1024 the 64 x 128 tile is 15 % ahead on streamed weights and 4-9 %
+    //  behind on cache-resident ones -- 512 x 4096 x 1024: 7.1 -> 7.7 us -- so it starts at K = 2048, where it is
+    //  10-13 % ahead on those too: 512 x 4096 x 4096 20.4 -> 17.8 us, 2048 x 768 x 3072 13.9 -> 12.3 us)
+    if (g.k_pad >= 2048 && (int64_t)((g.m + 127) / 128) * cols64 <= 256)
+      return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 8>(g, rq, dq, stream);
+  }
   // The 256 x 256 tile does a unit of work in little more than half the time the 128 x 128 tiles need, so with int8
   // output it is taken as soon as the 128 x 128 tiles would no longer fit the device in one go (more than 512 of
   // them, i.e. more than 128 large tiles): 2304 x 4096 x 4096 51.6 -> 41.2 us, 2816 x 4096 x 1024 20.4 -> 17.8 us;
@@ -1149,12 +1167,7 @@ static int launch_pick_tile(const GemmArgs &g, const RequantParams &rq, const De
   if (EPI == EPI_DEQUANT && tiles_m >= 128 && tiles_m < 256 && g.k <= 1024)
     return launch_cfg<64, 128, EPI, HAS_ZW, FAST, 4, 3>(g, rq, dq, stream);
   if (tiles_m >= 128) return launch_cfg<128, 128, EPI, HAS_ZW, FAST, 4, 2>(g, rq, dq, stream);
-  // What is left has few tiles, so a workgroup walks its whole K alone: with a long K and weights that are not
-  // cache-resident, three 64-byte steps in flight leave it waiting on memory.  Eight stages, two workgroups per CU
-  // (us per launch, weights streamed from HBM): 256 x 4096 x 4096 23.2 -> 15.3, 256 x 4096 x 11008 55.0 -> 34.8,
-  // 384 x 4096 x 4096 42.8 -> 26.1 (384 tiles: one round instead of two); with the weights in the L2s
-  // 300 x 4096 x 2048 16.4 -> 11.0, 640 x 2048 x 1024 8.5 -> 6.9, and 5 % slower where fewer than a hundred tiles
-  // find them there (512 x 768 x 3072: 8.5 -> 9.0).  Sixteen stages are no better than eight.
+  // (what is left has few tiles of any size; with a long K the 64 x 64 tiles take eight stages as above)
   if (g.k_pad >= 1024) return launch_cfg<64, 64, EPI, HAS_ZW, FAST, 8, 2>(g, rq, dq, stream);
   return launch_cfg<64, 64, EPI, HAS_ZW, FAST>(g, rq, dq, stream);
 }

@@ -53,6 +53,8 @@ MM_SHAPES = [(1, 1, 1), (1, 64, 16), (2, 5, 7), (3, 100, 15), (4, 256, 128), (5,
              (65, 100, 1024), (128, 260, 2048), (100, 64, 1280),
              # more than 128 rows, few tiles and a long K: the 64 x 64 tiles on eight stages, two workgroups per CU
              (129, 260, 2048), (300, 500, 1040), (200, 4100, 1024), (384, 333, 4112),
+             # too many 64 x 64 tiles for one round but not too many 64-channel x 128-row ones, K >= 2048
+             (384, 4100, 2048), (1100, 1000, 2100),
              # a few hundred rows against many channels: the 256-channel x 128-row tile; two workgroups per CU on the
              # 128 x 128 tile (4224 x 2100 gives 33 x 17 of them)
              (300, 11008, 80), (512, 8196, 272), (129, 32772, 48), (4224, 2100, 144)]
@@ -443,7 +445,7 @@ def test_dynamic_matmul(orc):
                                     # 768 tiles and more; and 306 tiles, which stay on the 64-byte-step loop
                                     (1500, 1420, 144), (1300, 1290, 2064), (4100, 3000, 144), (2100, 2304, 208),
                                     # few tiles and a long K: 64 x 64 tiles on eight stages
-                                    (260, 516, 1100), (129, 100, 2048)]):
+                                    (260, 516, 1100), (129, 100, 2048), (520, 2100, 2064)]):
         a = rng.integers(-128, 128, (m, k), dtype=np.int8)
         w = rng.integers(-128, 128, (n, k), dtype=np.int8)
         nf = n if it & 1 else 1
