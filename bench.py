@@ -647,14 +647,19 @@ def main():
                                                          frac_of_hbm_peak=solo["gbps"] / PEAK_HBM_GBPS,
                                                          launches_per_step=solo["launches_per_step"])
             extra["gemv_decode_m%d" % m] = best
-        # the same decoder layer as dynamic-quant MatMuls (run-time input scale, fp32 out), one launch per matrix;
-        # beside it the same rows on handles without the blocked weight copy (2 rows and more then run on the GEMM
-        # tiles; one row needs no copy)
+        # the same decoder layer as dynamic-quant MatMuls (run-time input scale, fp32 out), gate and up as one launch
+        # (mi_dynmm_run_group); beside it one launch per matrix, and the same rows on handles without the blocked
+        # weight copy (2 rows and more then run on the GEMM tiles; one row needs no copy)
         for m in (1, 8):
             dyn = native_bench("dyndecode", m, 3, 500, 50, 0)
             if dyn and "gbps" in dyn:
                 entry = dict(dyn, host="native C++ over the C ABI", bound="hbm", frac=dyn["gbps"] / PEAK_HBM_GBPS,
                              frac_of_hbm_peak=dyn["gbps"] / PEAK_HBM_GBPS)
+                solo = native_bench("dyndecode", m, 3, 500, 50, 0, env={"NATIVE_BENCH_NO_GROUP": "1"})
+                if solo and "gbps" in solo:
+                    entry["one_launch_per_matrix"] = dict(ms_per_step=solo["ms_per_step"], gbps=solo["gbps"],
+                                                          frac_of_hbm_peak=solo["gbps"] / PEAK_HBM_GBPS,
+                                                          launches_per_step=solo["launches_per_step"])
                 tiles = native_bench("dyndecode", m, 3, 200, 20, 1)
                 if tiles and "gbps" in tiles:
                     entry["without_the_blocked_copy"] = dict(ms_per_step=tiles["ms_per_step"], gbps=tiles["gbps"])
