@@ -316,7 +316,7 @@ struct RequantState {
       for (int c = 0; c < n; ++c) memcpy(packed.data() + (size_t)c * ldw, w_nk + (size_t)c * k, (size_t)k);
       if ((rc = upload(&w, packed)) != MI_OK) return rc;
       if (pack_decode) {
-        // The blocked copy is an optimisation for 2..32 activation rows, not a requirement: without it those row
+        // The blocked copy is an optimisation for 2..64 activation rows (some shapes: ..128), not a requirement: without it those row
         // counts run on the v_dot4 kernel (two rows) or the GEMM tiles.  A device that has no room for it still gets
         // a working handle.
         rc = w_blocked.ensure((size_t)n_pad * k_pad);

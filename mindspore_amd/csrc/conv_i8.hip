@@ -145,6 +145,26 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const int8_t *__restri
   const int ih0 = oh * g.stride_h - g.pad_u, iw0 = ow * g.stride_w - g.pad_l;
   const int8_t *img = in + (int64_t)b * g.in_h * g.in_w * g.in_c;
 
+  // The requantisation parameters of the lane's channels, a block of 32 output channels at a time: prm[q][..] are
+  // channels 32 * ob + 8 * q + 4 * h .. + 3.  Fetched without a branch on the channel or on the kind of parameters
+  // (the arrays are padded to a multiple of 256 channels and all exist) and all sixteen-plus-four at once: the first
+  // block's before the gather, so that they arrive behind it.  Fetched where they are used, one group of four
+  // channels after the other and behind the branches of the previous group's arithmetic, they were four round trips
+  // in a row at the end of a 32-channel stem.
+  v4i prm[4][5];
+  auto fetch_params = [&](int ob) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int nb = ob * 32 + q * 8 + h * 4;
+      prm[q][0] = *reinterpret_cast<const v4i *>(rq.mult + nb);
+      prm[q][1] = *reinterpret_cast<const v4i *>(rq.bias2 + nb);
+      prm[q][2] = *reinterpret_cast<const v4i *>(rq.rshift + nb);
+      prm[q][3] = *reinterpret_cast<const v4i *>(rq.zw + nb);
+      prm[q][4] = *reinterpret_cast<const v4i *>(rq.lshift + nb);
+    }
+  };
+  fetch_params(0);
+
   union Frag {
     v4i v;
     int8_t b[16];
@@ -204,16 +224,11 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const int8_t *__restri
   // acc[ob][4 * q + e] is output channel 32 * ob + 8 * q + 4 * h + e of pixel r
 #pragma unroll
   for (int ob = 0; ob < OCB; ++ob) {
+    if (ob > 0) fetch_params(ob);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int nb = ob * 32 + q * 8 + h * 4;
-      if (nb >= g.out_c) continue;
-      const v4i mult4 = *reinterpret_cast<const v4i *>(rq.mult + nb);
-      const v4i bias4 = *reinterpret_cast<const v4i *>(rq.bias2 + nb);
-      const v4i e4 = *reinterpret_cast<const v4i *>(rq.rshift + nb);
-      v4i zw4 = {0, 0, 0, 0}, ls4 = {0, 0, 0, 0};
-      if (rq.has_zw) zw4 = *reinterpret_cast<const v4i *>(rq.zw + nb);
-      if (!rq.fast) ls4 = *reinterpret_cast<const v4i *>(rq.lshift + nb);
+      const v4i mult4 = prm[q][0], bias4 = prm[q][1], e4 = prm[q][2], zw4 = prm[q][3], ls4 = prm[q][4];
       union {
         uint32_t u;
         int8_t b[4];
@@ -234,7 +249,7 @@ __global__ __launch_bounds__(256) void conv_smallk_kernel(const int8_t *__restri
         t = t > rq.amin ? t : rq.amin;
         o.b[e] = (int8_t)t;
       }
-      if (live) *reinterpret_cast<uint32_t *>(out + p * g.out_c + nb) = o.u;
+      if (live && nb < g.out_c) *reinterpret_cast<uint32_t *>(out + p * g.out_c + nb) = o.u;
     }
   }
 }
