@@ -801,7 +801,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 // above.  T = 2 (128 x 128, slots of 16 KiB, 80 KiB of LDS, a quarter of the registers) lets two workgroups share a
 // CU: for shapes with fewer than one 256 x 256 tile per CU, or short K, where one tile's prologue and epilogue have
 // to overlap another tile's main loop.  Per quarter a wave then has 4 MFMAs, 4 fragment reads and 2 loads.
-template <int T, int EPI, bool HAS_ZW, bool FAST>
+// DIAG: timing what-ifs of the main loop (wrong results, see diag_kblock128()): bit 0 = no operand loads after the
+// first two K blocks, bit 1 = no wait and no barrier between K blocks.
+template <int T, int EPI, bool HAS_ZW, bool FAST, int DIAG = 0>
 __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const RequantParams &rq, const DequantParams &dq) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the buffer-resource type exists in the device pass only; the host pass needs just the stub
   constexpr int TILE = 64 * T, KB = 128;  // wave tile 32 T x 32 T = T x T MFMA tiles
@@ -859,6 +861,7 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
   auto lds_ptr = [](char *p) { return (__attribute__((address_space(3))) void *)p; };
   // half: 0 = the first half of the wave's loader instructions (the upper half of its rows), 1 = the other half
   auto dma_w = [&](int slot, int kb, int half) {
+    if ((DIAG & 1) && kb > 1) return;
     char *dst = lds + slot * SLOT + wave * WROWS * KB;
 #pragma unroll
     for (int ii = 0; ii < LPW / 2; ++ii) {
@@ -868,6 +871,7 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
     }
   };
   auto dma_a = [&](int slot, int kb, int half) {
+    if ((DIAG & 1) && kb > 1) return;
     char *dst = lds + (3 + slot) * SLOT + wave * WROWS * KB;
 #pragma unroll
     for (int ii = 0; ii < LPW / 2; ++ii) {
@@ -1012,7 +1016,9 @@ __device__ __forceinline__ void gemm_kblock_body(const GemmArgs &g, const Requan
     if (NEXT2) dma_w(ws2, b + 2, 1);
     mma(f0, b * 8 + 4 + h);
     hints();
-    if (NEXT2) {
+    if (DIAG & 2) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    } else if (NEXT2) {
       // everything but the loads of W block b+2 has landed: that includes all of block b+1
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(LPW) : "memory");
     } else if (NEXT1) {
@@ -1063,6 +1069,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   gemm_kblock_body<2, EPI, HAS_ZW, FAST>(g, rq, dq);
 }
 
+template <int EPI, int DIAG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_kblock128_diag_kernel(
+    GemmArgs g, RequantParams rq, DequantParams dq) {
+  gemm_kblock_body<2, EPI, false, true, DIAG>(g, rq, dq);
+}
+
 // ---- host side -----------------------------------------------------------------------------------------------
 // Measurement aid, off unless the environment says MI355X_DIAG_SAME_PANEL=1 when the library is first used: the
 // K-block kernels then fetch tile (0, 0)'s operands for every tile, so that every operand line is an L2 hit.  The
@@ -1073,6 +1085,18 @@ static int diag_same_panel() {
     return (e != nullptr && e[0] == '1') ? 1 : 0;
   }();
   return on;
+}
+
+// A second one, MI355X_DIAG_KBLOCK128=<1|2|3>: builds of the 128 x 128 K-block kernel (no weight zero point, the
+// one-multiply epilogue) without the operand loads after the first two K blocks (1), without the wait and the barrier
+// between K blocks (2), or without both (3).  The results are wrong; the launch times say what the main loop spends
+// on the matrix cores and what on feeding them.
+static int diag_kblock128() {
+  static const int v = [] {
+    const char *e = getenv("MI355X_DIAG_KBLOCK128");
+    return (e != nullptr && e[0] >= '1' && e[0] <= '3') ? e[0] - '0' : 0;
+  }();
+  return v;
 }
 
 template <int TILE_N, int TILE_M, int EPI, bool HAS_ZW, bool FAST, int NST = 4, int OCC = 1>
@@ -1102,6 +1126,16 @@ static int launch_kblock128(GemmArgs g, const RequantParams &rq, const DequantPa
   g.tiles_m = (g.m + 127) / 128;
   g.tiles_n = (g.n + 127) / 128;
   if ((g.m & 127) != 0 || (g.n & 127) != 0) g.diag_same_panel = 0;
+  if constexpr (!HAS_ZW && FAST) {
+    if (const int d = diag_kblock128(); d != 0) {
+      auto kern = d == 1   ? gemm_kblock128_diag_kernel<EPI, 1>
+                  : d == 2 ? gemm_kblock128_diag_kernel<EPI, 2>
+                           : gemm_kblock128_diag_kernel<EPI, 3>;
+      hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g, rq, dq);
+      MI_HIP_CHECK(hipGetLastError());
+      return MI_OK;
+    }
+  }
   hipLaunchKernelGGL((gemm_kblock128_kernel<EPI, HAS_ZW, FAST>), dim3(g.tiles_m * g.tiles_n), dim3(256), 0, stream, g,
                      rq, dq);
   MI_HIP_CHECK(hipGetLastError());
