@@ -209,7 +209,7 @@ struct RequantState {
   int n = 0, k = 0, n_pad = 0, k_pad = 0, ldw = 0;
   DevBuf w, mult, bias2, rshift, lshift, zw;
   DevBuf mult2, c2lo, c2hi, pre;  // the GEMM epilogue's per-channel constants (RequantParams::fast2)
-  DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (2..32 activation rows); built in create or absent
+  DevBuf w_blocked;  // the same weights in 1 KiB matrix-core blocks (2..64 activation rows, some shapes ..128); built in create or absent
   std::vector<int32_t> h_mult, h_ls, h_rs, h_bias2;
   int32_t amin = -128, amax = 127, zo = 0;
   bool has_zw = false, fast = false, fast2 = false;
@@ -470,7 +470,7 @@ struct mi_dynmm {
   int32_t zw0 = 0;
   bool has_bias = false;
   DevBuf w, wscale, wsum, bias, a_ws, c_ws, h_in, h_out, h_params;
-  DevBuf w_blocked;  // the weights in 1 KiB matrix-core blocks for 1..32 activation rows; built in create or absent
+  DevBuf w_blocked;  // the weights in 1 KiB matrix-core blocks for 2..64 activation rows (some shapes ..128); built in create or absent
 };
 
 // No C++ exception may cross the C ABI: host allocations in the create calls can throw.
