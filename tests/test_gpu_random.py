@@ -36,6 +36,38 @@ def test_random_matmul(orc, seed):
         assert np.array_equal(got, want), (seed, it, m, n, k, int((got != want).sum()))
 
 
+@pytest.mark.parametrize("seed", [5])
+def test_random_few_tiles_long_k(orc, seed):
+    """A few hundred rows against a reduction of 1024 bytes and more: the 64 x 64 and 64-channel x 128-row tiles on eight
+    stages that such shapes take while they fit the device in one round, and their neighbours (the K-block tiles
+    beyond); handles with and without the blocked weight copy; int8 and fp32 output."""
+    rng = np.random.default_rng(seed)
+    orc.set_threads(16)
+    for it in range(40):
+        m = int(rng.integers(129, 1200))
+        n = _pick(rng, [64, 100, 256, 500, 768, 1000, 2048, 4100]) if rng.random() < 0.5 else int(rng.integers(4, 3000))
+        k = _pick(rng, [1024, 1040, 2048, 2064, 3072, 4096, 4112]) if rng.random() < 0.6 else int(rng.integers(1009, 4600))
+        if m * n * k > 4e9:
+            m = max(129, int(4e9 / (n * k)))
+        if it % 4 != 3:
+            case = T._mm_case(rng, m, n, k, _flag(rng), _flag(rng), _flag(rng), _pick(rng, [0, 1, 3]), _flag(rng))
+            got, _ = T._gpu_matmul(case, device_tensors=_flag(rng), decode_pack=_flag(rng))
+            want = orc.matmul_int8(**case)
+            assert np.array_equal(got, want), (seed, it, m, n, k, int((got != want).sum()))
+        else:
+            a = rng.integers(-128, 128, (m, k), dtype=np.int8)
+            w = rng.integers(-128, 128, (n, k), dtype=np.int8)
+            nf = n if _flag(rng) else 1
+            sw = rng.uniform(1e-3, 1e-2, nf).astype(np.float32).astype(np.float64)
+            zw = np.full(nf, 0 if _flag(rng) else int(rng.integers(-5, 6)), np.int32)
+            bias = rng.standard_normal(n).astype(np.float32) if _flag(rng) else None
+            sx, zx, act = float(rng.uniform(0.01, 0.1)), int(rng.integers(-128, 128)), _pick(rng, [0, 1, 3])
+            kern = K.MatmulDynamicInt8Kernel(w, bias, T._qps(sw, zw), True, act)
+            want = orc.dynamic_matmul(a, w, bias, sx, zx, sw, zw, act, True)
+            got = kern.run(a, K.QuantParam(sx, zx))
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (seed, it, m, n, k)
+
+
 @pytest.mark.parametrize("seed", [11])
 def test_random_decode_rows_against_wide_matrices(orc, seed):
     """2..32 activation rows against 8192 channels and more with K up to 4096: the matrix-core decode kernel with three
