@@ -129,7 +129,7 @@ def test_random_conv(orc, seed):
     ran = 0
     for it in range(400):
         b, ih, iw = int(rng.integers(1, 3)), int(rng.integers(1, 20)), int(rng.integers(1, 20))
-        ic, oc = _pick(rng, [1, 3, 4, 7, 16, 17, 32]), _pick(rng, [1, 3, 4, 8, 17, 32, 65])
+        ic, oc = _pick(rng, [1, 3, 4, 7, 16, 17, 32]), _pick(rng, [1, 3, 4, 8, 17, 32, 65, 64, 100, 128])
         kh, kw, stride, dil, pad = _geometry(rng)
         if ih + pad[0] + pad[1] < (kh - 1) * dil[0] + 1 or iw + pad[2] + pad[3] < (kw - 1) * dil[1] + 1:
             continue
